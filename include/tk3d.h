@@ -1,0 +1,187 @@
+/*
+ * tk3d.h - C ABI of the MI355X (gfx950) point-cloud operator library.
+ *
+ * One entry point per kernel family of the reference extension torkit3d._C
+ * (torkit3d/csrc/torkit3d.cpp:13-21). Each function below names the reference
+ * interface it replaces. The reference passes at::Tensor objects and allocates
+ * its outputs; here every argument is a plain device pointer, a size or a scalar:
+ *
+ *   - all pointers are DEVICE pointers on the current HIP device, 16-byte aligned
+ *     or better is not required (natural alignment of the element type is);
+ *   - tensors are dense row-major: xyz [B,N,3], features [B,C,N], indices int64;
+ *   - outputs are caller-allocated and fully overwritten (no pre-zeroing needed);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     kernels are enqueued on it and the call returns without synchronising;
+ *   - nothing is allocated or freed, nothing throws;
+ *   - the return value is TK3D_OK (0), a negative TK3D_ERR_* argument error
+ *     (nothing was launched), or a positive hipError_t from the launch.
+ *
+ * `_f32` entry points take float data, `_f64` double data (the reference
+ * instantiates both through AT_DISPATCH_FLOATING_TYPES).
+ *
+ * Distances are squared Euclidean, evaluated for key k and query q as
+ *   fma(dz,dz, fma(dy,dy, dx*dx)),  dx = k.x - q.x, ...
+ * which is what the reference kernels compute under nvcc's default contraction.
+ */
+#ifndef TK3D_H
+#define TK3D_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TK3D_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum {
+    TK3D_OK = 0,
+    TK3D_ERR_NULL_POINTER = -1,  /* a required pointer is NULL              */
+    TK3D_ERR_BAD_SIZE = -2,      /* negative size, or a product overflows   */
+    TK3D_ERR_BAD_K = -3,         /* k / num_samples outside the legal range */
+    TK3D_ERR_BAD_VERSION = -4,   /* knn `version` not 0 or 1                */
+    TK3D_ERR_WORKSPACE = -5,     /* workspace missing or too small          */
+    TK3D_ERR_UNSUPPORTED = -6    /* shape beyond what the kernels index     */
+};
+
+/* Library version (TK3D_VERSION of the build). */
+int tk3d_version(void);
+
+/* Static, human-readable text for a return code of this library (negative codes)
+ * or of the HIP runtime (positive codes). Never NULL. */
+const char *tk3d_error_string(int code);
+
+/* ---- chamfer / nearest-neighbour distance ---------------------------------
+ * Replaces chamfer_distance_forward_cuda
+ * (torkit3d/csrc/include/chamfer_distance.h:6-8, cuda/chamfer_distance_kernel.cu:91-151).
+ * dist1[b,i] = min_j d2(xyz1[b,i], xyz2[b,j]), idx1[b,i] = the lowest such j;
+ * dist2/idx2 likewise with the clouds swapped. An empty or all-NaN opposite
+ * cloud gives (+inf, -1) in fp32. B, N1, N2 may be 0. */
+int tk3d_chamfer_distance_forward_f32(const float *xyz1, const float *xyz2,
+                                      int64_t B, int64_t N1, int64_t N2,
+                                      float *dist1, int64_t *idx1, float *dist2,
+                                      int64_t *idx2, void *stream);
+int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2,
+                                      int64_t B, int64_t N1, int64_t N2,
+                                      double *dist1, int64_t *idx1, double *dist2,
+                                      int64_t *idx2, void *stream);
+
+/* Replaces chamfer_distance_backward_cuda
+ * (chamfer_distance.h:10-16, chamfer_distance_kernel.cu:200-274).
+ * grad_xyz1[b,i] = 2*gd1[b,i]*(x1[b,i]-x2[b,idx1[b,i]])
+ *                  - sum over {j: idx2[b,j]==i} 2*gd2[b,j]*(x2[b,j]-x1[b,i]),
+ * and symmetrically for grad_xyz2. Index entries outside [0,N) contribute nothing. */
+int tk3d_chamfer_distance_backward_f32(const float *grad_dist1,
+                                       const float *grad_dist2, const float *xyz1,
+                                       const float *xyz2, const int64_t *idx1,
+                                       const int64_t *idx2, int64_t B, int64_t N1,
+                                       int64_t N2, float *grad_xyz1,
+                                       float *grad_xyz2, void *stream);
+int tk3d_chamfer_distance_backward_f64(const double *grad_dist1,
+                                       const double *grad_dist2,
+                                       const double *xyz1, const double *xyz2,
+                                       const int64_t *idx1, const int64_t *idx2,
+                                       int64_t B, int64_t N1, int64_t N2,
+                                       double *grad_xyz1, double *grad_xyz2,
+                                       void *stream);
+
+/* ---- k nearest neighbours --------------------------------------------------
+ * Replaces knn_distance_cuda
+ * (torkit3d/csrc/include/knn_distance.h:7-11, cuda/knn_distance_kernel.cu:187-298).
+ * distance/index are [B,N1,k]: the k smallest squared distances and their key
+ * indices in the slot order of the reference's MinK structure
+ * (torkit3d/csrc/include/mink.cuh:61-89), not sorted. Requires 1 <= k <= N2.
+ * `version` (0 or 1) selects between two kernels in the reference that return
+ * identical results; it is validated and otherwise ignored. */
+int tk3d_knn_distance_f32(const float *query, const float *key, int64_t B,
+                          int64_t N1, int64_t N2, int64_t k, int version,
+                          float *distance, int64_t *index, void *stream);
+int tk3d_knn_distance_f64(const double *query, const double *key, int64_t B,
+                          int64_t N1, int64_t N2, int64_t k, int version,
+                          double *distance, int64_t *index, void *stream);
+
+/* ---- ball query --------------------------------------------------------------
+ * Replaces ball_query_cuda
+ * (torkit3d/csrc/include/ball_query.h:6-10, cuda/ball_query_kernel.cu:105-173).
+ * index[b,i,:] = the first max_neighbors key indices j (ascending) with
+ * d2(key[b,j], query[b,i]) < r*r, r = radius converted to the data type; slots
+ * after the last hit repeat the first hit; a row with no hit is all -1. */
+int tk3d_ball_query_f32(const float *query, const float *key, int64_t B,
+                        int64_t N1, int64_t N2, float radius,
+                        int64_t max_neighbors, int64_t *index, void *stream);
+int tk3d_ball_query_f64(const double *query, const double *key, int64_t B,
+                        int64_t N1, int64_t N2, float radius,
+                        int64_t max_neighbors, int64_t *index, void *stream);
+
+/* ---- farthest point sampling ---------------------------------------------------
+ * Replaces sample_farthest_points_cuda
+ * (torkit3d/csrc/include/sample_farthest_points.h:6-8,
+ *  cuda/sample_farthest_points_kernel.cu:106-165).
+ * index[b,0] = 0; index[b,i] = the point farthest from {index[b,0..i-1]}.
+ * Exact ties for the maximum are resolved as the reference kernel resolves them
+ * (its per-thread scan and shared-memory tree, block size = the power of two
+ * >= N capped at 512). Requires 1 <= num_samples <= N.
+ *
+ * Clouds too large for the register-resident kernel need a device workspace of
+ * tk3d_sample_farthest_points_workspace_bytes(B, N, elem_size) bytes (0 when none
+ * is needed; then `workspace` may be NULL). */
+size_t tk3d_sample_farthest_points_workspace_bytes(int64_t B, int64_t N,
+                                                   size_t elem_size);
+int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,
+                                    int64_t num_samples, int64_t *index,
+                                    void *workspace, size_t workspace_bytes,
+                                    void *stream);
+int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
+                                    int64_t num_samples, int64_t *index,
+                                    void *workspace, size_t workspace_bytes,
+                                    void *stream);
+
+/* ---- group points (gather) -------------------------------------------------------
+ * Replaces group_points_forward_cuda / group_points_backward_cuda
+ * (torkit3d/csrc/include/group_points.h:6-13, cuda/group_points_kernel.cu:8-114).
+ * forward:  output[b,c,m,s] = input[b,c,index[b,m,s]]          output [B,C,N2,K]
+ * backward: grad_input[b,c,index[b,m,s]] += grad_output[b,c,m,s] grad_input [B,C,N1]
+ * An index outside [0,N1) reads as 0 / contributes nothing (the reference
+ * asserts on the device). */
+int tk3d_group_points_forward_f32(const float *input, const int64_t *index,
+                                  int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                  int64_t K, float *output, void *stream);
+int tk3d_group_points_forward_f64(const double *input, const int64_t *index,
+                                  int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                  int64_t K, double *output, void *stream);
+int tk3d_group_points_backward_f32(const float *grad_output, const int64_t *index,
+                                   int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                   int64_t K, float *grad_input, void *stream);
+int tk3d_group_points_backward_f64(const double *grad_output,
+                                   const int64_t *index, int64_t B, int64_t C,
+                                   int64_t N1, int64_t N2, int64_t K,
+                                   double *grad_input, void *stream);
+
+/* ---- feature interpolation ----------------------------------------------------------
+ * Replaces interpolate_forward_cuda / interpolate_backward_cuda
+ * (torkit3d/csrc/include/interpolate.h:7-16, cuda/interpolate_kernel.cu:49-201).
+ * forward:  output[b,c,n] = sum_{i<K} input[b,c,index[b,n,i]] * weight[b,n,i]
+ * backward: grad_input[b,c,index[b,n,i]] += grad_output[b,c,n] * weight[b,n,i]
+ * The reference accepts K == 3 only; this library takes 1 <= K <= 8. */
+int tk3d_interpolate_forward_f32(const float *input, const int64_t *index,
+                                 const float *weight, int64_t B, int64_t C,
+                                 int64_t N1, int64_t N2, int64_t K, float *output,
+                                 void *stream);
+int tk3d_interpolate_forward_f64(const double *input, const int64_t *index,
+                                 const double *weight, int64_t B, int64_t C,
+                                 int64_t N1, int64_t N2, int64_t K, double *output,
+                                 void *stream);
+int tk3d_interpolate_backward_f32(const float *grad_output, const int64_t *index,
+                                  const float *weight, int64_t B, int64_t C,
+                                  int64_t N1, int64_t N2, int64_t K,
+                                  float *grad_input, void *stream);
+int tk3d_interpolate_backward_f64(const double *grad_output, const int64_t *index,
+                                  const double *weight, int64_t B, int64_t C,
+                                  int64_t N1, int64_t N2, int64_t K,
+                                  double *grad_input, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TK3D_H */

@@ -1,0 +1,67 @@
+"""ctypes loader for ``libtk3d.so`` (the hand-written HIP kernels behind a C ABI).
+
+There is no CPU fallback: if the library is missing or a call fails, an exception
+is raised.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads the HIP runtime the library resolves against)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtk3d.so")
+_lib = None
+
+
+def lib():
+    """The loaded ``libtk3d.so``; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "torkit3d_amd: %s is missing; build it with `python -m torkit3d_amd.build` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        handle.tk3d_error_string.restype = ctypes.c_char_p
+        handle.tk3d_error_string.argtypes = [ctypes.c_int]
+        handle.tk3d_version.restype = ctypes.c_int
+        _lib = handle
+    return _lib
+
+
+def error_string(code):
+    return lib().tk3d_error_string(int(code)).decode()
+
+
+def check(code, what):
+    """Raise RuntimeError (as TORCH_CHECK does in the reference) on a non-zero code."""
+    if code != 0:
+        raise RuntimeError("%s failed: %s (code %d)" % (what, error_string(code), code))
+
+
+def ptr(t):
+    """Device pointer of a tensor as a ctypes void pointer (NULL for empty tensors)."""
+    return ctypes.c_void_p(t.data_ptr() if t.numel() > 0 else 0)
+
+
+def i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def stream_of(t):
+    """The torch current stream on the tensor's device, as a void pointer."""
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def suffix(t):
+    if t.dtype == torch.float32:
+        return "_f32"
+    if t.dtype == torch.float64:
+        return "_f64"
+    raise RuntimeError("torkit3d_amd supports float32 and float64 tensors, got %s" % t.dtype)
+
+
+def call(name, tensor_for_dtype, *args):
+    fn = getattr(lib(), name + suffix(tensor_for_dtype))
+    fn.restype = ctypes.c_int
+    check(fn(*args), name)

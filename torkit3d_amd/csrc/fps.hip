@@ -1,0 +1,370 @@
+// Farthest point sampling for gfx950.
+//
+// One workgroup samples one cloud. The K-1 selection steps are strictly serial, so
+// the kernel is built for latency per step, not throughput:
+//   * every lane keeps P points and their running minimum distance in registers
+//     for the whole kernel - the loop touches no global memory except the one
+//     index it emits per step;
+//   * per step a lane updates its P minima and finds its local maximum, the wave
+//     reduces with DPP row shifts / row broadcasts (no LDS), ballot + find-first
+//     pick the winning lane on the scalar unit;
+//   * waves exchange (value, point index, xyz) through double-buffered LDS slots,
+//     so a step costs a single s_barrier, and every wave redoes the tiny
+//     cross-wave reduction itself instead of waiting for a broadcast.
+//
+// Ties. The reference resolves equal maxima by its thread layout: thread t scans
+// j = t, t+BS, ... keeping the first maximum, then a shared-memory tree keeps the
+// left operand (sample_farthest_points_kernel.cu:46-72, :75-95), i.e. the winner
+// is the candidate with the smallest (bit-reversed t, j / BS). The points are
+// laid out here in exactly that priority order ("positions"), lanes take
+// consecutive positions, and every reduction keeps the lowest position among
+// equal values, which reproduces the reference's choice.
+#include "tk3d_common.h"
+
+namespace {
+
+template <typename T> struct Bits;
+template <> struct Bits<float> { using type = int; };
+template <> struct Bits<double> { using type = long long; };
+
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_move(float v)
+{
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),
+                                           __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF,
+                                           false));
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ double dpp_move(double v)
+{
+    const long long b = __builtin_bit_cast(long long, v);
+    int lo = (int)b, hi = (int)(b >> 32);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xF, false);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xF, false);
+    return __builtin_bit_cast(double,
+                              ((long long)hi << 32) | (long long)(unsigned)lo);
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane)
+{
+    return __builtin_bit_cast(float,
+                              __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ int read_lane(int v, int lane)
+{
+    return __builtin_amdgcn_readlane(v, lane);
+}
+__device__ __forceinline__ double read_lane(double v, int lane)
+{
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_readlane((int)b, lane);
+    const int hi = __builtin_amdgcn_readlane((int)(b >> 32), lane);
+    return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)(unsigned)lo);
+}
+
+// Maximum over the 64 lanes, returned as a wave-uniform value. Inclusive scan
+// inside each row of 16 (row_shr 1,2,4,8), then row_bcast15 / row_bcast31 carry
+// the row totals up so that lane 63 holds the result.
+template <typename T> __device__ __forceinline__ T wave_max(T v)
+{
+    v = tk_max<T>(v, dpp_move<0x111, 0xF>(v));
+    v = tk_max<T>(v, dpp_move<0x112, 0xF>(v));
+    v = tk_max<T>(v, dpp_move<0x114, 0xF>(v));
+    v = tk_max<T>(v, dpp_move<0x118, 0xF>(v));
+    v = tk_max<T>(v, dpp_move<0x142, 0xA>(v));
+    v = tk_max<T>(v, dpp_move<0x143, 0xC>(v));
+    return read_lane(v, 63);
+}
+
+struct FpsLayout {
+    int n;        // points per cloud
+    int k;        // samples per cloud
+    int bs;       // the reference's block size for this n (power of two, 32..512)
+    int log2_bs;
+    int c;        // ceil(n / bs): points per reference thread
+    float inv_c;  // 1 / c
+};
+
+// Point index of a position in the priority order described at the top.
+__device__ __forceinline__ int fps_point_of_position(int pos, const FpsLayout &L)
+{
+    int r = (int)(((float)pos + 0.5f) * L.inv_c);
+    // One correction step makes the float estimate exact for every pos < 2^24.
+    r += ((r + 1) * L.c <= pos) ? 1 : 0;
+    r -= (r * L.c > pos) ? 1 : 0;
+    const int cc = pos - r * L.c;
+    const int t = (int)(__builtin_bitreverse32((unsigned)r) >> (32 - L.log2_bs));
+    return t + cc * L.bs;
+}
+
+template <typename T, int P, int NT>
+__global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ points,
+                                                          int64_t *__restrict__ index,
+                                                          FpsLayout L)
+{
+    constexpr int NW = NT / TK_WAVE;
+    __shared__ T s_val[2][NW], s_x[2][NW], s_y[2][NW], s_z[2][NW];
+    __shared__ int s_j[2][NW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const T *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
+    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
+
+    T x[P], y[P], z[P], md[P];
+    const int npos = L.bs * L.c;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int pos = tid * P + p;
+        const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
+        const bool ok = j < L.n;
+        x[p] = ok ? pts[(int64_t)j * 3 + 0] : (T)0;
+        y[p] = ok ? pts[(int64_t)j * 3 + 1] : (T)0;
+        z[p] = ok ? pts[(int64_t)j * 3 + 2] : (T)0;
+        // Unused slots sit at -1: min() keeps them there and they never exceed 0.
+        md[p] = ok ? tk_inf<T>() : (T)-1;
+    }
+
+    int sel_j = 0;
+    T cx = pts[0], cy = pts[1], cz = pts[2];
+    if (tid == 0)
+        out[0] = 0;
+
+    for (int it = 1; it < L.k; ++it) {
+        // Lane-local update and first maximum above zero (strict '>' from zero, as
+        // the reference thread does).
+        T best = (T)0;
+        int bp = 0;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const T d = tk_dist2<T>(x[p], y[p], z[p], cx, cy, cz);
+            md[p] = tk_min<T>(md[p], d);
+            const bool up = md[p] > best;
+            best = up ? md[p] : best;
+            bp = up ? p : bp;
+        }
+        const T wmax = wave_max<T>(best);
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(best == wmax);
+        const int wl = __builtin_ctzll(hit);  // lowest lane holding the maximum
+        const int wp = read_lane(bp, wl);
+        T sx = x[0], sy = y[0], sz = z[0];
+#pragma unroll
+        for (int p = 1; p < P; ++p) {
+            if (wp == p) {  // wave-uniform: a scalar branch
+                sx = x[p];
+                sy = y[p];
+                sz = z[p];
+            }
+        }
+        // Cross-lane reads happen with the whole wave active: a lane switched off
+        // by a branch has no defined value to hand over.
+        const T wx = read_lane(sx, wl), wy = read_lane(sy, wl), wz = read_lane(sz, wl);
+        const int wj = fps_point_of_position((wave * TK_WAVE + wl) * P + wp, L);
+        const int buf = it & 1;
+        if (lane == 0) {
+            s_val[buf][wave] = wmax;
+            s_j[buf][wave] = wj;
+            s_x[buf][wave] = wx;
+            s_y[buf][wave] = wy;
+            s_z[buf][wave] = wz;
+        }
+        __syncthreads();
+        // Every wave reduces the NW candidates itself. Lower waves hold lower
+        // positions, so the lowest lane among equal values is the right winner.
+        const bool has = lane < NW;
+        const T cv = has ? s_val[buf][has ? lane : 0] : (T)-1;
+        const T gmax = wave_max<T>(cv);
+        if (gmax > (T)0) {
+            const int gl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(cv == gmax));
+            sel_j = s_j[buf][gl];
+            cx = s_x[buf][gl];
+            cy = s_y[buf][gl];
+            cz = s_z[buf][gl];
+        }
+        // gmax == 0: no point lies away from the chosen set; the previous choice
+        // is emitted again, as the reference does.
+        if (tid == 0)
+            out[it] = (int64_t)sel_j;
+    }
+}
+
+// Clouds that do not fit in registers: minimum distances live in a global
+// workspace, coordinates are re-read every step (they stay in L2). Same selection
+// rule; positions are visited in priority order so the tie rule is unchanged.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__ points,
+                                                           int64_t *__restrict__ index,
+                                                           T *__restrict__ min_dist,
+                                                           FpsLayout L)
+{
+    constexpr int NW = NT / TK_WAVE;
+    __shared__ T s_val[2][NW];
+    __shared__ int s_pos[2][NW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const T *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
+    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
+    T *__restrict__ md = min_dist + (int64_t)blockIdx.x * L.bs * L.c;
+
+    const int npos = L.bs * L.c;
+    // A thread owns a contiguous run of positions so that thread order == position order.
+    const int per = (npos + NT - 1) / NT;
+    const int p0 = tid * per;
+    const int p1 = (p0 + per < npos) ? p0 + per : npos;
+    for (int pos = p0; pos < p1; ++pos)
+        md[pos] = fps_point_of_position(pos, L) < L.n ? tk_inf<T>() : (T)-1;
+
+    int sel_j = 0;
+    if (tid == 0)
+        out[0] = 0;
+    for (int it = 1; it < L.k; ++it) {
+        const T cx = pts[(int64_t)sel_j * 3 + 0], cy = pts[(int64_t)sel_j * 3 + 1],
+                cz = pts[(int64_t)sel_j * 3 + 2];
+        T best = (T)0;
+        int bpos = 0;
+        for (int pos = p0; pos < p1; ++pos) {
+            const T m = md[pos];
+            if (m < (T)0)
+                continue;
+            const int j = fps_point_of_position(pos, L);
+            const T d = tk_dist2<T>(pts[(int64_t)j * 3 + 0], pts[(int64_t)j * 3 + 1],
+                                    pts[(int64_t)j * 3 + 2], cx, cy, cz);
+            const T nm = tk_min<T>(m, d);
+            md[pos] = nm;
+            if (nm > best) {
+                best = nm;
+                bpos = pos;
+            }
+        }
+        const T wmax = wave_max<T>(best);
+        const int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
+        const int wpos = read_lane(bpos, wl);
+        const int buf = it & 1;
+        if (lane == 0) {
+            s_val[buf][wave] = wmax;
+            s_pos[buf][wave] = wpos;
+        }
+        __syncthreads();
+        const bool has = lane < NW;
+        const T cv = has ? s_val[buf][has ? lane : 0] : (T)-1;
+        const T gmax = wave_max<T>(cv);
+        if (gmax > (T)0) {
+            const int gl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(cv == gmax));
+            sel_j = fps_point_of_position(s_pos[buf][gl], L);
+        }
+        if (tid == 0)
+            out[it] = (int64_t)sel_j;
+    }
+}
+
+FpsLayout fps_layout(int64_t n, int64_t k)
+{
+    FpsLayout L;
+    L.n = (int)n;
+    L.k = (int)k;
+    int bs = 1, lg = 0;
+    // Block size of the reference: smallest power of two >= n, capped at 512
+    // (sample_farthest_points_kernel.cu:132-133); its switch runs 32 threads for
+    // anything smaller (:153-161).
+    while (bs < n && bs < 512) {
+        bs *= 2;
+        ++lg;
+    }
+    while (bs < 32) {
+        bs *= 2;
+        ++lg;
+    }
+    L.bs = bs;
+    L.log2_bs = lg;
+    L.c = (int)((n + bs - 1) / bs);
+    L.inv_c = 1.0f / (float)L.c;
+    return L;
+}
+
+// Largest number of positions the register kernel holds for element size `es`.
+int64_t fps_register_capacity(size_t es) { return es == 4 ? 1024 * 16 : 1024 * 8; }
+
+template <typename T, int P, int NT>
+void fps_launch(const T *points, int64_t B, int64_t *index, const FpsLayout &L,
+                hipStream_t s)
+{
+    hipLaunchKernelGGL((fps_register_kernel<T, P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
+                       points, index, L);
+}
+
+template <typename T>
+int fps(const T *points, int64_t B, int64_t N, int64_t K, int64_t *index, void *workspace,
+        size_t workspace_bytes, void *stream)
+{
+    if (B < 0 || N < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (K <= 0 || K > N)
+        return TK3D_ERR_BAD_K;
+    if (N > ((int64_t)1 << 23) || B > TK_MAX_I32 || !tk_fits(TK_MAX_ELEMS, B, N, 3))
+        return TK3D_ERR_UNSUPPORTED;
+    if (B == 0)
+        return TK3D_OK;
+    if (!points || !index)
+        return TK3D_ERR_NULL_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    const FpsLayout L = fps_layout(N, K);
+    const int64_t npos = (int64_t)L.bs * L.c;
+    if (npos <= fps_register_capacity(sizeof(T))) {
+        // Fewest points per lane that still covers the cloud: short serial chains.
+        if (npos <= 256 * 1)
+            fps_launch<T, 1, 256>(points, B, index, L, s);
+        else if (npos <= 256 * 2)
+            fps_launch<T, 2, 256>(points, B, index, L, s);
+        else if (npos <= 512 * 2)
+            fps_launch<T, 2, 512>(points, B, index, L, s);
+        else if (npos <= 1024 * 2)
+            fps_launch<T, 2, 1024>(points, B, index, L, s);
+        else if (npos <= 1024 * 4)
+            fps_launch<T, 4, 1024>(points, B, index, L, s);
+        else if (npos <= 1024 * 8)
+            fps_launch<T, 8, 1024>(points, B, index, L, s);
+        else if constexpr (sizeof(T) == 4)
+            fps_launch<T, 16, 1024>(points, B, index, L, s);
+        return tk_launch_status();
+    }
+    const size_t need = (size_t)B * (size_t)npos * sizeof(T);
+    if (!workspace || workspace_bytes < need)
+        return TK3D_ERR_WORKSPACE;
+    hipLaunchKernelGGL((fps_streaming_kernel<T, 1024>), dim3((unsigned)B), dim3(1024), 0, s,
+                       points, index, (T *)workspace, L);
+    return tk_launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t tk3d_sample_farthest_points_workspace_bytes(int64_t B, int64_t N, size_t elem_size)
+{
+    if (B <= 0 || N <= 0 || (elem_size != 4 && elem_size != 8))
+        return 0;
+    const FpsLayout L = fps_layout(N, 1);
+    const int64_t npos = (int64_t)L.bs * L.c;
+    if (npos <= fps_register_capacity(elem_size))
+        return 0;
+    return (size_t)B * (size_t)npos * elem_size;
+}
+
+int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,
+                                    int64_t num_samples, int64_t *index, void *workspace,
+                                    size_t workspace_bytes, void *stream)
+{
+    return fps<float>(points, B, N, num_samples, index, workspace, workspace_bytes, stream);
+}
+
+int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
+                                    int64_t num_samples, int64_t *index, void *workspace,
+                                    size_t workspace_bytes, void *stream)
+{
+    return fps<double>(points, B, N, num_samples, index, workspace, workspace_bytes,
+                       stream);
+}
+
+}  // extern "C"

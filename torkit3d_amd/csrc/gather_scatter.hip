@@ -1,0 +1,433 @@
+// Group points (gather) and feature interpolation for gfx950, forward and backward.
+//
+// Both ops are the same two memory-bound patterns over feature rows [B,C,N1]:
+//
+//   gather :  out[b,c,p]            = sum_{i<KK} in[b,c,idx[b,p,i]] * w[b,p,i]
+//   scatter:  gin[b,c,idx[b,p,i]] += gout[b,c,p] * w[b,p,i]
+//
+// group points is KK = 1 without weights over p = (m,s) flattened (N2*K points);
+// interpolation is KK = K (3 in the reference) with weights over p = n.
+//
+// gather: a workgroup owns a tile of p and a group of channels. The indices (and
+// weights) of the tile are read once, checked, narrowed to 32 bits and kept in
+// registers; the channel loop then issues only the row gathers and one coalesced
+// store per channel, where the reference re-reads index and weight for every
+// channel (interpolate_kernel.cu:34-41) or pays ATen's generic gather
+// (group_points_kernel.cu:26-29).
+//
+// scatter: a workgroup owns CG destination rows [CG][N1] in LDS, streams its
+// share of p with coalesced reads of gout and accumulates with LDS float atomics
+// (ds_add), then writes the rows out with plain coalesced stores - no global
+// atomics and no zero-fill when one workgroup covers all p. When B*C is too
+// small to fill the chip the p range is split over several workgroups that merge
+// into a zero-filled output with global atomics. Rows too long for LDS use
+// global atomics directly. Summation order differs from run to run exactly as in
+// the reference (which uses one global atomicAdd per element,
+// group_points_kernel.cu:63, interpolate_kernel.cu:142).
+#include "tk3d_common.h"
+
+namespace {
+
+constexpr int GS_BLOCK = 256;
+
+// ---- gather -------------------------------------------------------------------
+
+template <typename T, int KK, bool HAS_W, int V>
+__global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
+    const T *__restrict__ in, const int64_t *__restrict__ idx, const T *__restrict__ w,
+    T *__restrict__ out, int c_total, int n1, int64_t np, int cg, int vec_ok)
+{
+    const int b = blockIdx.z;
+    const int c0 = blockIdx.y * cg;
+    const int c1 = (c0 + cg < c_total) ? c0 + cg : c_total;
+    const int64_t p0 = ((int64_t)blockIdx.x * GS_BLOCK + threadIdx.x) * V;
+    if (p0 >= np)
+        return;
+
+    int src[V][KK];
+    T wt[V][KK];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+#pragma unroll
+        for (int i = 0; i < KK; ++i) {
+            const int64_t p = p0 + v;
+            int64_t j = -1;
+            T ww = (T)0;
+            if (p < np) {
+                j = idx[((int64_t)b * np + p) * KK + i];
+                if (HAS_W)
+                    ww = w[((int64_t)b * np + p) * KK + i];
+            }
+            const bool ok = j >= 0 && j < n1;
+            src[v][i] = ok ? (int)j : -1;
+            wt[v][i] = ww;
+        }
+    }
+
+    const bool full = (p0 + V <= np);
+    for (int c = c0; c < c1; ++c) {
+        const T *__restrict__ row = in + ((int64_t)b * c_total + c) * n1;
+        T *__restrict__ orow = out + ((int64_t)b * c_total + c) * np;
+        T val[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            if (HAS_W) {
+                // out = 0; out = fma(in, w, out) per neighbour, in slot order
+                // (interpolate_kernel.cu:31-42 under default contraction).
+                T acc = (T)0;
+#pragma unroll
+                for (int i = 0; i < KK; ++i)
+                    if (src[v][i] >= 0)
+                        acc = tk_fma<T>(row[src[v][i]], wt[v][i], acc);
+                val[v] = acc;
+            } else {
+                val[v] = src[v][0] >= 0 ? row[src[v][0]] : (T)0;
+            }
+        }
+        if (full && vec_ok && V == 4 && sizeof(T) == 4) {
+            float4 pack;
+            pack.x = (float)val[0];
+            pack.y = (float)val[1 % V];
+            pack.z = (float)val[2 % V];
+            pack.w = (float)val[3 % V];
+            *reinterpret_cast<float4 *>(orow + p0) = pack;
+        } else if (full && vec_ok && V == 2 && sizeof(T) == 8) {
+            double2 pack;
+            pack.x = (double)val[0];
+            pack.y = (double)val[1 % V];
+            *reinterpret_cast<double2 *>(orow + p0) = pack;
+        } else {
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                if (p0 + v < np)
+                    orow[p0 + v] = val[v];
+        }
+    }
+}
+
+// ---- scatter ---------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(GS_BLOCK) void fill_zero_kernel(T *__restrict__ p, int64_t n)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        p[i] = (T)0;
+}
+
+// LDS-resident destination rows. grid = (segments, channel groups, B).
+template <typename T, int KK, bool HAS_W, int NT>
+__global__ __launch_bounds__(NT) void scatter_lds_kernel(
+    const T *__restrict__ gout, const int64_t *__restrict__ idx, const T *__restrict__ w,
+    T *__restrict__ gin, int c_total, int n1, int64_t np, int cg, int64_t seg_len,
+    int merge_with_atomics)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *rows = reinterpret_cast<T *>(smem_raw);  // [cg][n1]
+    const int b = blockIdx.z;
+    const int c0 = blockIdx.y * cg;
+    const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
+    const int64_t ps = (int64_t)blockIdx.x * seg_len;
+    const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
+
+    for (int i = threadIdx.x; i < nc * n1; i += NT)
+        rows[i] = (T)0;
+    __syncthreads();
+
+    for (int64_t p = ps + threadIdx.x; p < pe; p += NT) {
+        int dst[KK];
+        T wt[KK];
+#pragma unroll
+        for (int i = 0; i < KK; ++i) {
+            const int64_t j = idx[((int64_t)b * np + p) * KK + i];
+            dst[i] = (j >= 0 && j < n1) ? (int)j : -1;
+            wt[i] = HAS_W ? w[((int64_t)b * np + p) * KK + i] : (T)1;
+        }
+        for (int c = 0; c < nc; ++c) {
+            const T g = gout[((int64_t)b * c_total + c0 + c) * np + p];
+#pragma unroll
+            for (int i = 0; i < KK; ++i)
+                if (dst[i] >= 0)
+                    atomicAdd(&rows[c * n1 + dst[i]], HAS_W ? g * wt[i] : g);
+        }
+    }
+    __syncthreads();
+
+    T *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
+    if (merge_with_atomics) {
+        for (int i = threadIdx.x; i < nc * n1; i += NT) {
+            const T v = rows[i];
+            if (v != (T)0)
+                unsafeAtomicAdd(&dstrows[i], v);
+        }
+    } else {
+        for (int i = threadIdx.x; i < nc * n1; i += NT)
+            dstrows[i] = rows[i];
+    }
+}
+
+// Rows too long for LDS: one global atomic per contribution into a zero-filled
+// output.
+template <typename T, int KK, bool HAS_W>
+__global__ __launch_bounds__(GS_BLOCK) void scatter_global_kernel(
+    const T *__restrict__ gout, const int64_t *__restrict__ idx, const T *__restrict__ w,
+    T *__restrict__ gin, int c_total, int n1, int64_t np, int cg)
+{
+    const int b = blockIdx.z;
+    const int c0 = blockIdx.y * cg;
+    const int c1 = (c0 + cg < c_total) ? c0 + cg : c_total;
+    const int64_t p = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
+    if (p >= np)
+        return;
+    int dst[KK];
+    T wt[KK];
+#pragma unroll
+    for (int i = 0; i < KK; ++i) {
+        const int64_t j = idx[((int64_t)b * np + p) * KK + i];
+        dst[i] = (j >= 0 && j < n1) ? (int)j : -1;
+        wt[i] = HAS_W ? w[((int64_t)b * np + p) * KK + i] : (T)1;
+    }
+    for (int c = c0; c < c1; ++c) {
+        const T g = gout[((int64_t)b * c_total + c) * np + p];
+        T *row = gin + ((int64_t)b * c_total + c) * n1;
+#pragma unroll
+        for (int i = 0; i < KK; ++i)
+            if (dst[i] >= 0)
+                unsafeAtomicAdd(&row[dst[i]], HAS_W ? g * wt[i] : g);
+    }
+}
+
+// ---- host ------------------------------------------------------------------------------
+
+int check_shape(int64_t B, int64_t C, int64_t N1, int64_t NP, int64_t KK)
+{
+    if (B < 0 || C < 0 || N1 < 0 || NP < 0 || KK < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (N1 > TK_MAX_I32 / 4 || C > TK_MAX_I32 / 4 || B > 65535 ||
+        !tk_fits(TK_MAX_ELEMS, B, C, N1) || !tk_fits(TK_MAX_ELEMS, B, C, NP) ||
+        !tk_fits(TK_MAX_ELEMS, B, NP, KK > 0 ? KK : 1))
+        return TK3D_ERR_UNSUPPORTED;
+    return TK3D_OK;
+}
+
+template <typename T, int KK, bool HAS_W>
+int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, int64_t N1,
+           int64_t NP, T *out, hipStream_t s)
+{
+    if (B * C * NP == 0)
+        return TK3D_OK;
+    if (!in && N1 > 0)
+        return TK3D_ERR_NULL_POINTER;
+    if (!idx || !out || (HAS_W && !w))
+        return TK3D_ERR_NULL_POINTER;
+    constexpr int V = (sizeof(T) == 4) ? 4 : 2;
+    const int64_t tiles = (NP + (int64_t)GS_BLOCK * V - 1) / ((int64_t)GS_BLOCK * V);
+    // Channels per workgroup: enough to amortise the index reads, few enough to
+    // keep at least ~2k workgroups in flight.
+    int cg = 16;
+    while (cg > 1 && tiles * ((C + cg - 1) / cg) * B < 2048)
+        cg /= 2;
+    const int64_t gy = (C + cg - 1) / cg;
+    if (tiles > TK_MAX_I32 || gy > 65535)
+        return TK3D_ERR_UNSUPPORTED;
+    // 16-byte stores need every output row to start on a 16-byte boundary.
+    const int vec_ok = (((uintptr_t)out & 15) == 0) && ((NP * (int64_t)sizeof(T)) % 16 == 0);
+    hipLaunchKernelGGL((gather_kernel<T, KK, HAS_W, V>),
+                       dim3((unsigned)tiles, (unsigned)gy, (unsigned)B), dim3(GS_BLOCK), 0, s,
+                       in, idx, w, out, (int)C, (int)N1, NP, cg, vec_ok);
+    return tk_launch_status();
+}
+
+template <typename T, int KK, bool HAS_W>
+int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C, int64_t N1,
+            int64_t NP, T *gin, hipStream_t s)
+{
+    const int64_t out_elems = B * C * N1;
+    if (out_elems == 0)
+        return TK3D_OK;
+    if (!gin)
+        return TK3D_ERR_NULL_POINTER;
+    if (NP > 0 && (!gout || !idx || (HAS_W && !w)))
+        return TK3D_ERR_NULL_POINTER;
+    int64_t zero_blocks = (out_elems + GS_BLOCK - 1) / GS_BLOCK;
+    if (zero_blocks > 16384)
+        zero_blocks = 16384;
+    if (NP == 0) {
+        hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks), dim3(GS_BLOCK),
+                           0, s, gin, out_elems);
+        return tk_launch_status();
+    }
+
+    constexpr int64_t LDS_BUDGET = 64 * 1024;
+    const int64_t row_bytes = N1 * (int64_t)sizeof(T);
+    if (row_bytes <= LDS_BUDGET) {
+        constexpr int NT = 512;
+        int cg = 8;
+        while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
+            cg /= 2;
+        // Prefer more workgroups over wider channel groups until the chip is full.
+        while (cg > 1 && B * ((C + cg - 1) / cg) < 512)
+            cg /= 2;
+        const int64_t gy = (C + cg - 1) / cg;
+        int64_t nseg = 1;
+        const int64_t groups = B * gy;
+        if (groups < 256) {
+            nseg = (512 + groups - 1) / groups;
+            const int64_t max_seg = (NP + 4 * NT - 1) / (4 * NT);  // >= 4 points per thread
+            if (nseg > max_seg)
+                nseg = max_seg;
+            if (nseg < 1)
+                nseg = 1;
+        }
+        const int64_t seg_len = (NP + nseg - 1) / nseg;
+        nseg = (NP + seg_len - 1) / seg_len;
+        if (gy > 65535 || nseg > TK_MAX_I32)
+            return TK3D_ERR_UNSUPPORTED;
+        if (nseg > 1)
+            hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
+                               dim3(GS_BLOCK), 0, s, gin, out_elems);
+        hipLaunchKernelGGL((scatter_lds_kernel<T, KK, HAS_W, NT>),
+                           dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
+                           (size_t)(cg * row_bytes), s, gout, idx, w, gin, (int)C, (int)N1, NP,
+                           cg, seg_len, nseg > 1 ? 1 : 0);
+        return tk_launch_status();
+    }
+
+    hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks), dim3(GS_BLOCK), 0, s,
+                       gin, out_elems);
+    const int64_t tiles = (NP + GS_BLOCK - 1) / GS_BLOCK;
+    int cg = 8;
+    while (cg > 1 && tiles * ((C + cg - 1) / cg) * B < 2048)
+        cg /= 2;
+    const int64_t gy = (C + cg - 1) / cg;
+    if (tiles > TK_MAX_I32 || gy > 65535)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((scatter_global_kernel<T, KK, HAS_W>),
+                       dim3((unsigned)tiles, (unsigned)gy, (unsigned)B), dim3(GS_BLOCK), 0, s,
+                       gout, idx, w, gin, (int)C, (int)N1, NP, cg);
+    return tk_launch_status();
+}
+
+template <typename T>
+int interpolate_forward(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C,
+                        int64_t N1, int64_t N2, int64_t K, T *out, void *stream)
+{
+    const int rc = check_shape(B, C, N1, N2, K);
+    if (rc != TK3D_OK)
+        return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (K) {
+    case 1: return gather<T, 1, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 2: return gather<T, 2, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 3: return gather<T, 3, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 4: return gather<T, 4, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 5: return gather<T, 5, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 6: return gather<T, 6, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 7: return gather<T, 7, true>(in, idx, w, B, C, N1, N2, out, s);
+    case 8: return gather<T, 8, true>(in, idx, w, B, C, N1, N2, out, s);
+    default: return TK3D_ERR_BAD_K;
+    }
+}
+
+template <typename T>
+int interpolate_backward(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
+                         int64_t N1, int64_t N2, int64_t K, T *gin, void *stream)
+{
+    const int rc = check_shape(B, C, N1, N2, K);
+    if (rc != TK3D_OK)
+        return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (K) {
+    case 1: return scatter<T, 1, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 2: return scatter<T, 2, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 3: return scatter<T, 3, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 4: return scatter<T, 4, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 5: return scatter<T, 5, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 6: return scatter<T, 6, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 7: return scatter<T, 7, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    case 8: return scatter<T, 8, true>(gout, idx, w, B, C, N1, N2, gin, s);
+    default: return TK3D_ERR_BAD_K;
+    }
+}
+
+template <typename T>
+int group_forward(const T *in, const int64_t *idx, int64_t B, int64_t C, int64_t N1,
+                  int64_t N2, int64_t K, T *out, void *stream)
+{
+    if (N2 < 0 || K < 0 || !tk_fits(TK_MAX_ELEMS, N2, K))
+        return N2 < 0 || K < 0 ? TK3D_ERR_BAD_SIZE : TK3D_ERR_UNSUPPORTED;
+    const int rc = check_shape(B, C, N1, N2 * K, 1);
+    if (rc != TK3D_OK)
+        return rc;
+    return gather<T, 1, false>(in, idx, nullptr, B, C, N1, N2 * K, out, (hipStream_t)stream);
+}
+
+template <typename T>
+int group_backward(const T *gout, const int64_t *idx, int64_t B, int64_t C, int64_t N1,
+                   int64_t N2, int64_t K, T *gin, void *stream)
+{
+    if (N2 < 0 || K < 0 || !tk_fits(TK_MAX_ELEMS, N2, K))
+        return N2 < 0 || K < 0 ? TK3D_ERR_BAD_SIZE : TK3D_ERR_UNSUPPORTED;
+    const int rc = check_shape(B, C, N1, N2 * K, 1);
+    if (rc != TK3D_OK)
+        return rc;
+    return scatter<T, 1, false>(gout, idx, nullptr, B, C, N1, N2 * K, gin,
+                                (hipStream_t)stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int tk3d_group_points_forward_f32(const float *input, const int64_t *index, int64_t B,
+                                  int64_t C, int64_t N1, int64_t N2, int64_t K,
+                                  float *output, void *stream)
+{
+    return group_forward<float>(input, index, B, C, N1, N2, K, output, stream);
+}
+int tk3d_group_points_forward_f64(const double *input, const int64_t *index, int64_t B,
+                                  int64_t C, int64_t N1, int64_t N2, int64_t K,
+                                  double *output, void *stream)
+{
+    return group_forward<double>(input, index, B, C, N1, N2, K, output, stream);
+}
+int tk3d_group_points_backward_f32(const float *grad_output, const int64_t *index, int64_t B,
+                                   int64_t C, int64_t N1, int64_t N2, int64_t K,
+                                   float *grad_input, void *stream)
+{
+    return group_backward<float>(grad_output, index, B, C, N1, N2, K, grad_input, stream);
+}
+int tk3d_group_points_backward_f64(const double *grad_output, const int64_t *index,
+                                   int64_t B, int64_t C, int64_t N1, int64_t N2, int64_t K,
+                                   double *grad_input, void *stream)
+{
+    return group_backward<double>(grad_output, index, B, C, N1, N2, K, grad_input, stream);
+}
+int tk3d_interpolate_forward_f32(const float *input, const int64_t *index,
+                                 const float *weight, int64_t B, int64_t C, int64_t N1,
+                                 int64_t N2, int64_t K, float *output, void *stream)
+{
+    return interpolate_forward<float>(input, index, weight, B, C, N1, N2, K, output, stream);
+}
+int tk3d_interpolate_forward_f64(const double *input, const int64_t *index,
+                                 const double *weight, int64_t B, int64_t C, int64_t N1,
+                                 int64_t N2, int64_t K, double *output, void *stream)
+{
+    return interpolate_forward<double>(input, index, weight, B, C, N1, N2, K, output, stream);
+}
+int tk3d_interpolate_backward_f32(const float *grad_output, const int64_t *index,
+                                  const float *weight, int64_t B, int64_t C, int64_t N1,
+                                  int64_t N2, int64_t K, float *grad_input, void *stream)
+{
+    return interpolate_backward<float>(grad_output, index, weight, B, C, N1, N2, K,
+                                       grad_input, stream);
+}
+int tk3d_interpolate_backward_f64(const double *grad_output, const int64_t *index,
+                                  const double *weight, int64_t B, int64_t C, int64_t N1,
+                                  int64_t N2, int64_t K, double *grad_input, void *stream)
+{
+    return interpolate_backward<double>(grad_output, index, weight, B, C, N1, N2, K,
+                                        grad_input, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,91 @@
+// Shared host/device helpers for the gfx950 point-cloud kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tk3d.h"
+
+// All kernels are written for 64-lane wavefronts.
+#define TK_WAVE 64
+
+// Every source file is compiled with -ffp-contract=off; the fused steps of the
+// canonical distance are written out here and nowhere else.
+template <typename T> __device__ __forceinline__ T tk_fma(T a, T b, T c);
+template <> __device__ __forceinline__ float tk_fma<float>(float a, float b, float c)
+{
+    return __builtin_fmaf(a, b, c);
+}
+template <> __device__ __forceinline__ double tk_fma<double>(double a, double b, double c)
+{
+    return __builtin_fma(a, b, c);
+}
+
+template <typename T> __device__ __forceinline__ T tk_min(T a, T b);
+template <> __device__ __forceinline__ float tk_min<float>(float a, float b)
+{
+    return __builtin_fminf(a, b);
+}
+template <> __device__ __forceinline__ double tk_min<double>(double a, double b)
+{
+    return __builtin_fmin(a, b);
+}
+template <typename T> __device__ __forceinline__ T tk_max(T a, T b);
+template <> __device__ __forceinline__ float tk_max<float>(float a, float b)
+{
+    return __builtin_fmaxf(a, b);
+}
+template <> __device__ __forceinline__ double tk_max<double>(double a, double b)
+{
+    return __builtin_fmax(a, b);
+}
+
+template <typename T> __device__ __forceinline__ T tk_inf()
+{
+    return (T)__builtin_huge_valf();
+}
+
+// Squared distance between key (kx,ky,kz) and query (qx,qy,qz):
+// fma(dz,dz, fma(dy,dy, dx*dx)) with dx = kx - qx, the value the reference
+// kernels produce (e.g. chamfer_distance_kernel.cu:65-71 under nvcc's default
+// contraction).
+template <typename T>
+__device__ __forceinline__ T tk_dist2(T kx, T ky, T kz, T qx, T qy, T qz)
+{
+    const T dx = kx - qx;
+    const T dy = ky - qy;
+    const T dz = kz - qz;
+    T d = dx * dx;
+    d = tk_fma<T>(dy, dy, d);
+    d = tk_fma<T>(dz, dz, d);
+    return d;
+}
+
+// ---- host side --------------------------------------------------------------
+
+static inline int tk_launch_status()
+{
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TK3D_OK : (int)e;
+}
+
+// True when a*b*c... of non-negative sizes fits in int64 and is below `limit`.
+static inline bool tk_fits(int64_t limit, int64_t a, int64_t b = 1, int64_t c = 1,
+                           int64_t d = 1)
+{
+    const int64_t v[4] = {a, b, c, d};
+    __int128 p = 1;
+    for (int i = 0; i < 4; ++i) {
+        if (v[i] < 0)
+            return false;
+        p *= v[i];
+        if (p > (__int128)limit)
+            return false;
+    }
+    return true;
+}
+
+// Largest element count a kernel addresses with a signed 64-bit offset in bytes.
+#define TK_MAX_ELEMS ((int64_t)1 << 58)
+// Largest value carried in a 32-bit in-kernel index.
+#define TK_MAX_I32 ((int64_t)0x7fffffff)

@@ -1,0 +1,34 @@
+"""Ball query (API of torkit3d/ops/ball_query.py)."""
+import torch
+
+from .. import _C
+
+
+class BallQueryFunction(torch.autograd.Function):
+    """Not differentiable (torkit3d/ops/ball_query.py:6-14)."""
+
+    @staticmethod
+    def forward(ctx, query, key, radius, max_neighbors):
+        index = _C.ball_query_cuda(query, key, radius, max_neighbors)
+        ctx.mark_non_differentiable(index)
+        return index
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        return (None,) * 4
+
+
+def ball_query(query, key, radius, max_neighbors, transpose=True):
+    """Neighbours of each query point within ``radius``.
+
+    Note the default ``transpose=True``: inputs are [B, 3, N] unless told otherwise
+    (torkit3d/ops/ball_query.py:17-38).
+
+    Returns:
+        index [B, N1, max_neighbors] int64: the first hits in key order, padded with
+        the first hit; all -1 where nothing lies within the radius.
+    """
+    if transpose:
+        query, key = query.transpose(1, 2), key.transpose(1, 2)
+    query, key = query.contiguous(), key.contiguous()
+    return BallQueryFunction.apply(query, key, radius, max_neighbors)
