@@ -1,0 +1,150 @@
+"""Group points and feature interpolation on the GPU. Forward results are
+bit-identical to the oracle; backward within 1e-5 relative / 1e-6 absolute per
+contribution (float atomics sum in a different order, as in the reference)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def scatter_atol(counts_max):
+    # 1e-6 per summed term
+    return 1e-6 * max(8, counts_max)
+
+
+@pytest.mark.parametrize("b,c,n1,n2,k", [(2, 3, 512, 128, 32), (5, 64, 513, 129, 33),
+                                          (32, 32, 1024, 512, 64), (16, 3, 8192, 2048, 32)])
+def test_group_reference_cases(cuda, b, c, n1, n2, k):
+    # tests/ops/test_group_points.py:15-45: fp32, torch.gather oracle, ones upstream
+    from torkit3d_amd.ops.group_points import group_points
+
+    torch.manual_seed(0)
+    feat = torch.randn(b, c, n1).to(cuda).requires_grad_()
+    index = torch.randint(0, n1, (b, n2, k)).to(cuda)
+    want = feat.unsqueeze(2).expand(b, c, n2, n1).gather(3, index.unsqueeze(1).expand(b, c, n2, k))
+    got = group_points(feat, index)
+    assert torch.equal(got, want)
+    got.backward(torch.ones_like(got))
+    mine = feat.grad.clone()
+    feat.grad = None
+    want.backward(torch.ones_like(want))
+    torch.testing.assert_close(mine, feat.grad, rtol=RTOL, atol=1e-6)
+
+
+def test_group_config_fp32(cuda):
+    # benchmark config 3: features (16,64,4096) gathered to (16,64,1024,32)
+    from torkit3d_amd import _C
+
+    g = gen(3)
+    feat = torch.randn(16, 64, 4096, generator=g)
+    index = torch.randint(0, 4096, (16, 1024, 32), generator=g)
+    out = _C.group_points_forward_cuda(feat.to(cuda), index.to(cuda))
+    np.testing.assert_array_equal(out.cpu().numpy(), oracle.group_forward(feat.numpy(), index.numpy()))
+    go = torch.randn(16, 64, 1024, 32, generator=g)
+    gin = _C.group_points_backward_cuda(go.to(cuda), index.to(cuda), 4096)
+    np.testing.assert_allclose(gin.cpu().numpy(), oracle.group_backward(go.numpy(), index.numpy(), 4096),
+                               rtol=RTOL, atol=scatter_atol(32))
+
+
+@pytest.mark.parametrize("b,c,n1,n2,k,dtype", [
+    (8, 32, 16384, 4096, 32, torch.float32),   # config 5 level 1: a 64 KiB row per channel
+    (2, 4, 20000, 300, 8, torch.float32),      # rows too long for LDS: global atomics
+    (1, 3, 700, 1000, 16, torch.float32),      # few rows: the point range is split
+    (2, 5, 100, 7, 3, torch.float64), (3, 2, 9000, 50, 5, torch.float64),
+    (1, 1, 1, 1, 1, torch.float32), (2, 3, 10, 0, 4, torch.float32)])
+def test_group_shapes_and_paths(cuda, b, c, n1, n2, k, dtype):
+    from torkit3d_amd import _C
+
+    g = gen(n1)
+    feat = torch.randn(b, c, n1, generator=g, dtype=dtype)
+    index = torch.randint(0, n1, (b, n2, k), generator=g)
+    out = _C.group_points_forward_cuda(feat.to(cuda), index.to(cuda))
+    np.testing.assert_array_equal(out.cpu().numpy(), oracle.group_forward(feat.numpy(), index.numpy()))
+    go = torch.randn(b, c, n2, k, generator=g, dtype=dtype)
+    gin = _C.group_points_backward_cuda(go.to(cuda), index.to(cuda), n1)
+    tol = dict(rtol=RTOL, atol=scatter_atol(64)) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gin.cpu().numpy(), oracle.group_backward(go.numpy(), index.numpy(), n1), **tol)
+
+
+def test_group_non_contiguous_inputs_and_out_of_range(cuda):
+    from torkit3d_amd import _C
+
+    g = gen(1)
+    feat = torch.randn(2, 40, 6, generator=g).to(cuda).transpose(1, 2)  # [2,6,40] strided
+    index = torch.randint(0, 40, (2, 5, 3), generator=g).to(cuda)
+    out = _C.group_points_forward_cuda(feat, index)
+    np.testing.assert_array_equal(out.cpu().numpy(),
+                                  oracle.group_forward(feat.contiguous().cpu().numpy(), index.cpu().numpy()))
+    # ball_query marks rows without a hit with -1: those gather 0 instead of faulting
+    index[0, 0, :] = -1
+    index[1, 1, 0] = 40
+    out = _C.group_points_forward_cuda(feat, index)
+    assert float(out[0, :, 0, :].abs().max()) == 0 and float(out[1, :, 1, 0].abs().max()) == 0
+
+
+@pytest.mark.parametrize("b,c,n1,n2", [(2, 64, 128, 512), (3, 65, 129, 513), (32, 64, 256, 1024),
+                                        (32, 64, 2048, 8192)])
+def test_interpolate_reference_cases_fp64(cuda, b, c, n1, n2):
+    # tests/ops/test_interpolate_feature.py:25-67: fp64, k=3, gather*weight oracle
+    from torkit3d_amd.ops.interpolate_feature import interpolate_feature
+
+    torch.manual_seed(0)
+    feat = torch.randn(b, c, n1, dtype=torch.float64).to(cuda).requires_grad_()
+    index = torch.randint(0, n1, (b, n2, 3)).to(cuda)
+    weight = torch.rand(b, n2, 3, dtype=torch.float64).to(cuda)
+    weight = weight / weight.sum(2, keepdim=True)
+    grouped = feat.unsqueeze(2).expand(b, c, n2, n1).gather(3, index.unsqueeze(1).expand(b, c, n2, 3))
+    want = (grouped * weight.unsqueeze(1)).sum(-1)
+    got = interpolate_feature(feat, index, weight)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-13)
+    go = torch.randn(b, c, n2, dtype=torch.float64, device=cuda)
+    got.backward(go)
+    mine = feat.grad.clone()
+    feat.grad = None
+    want.backward(go)
+    torch.testing.assert_close(mine, feat.grad, rtol=1e-11, atol=1e-12)
+
+
+def test_interpolation_config_fp32(cuda):
+    # benchmark config 4: knn(3) -> inverse squared distance weights -> interpolate
+    # features (32,128,2048) onto 8192 queries, forward and backward
+    from torkit3d_amd import _C
+    from torkit3d_amd.ops.interpolate_feature import three_nn_weights
+    from util import uniform_cloud
+
+    g = gen(4)
+    q, key = uniform_cloud(g, 32, 8192), uniform_cloud(g, 32, 2048)
+    feat = torch.randn(32, 128, 2048, generator=g)
+    d2, idx = _C.knn_distance_cuda(q.to(cuda), key.to(cuda), 3, 1)
+    w = three_nn_weights(d2)
+    od2, oidx = oracle.knn(q.numpy(), key.numpy(), 3)
+    ow = oracle.three_nn_weights(od2)
+    np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+    np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=RTOL, atol=1e-6)
+    out = _C.interpolate_forward_cuda(feat.to(cuda), idx, w)
+    want = oracle.interpolate_forward(feat.numpy(), idx.cpu().numpy(), w.cpu().numpy())
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    go = torch.randn(32, 128, 8192, generator=g)
+    gin = _C.interpolate_backward_cuda(go.to(cuda), idx, w, 2048)
+    ogin = oracle.interpolate_backward(go.numpy(), idx.cpu().numpy(), w.cpu().numpy(), 2048)
+    np.testing.assert_allclose(gin.cpu().numpy(), ogin, rtol=RTOL, atol=scatter_atol(32))
+
+
+def test_interpolate_only_k3_through_the_reference_interface(cuda):
+    from torkit3d_amd import _C
+
+    feat = torch.zeros(1, 2, 5, device=cuda)
+    idx = torch.zeros(1, 4, 2, dtype=torch.int64, device=cuda)
+    w = torch.zeros(1, 4, 2, device=cuda)
+    with pytest.raises(RuntimeError):
+        _C.interpolate_forward_cuda(feat, idx, w)
+    with pytest.raises(RuntimeError, match="Only support k=3"):
+        _C.interpolate_backward_cuda(torch.zeros(1, 2, 4, device=cuda), idx, w, 5)

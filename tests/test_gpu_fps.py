@@ -1,0 +1,109 @@
+"""Farthest point sampling on the GPU: indices bit-identical to the oracle (which
+replays the reference kernel's threads, including its tie order)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import fps_numpy, gaussian_mixture_cloud, lattice_cloud
+
+pytestmark = pytest.mark.gpu
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def run(points, k, cuda, transpose=False):
+    from torkit3d_amd.ops.sample_farthest_points import sample_farthest_points
+
+    return sample_farthest_points(points.to(cuda), k, transpose=transpose).cpu().numpy()
+
+
+@pytest.mark.parametrize("b,n,k,transpose", [(1, 31, 2, True), (2, 1024, 128, True),
+                                              (3, 1025, 129, False), (3, 1025, 129, True),
+                                              (16, 1024, 512, False), (32, 1024, 512, True),
+                                              (32, 8192, 2048, False)])
+def test_reference_cases_fp64(cuda, b, n, k, transpose):
+    # tests/ops/test_sample_farthest_points.py:41-62: fp64 uniform points vs numpy
+    np.random.seed(0)
+    pts = np.random.rand(b, n, 3)
+    want = oracle.sample_farthest_points(pts, k)
+    if b * n * k <= 3 * 1025 * 129:
+        np.testing.assert_array_equal(want, fps_numpy(pts, k))
+    t = torch.from_numpy(pts)
+    if transpose:
+        t = t.transpose(1, 2).contiguous()
+    np.testing.assert_array_equal(run(t, k, cuda, transpose), want)
+
+
+def test_sampling_config_fp32(cuda):
+    # benchmark config 2: B=16, N=4096 from a mixture of 8 Gaussians, 1024 samples
+    pts = gaussian_mixture_cloud(gen(2), 16, 4096)
+    got = run(pts, 1024, cuda)
+    np.testing.assert_array_equal(got, oracle.sample_farthest_points(pts.numpy(), 1024))
+    assert (got[:, 0] == 0).all()
+    assert all(len(set(row)) == 1024 for row in got)
+
+
+def test_set_abstraction_chain_fp32(cuda):
+    # benchmark config 5: B=8, 16384 -> 4096 -> 1024 -> 256, each level on the previous picks
+    from torkit3d_amd import _C
+
+    g = gen(5)
+    xyz = torch.rand(8, 16384, 3, generator=g)
+    cur_gpu, cur_cpu = xyz.to(cuda), xyz.numpy()
+    for k in (4096, 1024, 256):
+        got = _C.sample_farthest_points_cuda(cur_gpu, k)
+        want = oracle.sample_farthest_points(cur_cpu, k)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+        cur_gpu = torch.gather(cur_gpu, 1, got[:, :, None].expand(-1, -1, 3)).contiguous()
+        cur_cpu = np.take_along_axis(cur_cpu, want[:, :, None], 1)
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 33, 64, 65, 255, 257, 511, 513, 1000, 2049, 4097,
+                                8191, 12000, 16384])
+def test_every_launch_shape_fp32(cuda, n):
+    pts = torch.rand(2, n, 3, generator=gen(n))
+    k = min(n, 70)
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
+
+
+@pytest.mark.parametrize("n,dtype", [(16385, torch.float32), (20000, torch.float32),
+                                      (8193, torch.float64)])
+def test_workspace_path_for_large_clouds(cuda, n, dtype):
+    pts = torch.rand(2, n, 3, generator=gen(n), dtype=dtype)
+    np.testing.assert_array_equal(run(pts, 40, cuda), oracle.sample_farthest_points(pts.numpy(), 40))
+
+
+@pytest.mark.parametrize("n", [64, 70, 600, 3000, 17000])
+def test_ties_follow_the_reference_tree_order(cuda, n):
+    # lattice clouds tie for the maximum all the time; the oracle replays the reference's
+    # per-thread scan and tree, which is not lowest-index order
+    pts = lattice_cloud(gen(n), 3, n, 2)
+    k = min(n, 60)
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    np.testing.assert_array_equal(run(pts, k, cuda), want)
+    if n == 600:
+        assert not np.array_equal(want, oracle.sample_farthest_points(pts.numpy(), k, "lowest"))
+
+
+def test_duplicates_and_full_sample(cuda):
+    ones = torch.ones(2, 500, 3)
+    np.testing.assert_array_equal(run(ones, 20, cuda), np.zeros((2, 20), np.int64))
+    pts = torch.rand(2, 700, 3, generator=gen(1))
+    got = run(pts, 700, cuda)
+    np.testing.assert_array_equal(np.sort(got, axis=1), np.tile(np.arange(700), (2, 1)))
+    np.testing.assert_array_equal(got, oracle.sample_farthest_points(pts.numpy(), 700))
+
+
+def test_errors(cuda):
+    from torkit3d_amd import _C
+
+    pts = torch.zeros(2, 8, 3, device=cuda)
+    with pytest.raises(RuntimeError):
+        _C.sample_farthest_points_cuda(pts, 0)
+    with pytest.raises(RuntimeError):
+        _C.sample_farthest_points_cuda(pts, 9)
+    with pytest.raises(RuntimeError):
+        _C.sample_farthest_points_cuda(torch.zeros(2, 8, 4, device=cuda), 2)

@@ -1,0 +1,98 @@
+"""K nearest neighbours on the GPU: bit-identical (distances, indices, slot order)
+to the oracle's MinK restatement; the reference's own checks against cdist/topk."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import lattice_cloud, uniform_cloud
+
+pytestmark = pytest.mark.gpu
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def check_raw(q, key, k, cuda, version=1):
+    from torkit3d_amd import _C
+
+    d, i = _C.knn_distance_cuda(q.to(cuda), key.to(cuda), k, version)
+    od, oi = oracle.knn(q.numpy(), key.numpy(), k)
+    np.testing.assert_array_equal(d.cpu().numpy(), od)
+    np.testing.assert_array_equal(i.cpu().numpy(), oi)
+
+
+@pytest.mark.parametrize("b,n1,n2,k,transpose", [(1, 512, 1024, 3, True), (2, 512, 1024, 32, False),
+                                                  (3, 511, 1025, 31, True),
+                                                  (32, 2048, 8192, 64, False)])
+def test_reference_cases_fp64(cuda, b, n1, n2, k, transpose):
+    # tests/ops/test_knn_distance.py:6-32: fp64 randn, compared with cdist + topk as
+    # sqrt distances (atol 5e-5, rtol 1e-4) and exact sorted indices.
+    from torkit3d_amd.ops.knn_points import knn_points
+    from torkit3d_amd.ops.native import knn
+
+    torch.manual_seed(0)
+    q = torch.randn(b, n1, 3, dtype=torch.float64)
+    key = torch.randn(b, n2, 3, dtype=torch.float64)
+    if transpose:
+        q, key = q.transpose(1, 2), key.transpose(1, 2)
+    qd, kd = q.to(cuda), key.to(cuda)
+    want_d, want_i = knn(qd, kd, k, sorted=True, transpose=transpose)
+    got_d, got_i = knn_points(qd, kd, k, sorted=True, sqrt_distance=True, transpose=transpose)
+    torch.testing.assert_close(got_d, want_d, atol=5e-5, rtol=1e-4)
+    assert torch.equal(got_i, want_i)
+    if b <= 3:
+        qc = (q.transpose(1, 2) if transpose else q).contiguous()
+        kc = (key.transpose(1, 2) if transpose else key).contiguous()
+        check_raw(qc, kc, k, cuda)
+
+
+@pytest.mark.parametrize("k", [16, 3])
+def test_interpolation_config_fp32(cuda, k):
+    # benchmark config 4: B=32, N=8192 queries, M=2048 keys, uniform in [-1,1]^3
+    g = gen(4)
+    q, key = uniform_cloud(g, 32, 8192), uniform_cloud(g, 32, 2048)
+    check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("b,n1,n2,k", [(2, 300, 2048, 1), (2, 100, 500, 4), (2, 77, 130, 5),
+                                        (2, 100, 500, 8), (1, 200, 3000, 17), (2, 100, 500, 64),
+                                        (1, 50, 300, 100), (2, 33, 40, 40), (2, 10, 5, 5),
+                                        (1, 1000, 1025, 33)])
+def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
+    g = gen(k)
+    q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
+    check_raw(q, key, k, cuda, version=0)
+    check_raw(q, key, k, cuda, version=1)
+
+
+def test_lattice_ties_follow_mink_eviction_order(cuda):
+    g = gen(9)
+    q, key = lattice_cloud(g, 2, 400, 4), lattice_cloud(g, 2, 1500, 4)
+    for k in (3, 6, 16, 33):
+        check_raw(q, key, k, cuda)
+
+
+def test_k1_equals_chamfer_argmin(cuda):
+    from torkit3d_amd import _C
+
+    g = gen(10)
+    q, key = uniform_cloud(g, 2, 2000).to(cuda), uniform_cloud(g, 2, 1500).to(cuda)
+    d, i = _C.knn_distance_cuda(q, key, 1, 1)
+    cd, ci, _, _ = _C.chamfer_distance_forward_cuda(q, key)
+    assert torch.equal(d[..., 0], cd) and torch.equal(i[..., 0], ci)
+
+
+def test_errors(cuda):
+    from torkit3d_amd import _C
+
+    q = torch.zeros(2, 8, 3, device=cuda)
+    with pytest.raises(RuntimeError):
+        _C.knn_distance_cuda(q, q, 9, 1)  # k > N2 (knn_distance_kernel.cu:199)
+    with pytest.raises(RuntimeError, match="Invalid version"):
+        _C.knn_distance_cuda(q, q, 2, 3)
+    with pytest.raises(RuntimeError):
+        _C.knn_distance_cuda(q, torch.zeros(3, 8, 3, device=cuda), 2, 1)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        _C.knn_distance_cuda(q.transpose(0, 1), q, 2, 1)
