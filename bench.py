@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the point-cloud hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one chamfer / nearest-neighbour forward pass (both directions, one
+kernel launch) over the stress configuration B=32, N=M=16384 with the inputs
+already resident in HBM. The headline value is pair-distances per second,
+2*B*N*M / t_step. The run also reports, on the same JSON line:
+
+  roofline      the chamfer forward kernel against the fp32 vector peak, from the
+                8 algorithmic FLOP per pair-distance and the launch duration
+                measured with events on the launching stream;
+  cpu_baseline  the CPU oracle (OpenMP C restatement of the reference algorithm)
+                timed on this box's host cores on a bounded sample of the same
+                workload;
+  secondary     milliseconds for farthest point sampling, ball query, group
+                points (B=16, N=4096) and the KNN / interpolation configuration.
+
+Everything runs on one GPU; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+FP32_VECTOR_PEAK_TFLOPS = 157.3   # MI355X: 256 CU x 256 FLOP/clk x 2.4 GHz
+HBM_PEAK_GBS = 8000.0
+FLOP_PER_PAIR = 8                 # 3 sub, 3 mul, 2 add
+
+# HBM bytes per chamfer-forward launch at B=32, N=M=16384, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
+# (profiles/chamfer_forward_B32_N16384.md).
+CHAMFER_TRAFFIC_BYTES = 194.9e6
+
+
+def sphere_cloud(gen, b, n, noise=0.01):
+    import torch
+
+    u = torch.randn(b, n, 3, generator=gen)
+    return u / u.norm(dim=2, keepdim=True) + noise * torch.randn(b, n, 3, generator=gen)
+
+
+def gpu_time_ms(fn, steps, warmup):
+    """Average milliseconds per call, from events on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def cpu_baseline_chamfer(a, c, budget_s=12.0):
+    """Time the oracle on a slice of the batch sized to about `budget_s` seconds."""
+    import oracle
+
+    n = a.shape[1]
+    t0 = time.perf_counter()
+    oracle.chamfer_forward(a[:1].numpy(), c[:1].numpy())
+    probe = time.perf_counter() - t0
+    nb = int(max(1, min(a.shape[0], budget_s / max(probe, 1e-3))))
+    t0 = time.perf_counter()
+    oracle.chamfer_forward(a[:nb].numpy(), c[:nb].numpy())
+    dt = time.perf_counter() - t0
+    pairs = 2.0 * nb * n * c.shape[1]
+    return {
+        "value": pairs / dt,
+        "unit": "pair-dists/s",
+        "cores": oracle.num_threads(),
+        "kind": "port",
+        "sample": "oracle chamfer forward on the first %d of %d clouds (N=M=%d), %.2f s" % (
+            nb, a.shape[0], n, dt),
+    }
+
+
+def secondary_metrics(dev, steps, warmup):
+    """ms per call for the other ops at their benchmark shapes (events, same stream)."""
+    import torch
+
+    from torkit3d_amd import _C
+    from torkit3d_amd.ops.interpolate_feature import three_nn_weights
+
+    out = {}
+    g = torch.Generator().manual_seed(2)
+    centres = torch.rand(16, 8, 3, generator=g) * 2 - 1
+    comp = torch.randint(0, 8, (16, 4096), generator=g)
+    pts = (torch.gather(centres, 1, comp[:, :, None].expand(-1, -1, 3))
+           + 0.1 * torch.randn(16, 4096, 3, generator=g)).to(dev)
+    out["fps_B16_N4096_K1024_ms"] = gpu_time_ms(
+        lambda: _C.sample_farthest_points_cuda(pts, 1024), steps, warmup)
+
+    g = torch.Generator().manual_seed(3)
+    xyz = torch.rand(16, 4096, 3, generator=g).to(dev)
+    fidx = _C.sample_farthest_points_cuda(xyz, 1024)
+    ctr = torch.gather(xyz, 1, fidx[:, :, None].expand(-1, -1, 3)).contiguous()
+    out["ball_query_B16_N1024x4096_r0.2_k32_ms"] = gpu_time_ms(
+        lambda: _C.ball_query_cuda(ctr, xyz, 0.2, 32), steps, warmup)
+    nbr = _C.ball_query_cuda(ctr, xyz, 0.2, 32)
+    feat = torch.randn(16, 64, 4096, generator=g).to(dev)
+    out["group_fwd_B16_C64_N4096_to_1024x32_ms"] = gpu_time_ms(
+        lambda: _C.group_points_forward_cuda(feat, nbr), steps, warmup)
+    go = torch.randn(16, 64, 1024, 32, generator=g).to(dev)
+    out["group_bwd_ms"] = gpu_time_ms(
+        lambda: _C.group_points_backward_cuda(go, nbr, 4096), steps, warmup)
+
+    g = torch.Generator().manual_seed(4)
+    q = (torch.rand(32, 8192, 3, generator=g) * 2 - 1).to(dev)
+    key = (torch.rand(32, 2048, 3, generator=g) * 2 - 1).to(dev)
+    out["knn_B32_N8192_M2048_k16_ms"] = gpu_time_ms(
+        lambda: _C.knn_distance_cuda(q, key, 16, 1), steps, warmup)
+    out["knn_B32_N8192_M2048_k3_ms"] = gpu_time_ms(
+        lambda: _C.knn_distance_cuda(q, key, 3, 1), steps, warmup)
+    d2, kidx = _C.knn_distance_cuda(q, key, 3, 1)
+    w = three_nn_weights(d2)
+    f4 = torch.randn(32, 128, 2048, generator=g).to(dev)
+    out["interpolate_fwd_B32_C128_ms"] = gpu_time_ms(
+        lambda: _C.interpolate_forward_cuda(f4, kidx, w), steps, warmup)
+    g4 = torch.randn(32, 128, 8192, generator=g).to(dev)
+    out["interpolate_bwd_ms"] = gpu_time_ms(
+        lambda: _C.interpolate_backward_cuda(g4, kidx, w, 2048), steps, warmup)
+    return {k: round(v, 5) for k, v in out.items()}
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="skip the CPU oracle timing (for profiler runs)")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="time only the chamfer step (for profiler runs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy, whose known traffic "
+                         "scales the profiler's FETCH_SIZE / WRITE_SIZE counters")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU; every op is independent across the "
+                 "batch, so more GPUs only shard B. Run with --gpus 1.")
+
+    import torch
+
+    from torkit3d_amd import _C, _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    _lib.lib()  # fail loudly if the HIP library is missing
+    dev = "cuda:0"
+    B, N, M = 32, 16384, 16384
+    gen = torch.Generator().manual_seed(5)
+    a_cpu, c_cpu = sphere_cloud(gen, B, N), sphere_cloud(gen, B, M)
+    a, c = a_cpu.to(dev), c_cpu.to(dev)
+
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    def step():
+        return _C.chamfer_distance_forward_cuda(a, c)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        out = step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = start.elapsed_time(stop) / args.steps  # one launch per step
+
+    pairs = 2.0 * B * N * M
+    value = pairs / (wall_ms * 1e-3)
+    achieved_tflops = pairs * FLOP_PER_PAIR / (kernel_ms * 1e-3) / 1e12
+
+    # cheap self-check so that a wrong kernel cannot post a number: every reported
+    # distance must be the distance to the reported index
+    d1, i1, d2, i2 = out
+    near = torch.gather(c, 1, i1[:, :, None].expand(-1, -1, 3))
+    if not torch.allclose(((a - near) ** 2).sum(-1), d1, rtol=1e-4, atol=1e-6):
+        sys.exit("bench.py: chamfer output failed its self-check")
+
+    line = {
+        "metric": "chamfer pair-dists/s at B=32,N=M=16384",
+        "value": value,
+        "unit": "pair-dists/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "chamfer forward (both directions), B=32, N=M=16384 fp32 points "
+                               "on unit spheres + N(0,0.01) noise (stress configuration)",
+                   "B": B, "N": N, "M": M},
+        "roofline": {
+            "bound": "valu_fp32",
+            "achieved": achieved_tflops,
+            "peak": FP32_VECTOR_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tflops / FP32_VECTOR_PEAK_TFLOPS,
+            "traffic": CHAMFER_TRAFFIC_BYTES,
+            "kernel": "chamfer_forward_kernel",
+            "kernel_ms": kernel_ms,
+            "flop_per_pair": FLOP_PER_PAIR,
+        },
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_chamfer(a_cpu, c_cpu)
+    if not args.no_secondary:
+        line["secondary"] = secondary_metrics(dev, max(5, args.steps // 2), args.warmup)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
