@@ -56,7 +56,15 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
     __shared__ T skey[STAGE * 4];
 
     const int tid = threadIdx.x;
+    // Workgroups are handed to the 8 XCDs round-robin by blockIdx. Remap so that each
+    // XCD works on a contiguous range of logical workgroups: the workgroups that
+    // sweep the same key cloud then share one L2 instead of fetching it 8 times.
     int lb = blockIdx.x;
+    {
+        const int nb = gridDim.x, per = nb >> 3, full = per << 3;
+        if (lb < full)
+            lb = (lb & 7) * per + (lb >> 3);
+    }
     const int which = lb >= args.nblocks0;
     if (which)
         lb -= args.nblocks0;
@@ -225,12 +233,11 @@ __global__ __launch_bounds__(256) void chamfer_backward_scatter_kernel(
     }
 }
 
-template <typename T, int QPL>
+template <typename T, int QPL, int BLOCK = 256, int TILE = 32, int STAGE = 1024>
 int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
                            int64_t N2, T *dist1, int64_t *idx1, T *dist2,
                            int64_t *idx2, hipStream_t stream)
 {
-    constexpr int BLOCK = 256, TILE = 32, STAGE = 1024;
     constexpr int QB = QPL * BLOCK;
     ChamferFwdArgs<T> a;
     a.dir[0] = {xyz1, xyz2, dist1, idx1, (int)N1, (int)N2, (int)((N1 + QB - 1) / QB)};
@@ -267,8 +274,8 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
     if (sizeof(T) == 8 || work < (int64_t)256 * 1024)
         return chamfer_forward_launch<T, 2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                             idx2, s);
-    return chamfer_forward_launch<T, 4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
-                                        s);
+    return chamfer_forward_launch<T, 4, 512, 64>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+                                                 idx2, s);
 }
 
 template <typename T>

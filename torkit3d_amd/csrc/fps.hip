@@ -188,6 +188,165 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
     }
 }
 
+// ---- fp32 fast path ------------------------------------------------------------
+// Same algorithm as fps_register_kernel, tuned for the serial step:
+//   * running minima are kept as the bit patterns of non-negative floats, which
+//     order like signed integers; integer min/max need no NaN canonicalisation
+//     and the -1.0f marker of unused slots (a negative integer) stays put;
+//   * a lane reduces its P minima through a binary tree of maxima kept in
+//     registers; the wave reduction is six v_max_i32 with DPP operands, written
+//     out because the compiler does not fold the lane moves into the max;
+//   * the winning lane comes from one ballot + scalar find-first; its winning
+//     point is found by walking the winner lane's tree with v_readlane and
+//     scalar branches (left child first = lowest position), and the leaf reached
+//     reads that point's coordinates from fixed registers - log2(P) steps, no
+//     per-point compares or select chains in the loop;
+//   * a wave publishes one 32-byte slot (value, point, xyz); after the single
+//     barrier every wave loads all slots at once and picks the winner with
+//     v_readlane, no second LDS round trip.
+__device__ __forceinline__ int wave_max_i32(int v)
+{
+    // VALU write -> DPP read of the same register needs two wait states (s_nop 1).
+    asm volatile("s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+                 "s_nop 1"
+                 : "+v"(v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
+struct __align__(16) FpsSlot {
+    int val;  // bit pattern of the wave's maximum
+    int j;    // point index of the wave's candidate
+    float x, y, z;
+    int pad[3];
+};
+
+struct FpsPick {
+    float x, y, z;
+    int j;
+};
+
+// Walks the tree of lane `wl` from NODE down to the first leaf equal to `wmax`.
+// t[1] is the root, t[2i] / t[2i+1] the children of t[i], t[P + p] the minimum of
+// point p. Every register index is a compile-time constant; the direction taken
+// at each node is wave-uniform, so the walk is scalar branches.
+template <int P, int NODE> struct FpsWalk {
+    static __device__ __forceinline__ void go(const int (&t)[2 * P], const float (&x)[P],
+                                              const float (&y)[P], const float (&z)[P],
+                                              const int (&jv)[P], int wl, int wmax,
+                                              FpsPick &out)
+    {
+        if constexpr (NODE >= P) {
+            constexpr int p = NODE - P;
+            out.x = read_lane(x[p], wl);
+            out.y = read_lane(y[p], wl);
+            out.z = read_lane(z[p], wl);
+            out.j = read_lane(jv[p], wl);
+            // Keeps each leaf a block of its own (no flattening into selects).
+            asm volatile("" ::"s"(out.j));
+        } else {
+            const int left = read_lane(t[2 * NODE], wl);
+            if (left == wmax)
+                FpsWalk<P, 2 * NODE>::go(t, x, y, z, jv, wl, wmax, out);
+            else
+                FpsWalk<P, 2 * NODE + 1>::go(t, x, y, z, jv, wl, wmax, out);
+        }
+    }
+};
+
+template <int P, int NT>
+__global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__restrict__ points,
+                                                              int64_t *__restrict__ index,
+                                                              FpsLayout L)
+{
+    static_assert((P & (P - 1)) == 0, "P must be a power of two");
+    constexpr int NW = NT / TK_WAVE;
+    constexpr int F32_INF = 0x7f800000;
+    constexpr int F32_NEG1 = (int)0xbf800000;
+    __shared__ FpsSlot slots[2][NW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const float *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
+    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
+
+    float x[P], y[P], z[P];
+    int jv[P];
+    int t[2 * P];  // t[P + p]: running minimum of point p (bits); t[1..P-1]: maxima
+    const int npos = L.bs * L.c;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int pos = tid * P + p;
+        const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
+        const bool ok = j < L.n;
+        x[p] = ok ? pts[(int64_t)j * 3 + 0] : 0.0f;
+        y[p] = ok ? pts[(int64_t)j * 3 + 1] : 0.0f;
+        z[p] = ok ? pts[(int64_t)j * 3 + 2] : 0.0f;
+        jv[p] = j;
+        t[P + p] = ok ? F32_INF : F32_NEG1;
+    }
+    t[0] = 0;
+
+    int sel_j = 0;
+    float cx = pts[0], cy = pts[1], cz = pts[2];
+    if (tid == 0)
+        out[0] = 0;
+
+    for (int it = 1; it < L.k; ++it) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const float d = tk_dist2<float>(x[p], y[p], z[p], cx, cy, cz);
+            const int db = __builtin_bit_cast(int, d);
+            t[P + p] = t[P + p] < db ? t[P + p] : db;
+        }
+#pragma unroll
+        for (int i = P - 1; i >= 1; --i)
+            t[i] = t[2 * i] > t[2 * i + 1] ? t[2 * i] : t[2 * i + 1];
+        // Only points strictly above zero are candidates (the reference starts its
+        // scan from max_dist = 0 with strict '>').
+        const int best = t[1] > 0 ? t[1] : 0;
+        const int wmax = wave_max_i32(best);
+        const int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
+        FpsPick pick;
+        FpsWalk<P, 1>::go(t, x, y, z, jv, wl, wmax, pick);
+        const int buf = it & 1;
+        if (lane == 0) {
+            FpsSlot s;
+            s.val = wmax;
+            s.j = pick.j;
+            s.x = pick.x;
+            s.y = pick.y;
+            s.z = pick.z;
+            s.pad[0] = s.pad[1] = s.pad[2] = 0;
+            slots[buf][wave] = s;
+        }
+        __syncthreads();
+        const FpsSlot mine = slots[buf][lane < NW ? lane : 0];
+        const int cv = lane < NW ? mine.val : F32_NEG1;
+        const int gmax = wave_max_i32(cv);
+        if (gmax > 0) {  // wave-uniform
+            const int gl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(cv == gmax));
+            sel_j = read_lane(mine.j, gl);
+            cx = read_lane(mine.x, gl);
+            cy = read_lane(mine.y, gl);
+            cz = read_lane(mine.z, gl);
+        }
+        if (tid == 0)
+            out[it] = (int64_t)sel_j;
+    }
+}
+
 // Clouds that do not fit in registers: minimum distances live in a global
 // workspace, coordinates are re-read every step (they stay in L2). Same selection
 // rule; positions are visited in priority order so the tie rule is unchanged.
@@ -294,6 +453,36 @@ void fps_launch(const T *points, int64_t B, int64_t *index, const FpsLayout &L,
                        points, index, L);
 }
 
+template <int P, int NT>
+void fps_launch_f32(const float *points, int64_t B, int64_t *index, const FpsLayout &L,
+                    hipStream_t s)
+{
+    hipLaunchKernelGGL((fps_register_kernel_f32<P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
+                       points, index, L);
+}
+
+// fp32: (points per lane, lanes) by cloud size, from timing every shape on an
+// MI355X: two waves per SIMD (512 lanes) hide each other's reduction latency; more
+// waves only repeat the per-wave reduction.
+void fps_dispatch_f32(const float *points, int64_t B, int64_t *index, const FpsLayout &L,
+                      int64_t npos, hipStream_t s)
+{
+    if (npos <= 64 * 2)
+        fps_launch_f32<2, 64>(points, B, index, L, s);
+    else if (npos <= 256 * 2)
+        fps_launch_f32<2, 256>(points, B, index, L, s);
+    else if (npos <= 512 * 2)
+        fps_launch_f32<2, 512>(points, B, index, L, s);
+    else if (npos <= 512 * 4)
+        fps_launch_f32<4, 512>(points, B, index, L, s);
+    else if (npos <= 512 * 8)
+        fps_launch_f32<8, 512>(points, B, index, L, s);
+    else if (npos <= 512 * 16)
+        fps_launch_f32<16, 512>(points, B, index, L, s);
+    else
+        fps_launch_f32<32, 512>(points, B, index, L, s);
+}
+
 template <typename T>
 int fps(const T *points, int64_t B, int64_t N, int64_t K, int64_t *index, void *workspace,
         size_t workspace_bytes, void *stream)
@@ -312,6 +501,10 @@ int fps(const T *points, int64_t B, int64_t N, int64_t K, int64_t *index, void *
     const FpsLayout L = fps_layout(N, K);
     const int64_t npos = (int64_t)L.bs * L.c;
     if (npos <= fps_register_capacity(sizeof(T))) {
+        if constexpr (sizeof(T) == 4) {
+            fps_dispatch_f32(points, B, index, L, npos, s);
+            return tk_launch_status();
+        }
         // Fewest points per lane that still covers the cloud: short serial chains.
         if (npos <= 256 * 1)
             fps_launch<T, 1, 256>(points, B, index, L, s);
