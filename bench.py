@@ -136,8 +136,8 @@ def secondary_metrics(dev, steps, warmup):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the CPU oracle timing (for profiler runs)")
     ap.add_argument("--no-secondary", action="store_true",
@@ -220,7 +220,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved_tflops / FP32_VECTOR_PEAK_TFLOPS,
             "traffic": CHAMFER_TRAFFIC_BYTES,
-            "kernel": "chamfer_forward_kernel",
+            "kernel": "chamfer_forward_filter_kernel",
             "kernel_ms": kernel_ms,
             "flop_per_pair": FLOP_PER_PAIR,
         },

@@ -150,3 +150,63 @@ def test_sqrt_option(cuda):
     s1, s2 = chamfer_distance(a, c, sqrt=True)
     assert torch.equal(s1, torch.sqrt(torch.clamp(d1, 1e-12)))
     assert torch.equal(s2, torch.sqrt(torch.clamp(d2, 1e-12)))
+
+
+# ---- inputs chosen against the pre-filtered fp32 kernel ------------------------------
+# Large fp32 clouds go through a kernel that rules pairs out with a cheaper score and
+# re-evaluates only candidate tiles exactly. Whatever the input, the result must be
+# bit-identical to the oracle: these cases aim at its error bound, its candidate
+# bookkeeping and its fallbacks.
+
+def _clouds(kind, g):
+    b, n1, n2 = 2, 1500, 3001
+    if kind == "lattice":            # exact ties everywhere: many candidate tiles
+        return lattice_cloud(g, b, 2048, 4), lattice_cloud(g, b, 2048, 4)
+    if kind == "coarse_lattice":     # 27 distinct positions: every tile ties
+        return lattice_cloud(g, b, 1100, 2), lattice_cloud(g, b, 1300, 2)
+    if kind == "duplicates":
+        return uniform_cloud(g, b, n1), uniform_cloud(g, b, 1).expand(b, n2, 3).contiguous()
+    if kind == "far_from_origin":    # magnitude >> spacing: the bound is loose
+        return uniform_cloud(g, b, n1) + 1000.0, uniform_cloud(g, b, n2) + 1000.0
+    if kind == "separated":          # queries far from every key
+        return uniform_cloud(g, b, n1) + 50.0, uniform_cloud(g, b, n2)
+    if kind == "wide_range":
+        return (uniform_cloud(g, b, n1) * 1e6, uniform_cloud(g, b, n2) * 1e6)
+    if kind == "tiny":               # squares underflow
+        return uniform_cloud(g, b, n1) * 1e-20, uniform_cloud(g, b, n2) * 1e-20
+    if kind == "huge":               # squares overflow the bound's range
+        return uniform_cloud(g, b, n1) * 1e18, uniform_cloud(g, b, n2) * 1e18
+    if kind == "overflowing":        # distances overflow to +inf
+        return uniform_cloud(g, b, n1) * 3e19, -uniform_cloud(g, b, n2).abs() * 3e19
+    if kind == "clusters":           # tight clusters far apart
+        centres = uniform_cloud(g, b, 8) * 100.0
+        def mk(n):
+            pick = torch.randint(0, 8, (b, n), generator=g)
+            base = torch.gather(centres, 1, pick[:, :, None].expand(-1, -1, 3))
+            return base + 1e-3 * uniform_cloud(g, b, n)
+        return mk(n1), mk(n2)
+    if kind == "nan_and_inf":
+        a, c = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
+        c[0, ::7, 1] = float("nan")
+        c[1, 5, 0] = float("inf")
+        a[0, 3, 2] = float("nan")
+        a[1, ::50] = float("inf")
+        return a, c
+    if kind == "all_nan_keys":
+        return uniform_cloud(g, b, n1), torch.full((b, n2, 3), float("nan"))
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["lattice", "coarse_lattice", "duplicates", "far_from_origin",
+                                  "separated", "wide_range", "tiny", "huge", "overflowing",
+                                  "clusters", "nan_and_inf", "all_nan_keys"])
+def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
+    a, c = _clouds(kind, gen(hash(kind) % 1000))
+    check_forward(a.contiguous(), c.contiguous(), cuda)
+
+
+@pytest.mark.parametrize("b,n1,n2", [(1, 1024, 1024), (2, 1025, 4097), (3, 8191, 1031),
+                                     (1, 20000, 1024), (64, 1024, 1100)])
+def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
+    g = gen(n1 + n2)
+    check_forward(sphere_cloud(g, b, n1), sphere_cloud(g, b, n2), cuda)

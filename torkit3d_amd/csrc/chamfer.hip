@@ -49,29 +49,36 @@ template <> __device__ __forceinline__ double chamfer_init_min<double>()
     return 1e40;
 }
 
-template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
-__global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T> args)
+// Decodes blockIdx into (direction, batch, query block). Workgroups are handed to
+// the 8 XCDs round-robin by blockIdx; the remap gives each XCD a contiguous range of
+// logical workgroups, so the workgroups that sweep the same key cloud share one L2
+// instead of fetching it 8 times.
+template <typename T>
+__device__ __forceinline__ const ChamferDir<T> &chamfer_decode_block(
+    const ChamferFwdArgs<T> &args, int &b, int &qblock)
 {
-    static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
-    __shared__ T skey[STAGE * 4];
-
-    const int tid = threadIdx.x;
-    // Workgroups are handed to the 8 XCDs round-robin by blockIdx. Remap so that each
-    // XCD works on a contiguous range of logical workgroups: the workgroups that
-    // sweep the same key cloud then share one L2 instead of fetching it 8 times.
     int lb = blockIdx.x;
-    {
-        const int nb = gridDim.x, per = nb >> 3, full = per << 3;
-        if (lb < full)
-            lb = (lb & 7) * per + (lb >> 3);
-    }
+    const int nb = gridDim.x, per = nb >> 3, full = per << 3;
+    if (lb < full)
+        lb = (lb & 7) * per + (lb >> 3);
     const int which = lb >= args.nblocks0;
     if (which)
         lb -= args.nblocks0;
     const ChamferDir<T> &d = args.dir[which];
+    b = lb / d.blocks_per_batch;
+    qblock = lb - b * d.blocks_per_batch;
+    return d;
+}
+
+// Exact sweep of one workgroup: QPL*BLOCK queries against the whole key cloud.
+// `skey` is STAGE*4 elements of LDS.
+template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
+__device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int b, int qblock,
+                                                    T *skey)
+{
+    static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
+    const int tid = threadIdx.x;
     const int nq = d.nq, nk = d.nk;
-    const int b = lb / d.blocks_per_batch;
-    const int qblock = lb - b * d.blocks_per_batch;
     const T *__restrict__ Q = d.query + (int64_t)b * nq * 3;
     const T *__restrict__ K = d.key + (int64_t)b * nk * 3;
 
@@ -157,6 +164,431 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
         }
         d.dist[(int64_t)b * nq + qi] = best[i];
         d.idx[(int64_t)b * nq + qi] = (int64_t)found;
+    }
+}
+
+template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
+__global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T> args)
+{
+    __shared__ T skey[STAGE * 4];
+    int b, qblock;
+    const ChamferDir<T> &d = chamfer_decode_block<T>(args, b, qblock);
+    chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+}
+
+// ---- fp32 forward with a bounded-error pre-filter -------------------------------
+//
+// The exact sweep spends 6.5 VALU instructions per pair. Most pairs only need to be
+// ruled out, which a cheaper score can do:
+//
+//     s(q,k) = |k'|^2 - 2 q'.k'   (k' = k - c, q' = q - c, c = centre of the key
+//                                  cloud's bounding box; three fused multiply-adds
+//                                  per pair, |k'|^2 staged with the key)
+//
+// d2(q,k) = s + |q'|^2 up to rounding. For one query the additive |q'|^2 is common to
+// all keys, so minima of s locate minima of d2 up to the rounding error of both
+// expressions. With u = 2^-24:
+//     |canonical d2 - true d2|  <= 5.01 u d2                (3 rounded differences,
+//                                                            1 product, 2 fmas)
+//     |s + |q'|^2 - true d2|    <= 8.1 u (|k'|+|q'|)^2      (centring 2 u, |k'|^2 3 u,
+//                                                            3 fmas 3 u)
+// hence |s + |q'|^2 - canonical d2| <= E = 13.2 u R, R = (max|k'| + |q'|)^2, and any
+// key whose canonical distance equals the minimum has s <= min(s) + 2E. The kernel
+// uses slack = 64 u R (> 2E plus the rounding of the comparison itself).
+//
+// Sweep: per tile of TILE keys only min(s) is formed (3 fma + half a min3 per
+// pair), and each query keeps the three smallest tile minima v0<=v1<=v2 with the
+// tile ids of the first two. Afterwards:
+//     v2 >  v0 + slack : at most two tiles can hold the argmin; they are
+//                        re-evaluated with the exact canonical arithmetic in
+//                        ascending key order (strict '<'), which yields exactly the
+//                        reference's distance and lowest-index argmin;
+//     v2 <= v0 + slack : three or more candidate tiles (heavy ties); the wave scans
+//                        the whole key cloud for that query with exact arithmetic.
+// Non-finite or huge coordinates (where the bound above does not hold) take the
+// exact sweep for the whole workgroup or the exact scan for the query.
+// Results are therefore bit-identical to the exact sweep for every input.
+
+#ifdef TK3D_CHAMFER_STATS
+// Tuning builds only: [0] queries with two candidate tiles, [1] queries sent to the
+// exact wave scan, [2] queries.
+__device__ unsigned long long tk3d_chamfer_stats[4];
+#endif
+
+__device__ __forceinline__ float wave_reduce_min(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = __builtin_fminf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_reduce_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = __builtin_fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// Exact nearest neighbour of one query, the whole workgroup cooperating: lane t scans
+// keys t, t+BLOCK, ... in ascending order with strict '<'; the workgroup keeps the
+// smallest distance and, among equal distances, the lowest key index. Every lane
+// returns the result. `sval` / `sidx` hold one entry per wave.
+template <int BLOCK>
+__device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict__ K, int nk,
+                                                         float qx, float qy, float qz,
+                                                         float *sval, int *sidx, float &out_d,
+                                                         int &out_j)
+{
+    constexpr int NW = BLOCK / TK_WAVE;
+    const int tid = threadIdx.x;
+    float best = __builtin_huge_valf();
+    int bj = -1;
+#pragma unroll 8
+    for (int j = tid; j < nk; j += BLOCK) {
+        const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
+                                        K[(int64_t)j * 3 + 2], qx, qy, qz);
+        if (d < best) {
+            best = d;
+            bj = j;
+        }
+    }
+    const float wmin = wave_reduce_min(best);
+    int cand = (best == wmin && bj >= 0) ? bj : 0x7fffffff;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int other = __shfl_xor(cand, o);
+        cand = other < cand ? other : cand;
+    }
+    __syncthreads();
+    if ((tid & (TK_WAVE - 1)) == 0) {
+        sval[tid / TK_WAVE] = wmin;
+        sidx[tid / TK_WAVE] = cand;
+    }
+    __syncthreads();
+    float g = __builtin_huge_valf();
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        g = __builtin_fminf(g, sval[w]);
+    int gj = 0x7fffffff;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        gj = (sval[w] == g && sidx[w] < gj) ? sidx[w] : gj;
+    out_d = g;
+    out_j = gj == 0x7fffffff ? -1 : gj;
+}
+
+template <int QPL, int BLOCK, int TILE, int STAGE>
+__global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFwdArgs<float> args)
+{
+    static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
+    constexpr int NW = BLOCK / TK_WAVE;
+    // More queries than this with three or more candidate tiles: the cloud is full of
+    // ties (quantised coordinates) and the exact sweep is the cheaper way out.
+    constexpr int MAX_SCANS = 96;
+    __shared__ __align__(16) float skey[2 * STAGE * 4];
+    __shared__ float sred[NW][8];
+    __shared__ int sidx[NW];
+    __shared__ int s_list[MAX_SCANS];
+    __shared__ int s_count;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    int b, qblock;
+    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock);
+    const int nq = d.nq, nk = d.nk;
+    const float *__restrict__ Q = d.query + (int64_t)b * nq * 3;
+    const float *__restrict__ K = d.key + (int64_t)b * nk * 3;
+    const float INF = __builtin_huge_valf();
+
+    // ---- bounding box of the key cloud -> centre ----
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    for (int j = tid; j < nk; j += BLOCK) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const float v = K[(int64_t)j * 3 + a];
+            lo[a] = __builtin_fminf(lo[a], v);
+            hi[a] = __builtin_fmaxf(hi[a], v);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        lo[a] = wave_reduce_min(lo[a]);
+        hi[a] = wave_reduce_max(hi[a]);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            sred[wave][a] = lo[a];
+            sred[wave][3 + a] = hi[a];
+        }
+    }
+    if (tid == 0)
+        s_count = 0;
+    __syncthreads();
+    float cc[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float l = INF, h = -INF;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][a]);
+            h = __builtin_fmaxf(h, sred[w][3 + a]);
+        }
+        cc[a] = 0.5f * l + 0.5f * h;
+    }
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    // ---- largest centred squared norm, computed as the staging below computes it ----
+    float kmax2 = 0.0f;
+    for (int j = tid; j < nk; j += BLOCK) {
+        const float x = K[(int64_t)j * 3 + 0] - c0;
+        const float y = K[(int64_t)j * 3 + 1] - c1;
+        const float z = K[(int64_t)j * 3 + 2] - c2;
+        kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
+    }
+    kmax2 = wave_reduce_max(kmax2);
+    if (lane == 0)
+        sred[wave][6] = kmax2;
+    __syncthreads();
+    kmax2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
+
+    // The error bound needs finite, moderate magnitudes; otherwise do the exact sweep.
+    const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
+                      (kmax2 < 1e30f);
+    if (!safe) {  // uniform over the workgroup
+        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+        return;
+    }
+    // sqrt and the norm carry a few u of rounding; 1e-6 covers them.
+    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+
+    // ---- queries: a = -2 (q - c) ----
+    float ax[QPL], ay[QPL], az[QPL];
+    float v0[QPL], v1[QPL], v2[QPL];
+    int id0[QPL], id1[QPL];
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+        const int qi = (qblock * QPL + i) * BLOCK + tid;
+        const bool ok = qi < nq;
+        ax[i] = -2.0f * ((ok ? Q[(int64_t)qi * 3 + 0] : c0) - c0);
+        ay[i] = -2.0f * ((ok ? Q[(int64_t)qi * 3 + 1] : c1) - c1);
+        az[i] = -2.0f * ((ok ? Q[(int64_t)qi * 3 + 2] : c2) - c2);
+        v0[i] = v1[i] = v2[i] = INF;
+        id0[i] = id1[i] = -1;
+    }
+    // slack = 32 u (max|k'| + |q'|)^2, from a = -2 q'. NaN / inf for a non-finite or
+    // huge query; the epilogue tests for that.
+    auto slack_of = [&](int i) {
+        const float qn = 0.5f * 1.000001f *
+                         __builtin_sqrtf(__builtin_fmaf(az[i], az[i],
+                                                        __builtin_fmaf(ay[i], ay[i], ax[i] * ax[i])));
+        const float r = kmax + qn;
+        return r * r * 1.9073486e-06f + 1e-37f;
+    };
+
+    // ---- sweep ----
+    // Keys are centred and staged as (x', y', z', |k'|^2) in two LDS buffers: the next
+    // stage is fetched into registers before the current one is consumed and stored
+    // to the other buffer afterwards, so a stage costs one barrier and its global
+    // loads overlap the arithmetic.
+    constexpr int PER = STAGE / BLOCK;
+    static_assert(STAGE % BLOCK == 0, "whole keys per lane and stage");
+    const int nstages = (nk + STAGE - 1) / STAGE;
+    float4 pre[PER];
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int kj = st * STAGE + r * BLOCK + tid;
+            float4 e = make_float4(0.0f, 0.0f, 0.0f, INF);  // past the end: s = +inf
+            if (kj < nk) {
+                e.x = K[(int64_t)kj * 3 + 0] - c0;
+                e.y = K[(int64_t)kj * 3 + 1] - c1;
+                e.z = K[(int64_t)kj * 3 + 2] - c2;
+                e.w = __builtin_fmaf(e.z, e.z, __builtin_fmaf(e.y, e.y, e.x * e.x));
+            }
+            pre[r] = e;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r)
+            reinterpret_cast<float4 *>(skey)[buf * STAGE + r * BLOCK + tid] = pre[r];
+    };
+    __syncthreads();
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int st = 0; st < nstages; ++st) {
+        const int stage0 = st * STAGE;
+        if (st + 1 < nstages)
+            fetch(st + 1);
+        const float4 *sbuf = reinterpret_cast<const float4 *>(skey) + (st & 1) * STAGE;
+
+        const int left = nk - stage0;
+        const int ntiles = ((left < STAGE ? left : STAGE) + TILE - 1) / TILE;
+        for (int t = 0; t < ntiles; ++t) {
+            float tmin[QPL];
+#pragma unroll
+            for (int i = 0; i < QPL; ++i)
+                tmin[i] = INF;
+            const float4 *tk = sbuf + t * TILE;
+#pragma unroll
+            for (int j = 0; j < TILE; j += 2) {
+                const float4 ka = tk[j], kb = tk[j + 1];
+#pragma unroll
+                for (int i = 0; i < QPL; ++i) {
+                    const float sa = __builtin_fmaf(
+                        ka.x, ax[i], __builtin_fmaf(ka.y, ay[i], __builtin_fmaf(ka.z, az[i], ka.w)));
+                    const float sb = __builtin_fmaf(
+                        kb.x, ax[i], __builtin_fmaf(kb.y, ay[i], __builtin_fmaf(kb.z, az[i], kb.w)));
+                    tmin[i] = __builtin_fminf(__builtin_fminf(tmin[i], sa), sb);
+                }
+            }
+            // Three smallest tile minima (ties keep the earlier tile in front).
+            const int tile_id = stage0 / TILE + t;
+#pragma unroll
+            for (int i = 0; i < QPL; ++i) {
+                const float x = tmin[i];
+                const bool lt0 = x < v0[i];
+                const bool lt1 = x < v1[i];
+                id1[i] = lt1 ? tile_id : id1[i];
+                id1[i] = lt0 ? id0[i] : id1[i];
+                id0[i] = lt0 ? tile_id : id0[i];
+                v2[i] = __builtin_amdgcn_fmed3f(v1[i], v2[i], x);
+                v1[i] = __builtin_amdgcn_fmed3f(v0[i], v1[i], x);
+                v0[i] = __builtin_amdgcn_fmed3f(-INF, v0[i], x);
+            }
+        }
+
+        if (st + 1 < nstages)
+            stash((st + 1) & 1);
+        __syncthreads();
+
+        // One look, an eighth of the way in: if a quarter of the queries already see
+        // three tiles within the slack, the cloud is quantised and will not get better.
+        if (nstages >= 8 && st == (nstages >> 3)) {
+            int tied = 0;
+#pragma unroll
+            for (int i = 0; i < QPL; ++i) {
+                const int qi = (qblock * QPL + i) * BLOCK + tid;
+                const bool t3 = qi < nq && v2[i] <= v0[i] + slack_of(i);
+                tied += __builtin_popcountll(__builtin_amdgcn_ballot_w64(t3));
+            }
+            if (lane == 0)
+                atomicAdd(&s_count, tied);
+            __syncthreads();
+            const int total = s_count;
+            __syncthreads();
+            if (tid == 0)
+                s_count = 0;
+            if (total * 4 > QPL * BLOCK) {  // uniform over the workgroup
+                chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+                return;
+            }
+        }
+    }
+
+    // ---- epilogue: exact evaluation of the candidate tiles ----
+    static_assert(TILE % 4 == 0, "tile of whole 16-byte groups");
+    const bool k_aligned = (reinterpret_cast<uintptr_t>(K) & 15) == 0;  // tiles are 768 B
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+        const int qi = (qblock * QPL + i) * BLOCK + tid;
+        const bool ok = qi < nq;
+        const float slack = slack_of(i);
+        const float thr = v0[i] + slack;
+        const bool usable = slack < 1e30f;  // false for NaN / inf / huge
+        // No finite score at all (nk == 0 or every key NaN): the exact result is (+inf, -1).
+        const bool none = !(v0[i] < INF);
+        const bool second = v1[i] <= thr;
+        const bool over = ok && !none && (!usable || v2[i] <= thr);
+        float bestd = INF;
+        int bestj = -1;
+        if (ok && !none && !over) {
+            const float qx = Q[(int64_t)qi * 3 + 0], qy = Q[(int64_t)qi * 3 + 1],
+                        qz = Q[(int64_t)qi * 3 + 2];
+            int ta = id0[i], tb = second ? id1[i] : -1;
+            if (tb >= 0 && tb < ta) {
+                const int tmp = ta;
+                ta = tb;
+                tb = tmp;
+            }
+            for (int pass = 0; pass < 2; ++pass) {
+                const int tile = pass == 0 ? ta : tb;
+                if (tile < 0)
+                    continue;
+                const int j0 = tile * TILE;
+                if (k_aligned && j0 + TILE <= nk) {
+                    // 16-byte loads: four keys per three quads.
+                    const float4 *p4 = reinterpret_cast<const float4 *>(K + (int64_t)j0 * 3);
+#pragma unroll 2
+                    for (int g = 0; g < TILE / 4; ++g) {
+                        const float4 f0 = p4[g * 3 + 0], f1 = p4[g * 3 + 1], f2 = p4[g * 3 + 2];
+                        const float dd0 = tk_dist2<float>(f0.x, f0.y, f0.z, qx, qy, qz);
+                        const float dd1 = tk_dist2<float>(f0.w, f1.x, f1.y, qx, qy, qz);
+                        const float dd2 = tk_dist2<float>(f1.z, f1.w, f2.x, qx, qy, qz);
+                        const float dd3 = tk_dist2<float>(f2.y, f2.z, f2.w, qx, qy, qz);
+                        const int j = j0 + g * 4;
+                        if (dd0 < bestd) { bestd = dd0; bestj = j; }
+                        if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
+                        if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
+                        if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
+                    }
+                } else {
+                    const int j1 = (j0 + TILE < nk) ? j0 + TILE : nk;
+                    for (int j = j0; j < j1; ++j) {
+                        const float dd = tk_dist2<float>(K[(int64_t)j * 3 + 0],
+                                                         K[(int64_t)j * 3 + 1],
+                                                         K[(int64_t)j * 3 + 2], qx, qy, qz);
+                        if (dd < bestd) {
+                            bestd = dd;
+                            bestj = j;
+                        }
+                    }
+                }
+            }
+        }
+        if (ok && !over) {
+            d.dist[(int64_t)b * nq + qi] = bestd;
+            d.idx[(int64_t)b * nq + qi] = (int64_t)bestj;
+        }
+        if (over) {
+            const int slot = atomicAdd(&s_count, 1);
+            if (slot < MAX_SCANS)
+                s_list[slot] = i * BLOCK + tid;
+        }
+#ifdef TK3D_CHAMFER_STATS
+        if (ok && !none && !over && second)
+            atomicAdd(&tk3d_chamfer_stats[0], 1ull);
+        if (over)
+            atomicAdd(&tk3d_chamfer_stats[1], 1ull);
+        if (ok)
+            atomicAdd(&tk3d_chamfer_stats[2], 1ull);
+#endif
+    }
+
+    // ---- queries with three or more candidate tiles ----
+    __syncthreads();
+    const int nscan = s_count;
+    if (nscan > MAX_SCANS) {  // uniform over the workgroup
+        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+        return;
+    }
+    for (int e = 0; e < nscan; ++e) {
+        const int slot = s_list[e];
+        const int qi = (qblock * QPL + slot / BLOCK) * BLOCK + (slot % BLOCK);
+        float bd;
+        int bj;
+        chamfer_block_exact_scan<BLOCK>(K, nk, Q[(int64_t)qi * 3 + 0], Q[(int64_t)qi * 3 + 1],
+                                        Q[(int64_t)qi * 3 + 2], &sred[0][0], sidx, bd, bj);
+        if (tid == 0) {
+            d.dist[(int64_t)b * nq + qi] = bd;
+            d.idx[(int64_t)b * nq + qi] = (int64_t)bj;
+        }
     }
 }
 
@@ -254,6 +686,27 @@ int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
     return tk_launch_status();
 }
 
+template <int QPL, int BLOCK = 256, int TILE = 64, int STAGE = 1024>
+int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
+                                  int64_t N2, float *dist1, int64_t *idx1, float *dist2,
+                                  int64_t *idx2, hipStream_t stream)
+{
+    constexpr int QB = QPL * BLOCK;
+    ChamferFwdArgs<float> a;
+    a.dir[0] = {xyz1, xyz2, dist1, idx1, (int)N1, (int)N2, (int)((N1 + QB - 1) / QB)};
+    a.dir[1] = {xyz2, xyz1, dist2, idx2, (int)N2, (int)N1, (int)((N2 + QB - 1) / QB)};
+    const int64_t nb0 = B * a.dir[0].blocks_per_batch;
+    const int64_t nb1 = B * a.dir[1].blocks_per_batch;
+    if (nb0 + nb1 == 0)
+        return TK3D_OK;
+    if (nb0 + nb1 > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    a.nblocks0 = (int)nb0;
+    hipLaunchKernelGGL((chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE>),
+                       dim3((unsigned)(nb0 + nb1)), dim3(BLOCK), 0, stream, a);
+    return tk_launch_status();
+}
+
 template <typename T>
 int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t N2,
                     T *dist1, int64_t *idx1, T *dist2, int64_t *idx2, void *stream)
@@ -271,6 +724,21 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
     // Fewer queries per lane when the clouds are small, so the launch still
     // spreads over the chip.
     const int64_t work = B * (N1 > N2 ? N1 : N2);
+    if constexpr (sizeof(T) == 4) {
+        // The pre-filter pays off once the key cloud is long enough to amortise its
+        // prologue (two passes over the keys per workgroup).
+        const int64_t nkmin = N1 < N2 ? N1 : N2;
+        if (nkmin >= 2048) {
+            // Shapes timed on an MI355X: 4 queries per lane; 512-lane workgroups once
+            // that still gives every CU two of them.
+            if (B * (N1 + N2) >= (int64_t)2048 * 512)
+                return chamfer_forward_filter_launch<4, 512, 64, 512>(
+                    xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s);
+            if (B * (N1 + N2) >= (int64_t)1024 * 256)
+                return chamfer_forward_filter_launch<4, 256, 64, 512>(
+                    xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s);
+        }
+    }
     if (sizeof(T) == 8 || work < (int64_t)256 * 1024)
         return chamfer_forward_launch<T, 2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                             idx2, s);
