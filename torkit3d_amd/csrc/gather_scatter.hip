@@ -105,6 +105,87 @@ __global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
     }
 }
 
+// Same gather with the source rows staged in LDS. Row gathers through the vector
+// cache cost one cache line per lane (64 lanes -> 64 lines per load instruction),
+// which caps the plain kernel near 2 TB/s of output; LDS serves the same random
+// reads at bank rate. grid = (point chunks, channel groups, B); LDS = cg*n1 elements.
+template <typename T, int KK, bool HAS_W, int V, int NT>
+__global__ __launch_bounds__(NT) void gather_lds_kernel(
+    const T *__restrict__ in, const int64_t *__restrict__ idx, const T *__restrict__ w,
+    T *__restrict__ out, int c_total, int n1, int64_t np, int cg, int64_t chunk_len, int vec_ok)
+{
+    extern __shared__ __align__(16) unsigned char gather_smem[];
+    T *rows = reinterpret_cast<T *>(gather_smem);  // [cg][n1]
+    const int b = blockIdx.z;
+    const int c0 = blockIdx.y * cg;
+    const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
+    const T *__restrict__ src_rows = in + ((int64_t)b * c_total + c0) * n1;
+    for (int i = threadIdx.x; i < nc * n1; i += NT)
+        rows[i] = src_rows[i];
+    __syncthreads();
+
+    const int64_t ps = (int64_t)blockIdx.x * chunk_len;
+    const int64_t pe = (ps + chunk_len < np) ? ps + chunk_len : np;
+    for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += (int64_t)NT * V) {
+        int src[V][KK];
+        T wt[V][KK];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+#pragma unroll
+            for (int i = 0; i < KK; ++i) {
+                const int64_t p = p0 + v;
+                int64_t j = -1;
+                T ww = (T)0;
+                if (p < pe) {
+                    j = idx[((int64_t)b * np + p) * KK + i];
+                    if (HAS_W)
+                        ww = w[((int64_t)b * np + p) * KK + i];
+                }
+                src[v][i] = (j >= 0 && j < n1) ? (int)j : -1;
+                wt[v][i] = ww;
+            }
+        }
+        const bool full = (p0 + V <= pe);
+#pragma unroll 4
+        for (int c = 0; c < nc; ++c) {
+            const T *row = rows + c * n1;
+            T *__restrict__ orow = out + ((int64_t)b * c_total + c0 + c) * np;
+            T val[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                if (HAS_W) {
+                    T acc = (T)0;
+#pragma unroll
+                    for (int i = 0; i < KK; ++i)
+                        if (src[v][i] >= 0)
+                            acc = tk_fma<T>(row[src[v][i]], wt[v][i], acc);
+                    val[v] = acc;
+                } else {
+                    val[v] = src[v][0] >= 0 ? row[src[v][0]] : (T)0;
+                }
+            }
+            if (full && vec_ok && V == 4 && sizeof(T) == 4) {
+                float4 pack;
+                pack.x = (float)val[0];
+                pack.y = (float)val[1 % V];
+                pack.z = (float)val[2 % V];
+                pack.w = (float)val[3 % V];
+                *reinterpret_cast<float4 *>(orow + p0) = pack;
+            } else if (full && vec_ok && V == 2 && sizeof(T) == 8) {
+                double2 pack;
+                pack.x = (double)val[0];
+                pack.y = (double)val[1 % V];
+                *reinterpret_cast<double2 *>(orow + p0) = pack;
+            } else {
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    if (p0 + v < pe)
+                        orow[p0 + v] = val[v];
+            }
+        }
+    }
+}
+
 // ---- scatter ---------------------------------------------------------------------
 
 template <typename T>
@@ -115,12 +196,74 @@ __global__ __launch_bounds__(GS_BLOCK) void fill_zero_kernel(T *__restrict__ p, 
         p[i] = (T)0;
 }
 
-// LDS-resident destination rows. grid = (segments, channel groups, B).
-template <typename T, int KK, bool HAS_W, int NT>
+// Streams the points [ps, pe) of one batch for `nc` channels starting at c0 and hands
+// every contribution to `sink(ctx, c, dst, value, weight)`, where `ctx = prep(c)` is
+// evaluated once per channel and lane iteration. A lane takes V consecutive
+// points so that the streamed operand is read with 16-byte loads, and the channel
+// loop is unrolled to keep several of them in flight.
+template <typename T, int KK, bool HAS_W, int V, int NT, typename Prep, typename Sink>
+__device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
+                                               const int64_t *__restrict__ idx,
+                                               const T *__restrict__ w, int b, int c_total,
+                                               int c0, int nc, int n1, int64_t np, int64_t ps,
+                                               int64_t pe, int vec_ok, Prep prep, Sink sink)
+{
+    for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += (int64_t)NT * V) {
+        int dst[V][KK];
+        T wt[V][KK];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+#pragma unroll
+            for (int i = 0; i < KK; ++i) {
+                int64_t j = -1;
+                T ww = (T)1;
+                if (p0 + v < pe) {
+                    j = idx[((int64_t)b * np + p0 + v) * KK + i];
+                    if (HAS_W)
+                        ww = w[((int64_t)b * np + p0 + v) * KK + i];
+                }
+                dst[v][i] = (j >= 0 && j < n1) ? (int)j : -1;
+                wt[v][i] = ww;
+            }
+        }
+        const bool full = (p0 + V <= pe);
+#pragma unroll 4
+        for (int c = 0; c < nc; ++c) {
+            const T *__restrict__ grow = gout + ((int64_t)b * c_total + c0 + c) * np;
+            T g[V];
+            if (full && vec_ok && V == 4 && sizeof(T) == 4) {
+                const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
+                g[0] = (T)pack.x;
+                g[1 % V] = (T)pack.y;
+                g[2 % V] = (T)pack.z;
+                g[3 % V] = (T)pack.w;
+            } else if (full && vec_ok && V == 2 && sizeof(T) == 8) {
+                const double2 pack = *reinterpret_cast<const double2 *>(grow + p0);
+                g[0] = (T)pack.x;
+                g[1 % V] = (T)pack.y;
+            } else {
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    g[v] = (p0 + v < pe) ? grow[p0 + v] : (T)0;
+            }
+            const auto ctx = prep(c);
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+#pragma unroll
+                for (int i = 0; i < KK; ++i)
+                    if (dst[v][i] >= 0)
+                        sink(ctx, c, dst[v][i], g[v], wt[v][i]);
+        }
+    }
+}
+
+// LDS-resident destination rows with floating-point LDS atomics.
+// grid = (segments, channel groups, B).
+template <typename T, int KK, bool HAS_W, int V, int NT>
 __global__ __launch_bounds__(NT) void scatter_lds_kernel(
     const T *__restrict__ gout, const int64_t *__restrict__ idx, const T *__restrict__ w,
     T *__restrict__ gin, int c_total, int n1, int64_t np, int cg, int64_t seg_len,
-    int merge_with_atomics)
+    int merge_with_atomics, int vec_ok)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *rows = reinterpret_cast<T *>(smem_raw);  // [cg][n1]
@@ -133,24 +276,9 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
     for (int i = threadIdx.x; i < nc * n1; i += NT)
         rows[i] = (T)0;
     __syncthreads();
-
-    for (int64_t p = ps + threadIdx.x; p < pe; p += NT) {
-        int dst[KK];
-        T wt[KK];
-#pragma unroll
-        for (int i = 0; i < KK; ++i) {
-            const int64_t j = idx[((int64_t)b * np + p) * KK + i];
-            dst[i] = (j >= 0 && j < n1) ? (int)j : -1;
-            wt[i] = HAS_W ? w[((int64_t)b * np + p) * KK + i] : (T)1;
-        }
-        for (int c = 0; c < nc; ++c) {
-            const T g = gout[((int64_t)b * c_total + c0 + c) * np + p];
-#pragma unroll
-            for (int i = 0; i < KK; ++i)
-                if (dst[i] >= 0)
-                    atomicAdd(&rows[c * n1 + dst[i]], HAS_W ? g * wt[i] : g);
-        }
-    }
+    scatter_stream<T, KK, HAS_W, V, NT>(
+        gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        [&](int, int c, int dst, T g, T ww) { atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g); });
     __syncthreads();
 
     T *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
@@ -163,6 +291,196 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
     } else {
         for (int i = threadIdx.x; i < nc * n1; i += NT)
             dstrows[i] = rows[i];
+    }
+}
+
+// fp32 scatter with 64-bit fixed-point accumulators in LDS.
+//
+// Floating-point LDS atomics on this GPU retire about one lane every three clocks
+// (measured: 195 clocks per wave instruction, conflicts or not); integer LDS
+// atomics run at the rate of a plain LDS write, 13 times faster. So each
+// contribution g*w (rounded to fp32 as the reference rounds it) is converted to an
+// integer at a per-row power-of-two scale and added with ds_add_u64:
+//   * magnitudes: the workgroup samples one 16-byte group in eight of its share of
+//     gout for max|g| per row (and reads all of w for max|w|), and allows 64 times
+//     that as the bound B_c of a row;
+//   * scale: 2^k with k the largest integer keeping B_c * 2^k below 2^50 and
+//     count * B_c * 2^k below 2^62, i.e. a resolution of 2^-40 of the row maximum
+//     or better for up to 2^16 terms per row; fp32 accumulation resolves 2^-24;
+//   * conversion: fma(double(term), 2^k, 1.5 * 2^52) leaves the rounded integer in
+//     the low mantissa bits (one cvt, one fma, one 64-bit subtract);
+//   * a term above its row's bound (the sample missed an outlier) raises a flag;
+//     the workgroup then repeats the pass with bounds from the full data.
+// Integer addition is associative, so unlike the reference the result does not
+// depend on the order in which the contributions arrive. A row holding NaN or inf
+// has no usable scale; the workgroup then takes the floating-point path.
+template <int KK, bool HAS_W, int V, int NT, int CGMAX>
+__global__ __launch_bounds__(NT) void scatter_fixed_kernel(
+    const float *__restrict__ gout, const int64_t *__restrict__ idx,
+    const float *__restrict__ w, float *__restrict__ gin, int c_total, int n1, int64_t np, int cg,
+    int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);  // [cg][n1]
+    __shared__ unsigned s_maxg[CGMAX];  // bit patterns of non-negative floats order as integers
+    __shared__ unsigned s_maxw;
+    __shared__ int s_kexp[CGMAX];
+    __shared__ double s_scale[CGMAX];
+    __shared__ float s_bound[CGMAX];
+    __shared__ int s_finite, s_exceeded;
+    const int b = blockIdx.z;
+    const int c0 = blockIdx.y * cg;
+    const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
+    const int64_t ps = (int64_t)blockIdx.x * seg_len;
+    const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
+    const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+
+    if (threadIdx.x == 0)
+        s_maxw = HAS_W ? 0u : 0x3f800000u;
+    if (HAS_W) {
+        __syncthreads();
+        unsigned mw = 0u;
+        for (int64_t e = ps * KK + threadIdx.x; e < pe * KK; e += NT) {
+            const unsigned bits =
+                __builtin_bit_cast(unsigned, w[(int64_t)b * np * KK + e]) & 0x7fffffffu;
+            mw = bits > mw ? bits : mw;
+        }
+        if (mw != 0u)
+            atomicMax(&s_maxw, mw);
+    }
+
+    for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
+        __syncthreads();
+        for (int i = threadIdx.x; i < nc * n1; i += NT)
+            acc[i] = 0ull;
+        if (threadIdx.x < CGMAX)
+            s_maxg[threadIdx.x] = 0u;
+        if (threadIdx.x == 0) {
+            s_finite = 1;
+            s_exceeded = 0;
+        }
+        __syncthreads();
+
+        // ---- magnitudes: every 8th group first, everything on the second attempt ----
+        {
+            const int64_t stride = (int64_t)NT * V * (attempt == 0 ? 8 : 1);
+            unsigned mg[CGMAX];
+#pragma unroll
+            for (int c = 0; c < CGMAX; ++c)
+                mg[c] = 0u;
+            for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += stride) {
+                const bool full = (p0 + V <= pe);
+#pragma unroll
+                for (int c = 0; c < CGMAX; ++c) {
+                    if (c >= nc)
+                        break;
+                    const float *__restrict__ grow = gout + ((int64_t)b * c_total + c0 + c) * np;
+                    float g[V];
+                    if (full && vec_ok && V == 4) {
+                        const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
+                        g[0] = pack.x;
+                        g[1 % V] = pack.y;
+                        g[2 % V] = pack.z;
+                        g[3 % V] = pack.w;
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < V; ++v)
+                            g[v] = (p0 + v < pe) ? grow[p0 + v] : 0.0f;
+                    }
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const unsigned bits = __builtin_bit_cast(unsigned, g[v]) & 0x7fffffffu;
+                        mg[c] = bits > mg[c] ? bits : mg[c];
+                    }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < CGMAX; ++c)
+                if (c < nc && mg[c] != 0u)
+                    atomicMax(&s_maxg[c], mg[c]);
+        }
+        __syncthreads();
+
+        // ---- bounds and scales: lane c < CGMAX works out row c ----
+        if (threadIdx.x < CGMAX) {
+            const float maxw = __builtin_bit_cast(float, s_maxw);
+            const float headroom = attempt == 0 ? 64.0f : 1.000001f;
+            const float bound = __builtin_bit_cast(float, s_maxg[threadIdx.x]) * maxw * headroom;
+            if (!(bound < 3.0e38f))  // NaN or inf (NaN has the largest bit pattern)
+                s_finite = 0;
+            int e = 0;
+            (void)__builtin_frexpf(bound, &e);  // bound < 2^e (bound == 0 gives e = 0)
+            // one term stays below 2^50 (the conversion below is exact to 2^51) and the
+            // sum of `count` terms below 2^62
+            s_kexp[threadIdx.x] = (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
+            s_scale[threadIdx.x] = __builtin_ldexp(1.0, s_kexp[threadIdx.x]);
+            s_bound[threadIdx.x] = bound;
+        }
+        __syncthreads();
+        if (!s_finite)
+            break;
+
+        struct RowScale {
+            double scale;
+            float bound;
+        };
+        bool exceeded = false;
+        scatter_stream<float, KK, HAS_W, V, NT>(
+            gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok,
+            [&](int c) {
+                RowScale r;
+                r.scale = s_scale[c];
+                r.bound = s_bound[c];
+                return r;
+            },
+            [&](const RowScale &r, int c, int dst, float g, float ww) {
+                const float term = HAS_W ? g * ww : g;
+                exceeded = exceeded || !(__builtin_fabsf(term) <= r.bound);  // also NaN
+                const double d = __builtin_fma((double)term, r.scale, MAGIC);
+                const unsigned long long q = __builtin_bit_cast(unsigned long long, d) -
+                                             __builtin_bit_cast(unsigned long long, MAGIC);
+                atomicAdd(&acc[c * n1 + dst], q);
+            });
+        if (exceeded)
+            s_exceeded = 1;
+        __syncthreads();
+        if (!s_exceeded) {
+            float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
+            for (int i = threadIdx.x; i < nc * n1; i += NT) {
+                const float v =
+                    (float)__builtin_ldexp((double)(long long)acc[i], -s_kexp[i / n1]);
+                if (merge_with_atomics) {
+                    if (v != 0.0f)
+                        unsafeAtomicAdd(&dstrows[i], v);
+                } else {
+                    dstrows[i] = v;
+                }
+            }
+            return;
+        }
+    }
+
+    // ---- non-finite input: floating-point accumulation in the same LDS ----
+    float *rows = reinterpret_cast<float *>(smem_raw);
+    __syncthreads();
+    for (int i = threadIdx.x; i < nc * n1; i += NT)
+        rows[i] = 0.0f;
+    __syncthreads();
+    scatter_stream<float, KK, HAS_W, V, NT>(
+        gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        [&](int, int c, int dst, float g, float ww) {
+            atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g);
+        });
+    __syncthreads();
+    float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
+    for (int i = threadIdx.x; i < nc * n1; i += NT) {
+        const float v = rows[i];
+        if (merge_with_atomics) {
+            if (v != 0.0f)
+                unsafeAtomicAdd(&dstrows[i], v);
+        } else {
+            dstrows[i] = v;
+        }
     }
 }
 
@@ -221,6 +539,36 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
     if (!idx || !out || (HAS_W && !w))
         return TK3D_ERR_NULL_POINTER;
     constexpr int V = (sizeof(T) == 4) ? 4 : 2;
+    // 16-byte stores need every output row to start on a 16-byte boundary.
+    const int vec_ok = (((uintptr_t)out & 15) == 0) && ((NP * (int64_t)sizeof(T)) % 16 == 0);
+
+    constexpr int64_t LDS_BUDGET = 64 * 1024;
+    const int64_t row_bytes = N1 * (int64_t)sizeof(T);
+    if (row_bytes > 0 && row_bytes <= LDS_BUDGET && NP >= 1024) {
+        constexpr int NT = 512;
+        int cg = 8;
+        while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
+            cg /= 2;
+        const int64_t gy = (C + cg - 1) / cg;
+        // Split the points until the chip is full; every chunk re-stages its rows, so
+        // keep a chunk well above the staged size.
+        int64_t chunks = 1;
+        const int64_t min_chunk = (int64_t)NT * V * 4;
+        while (B * gy * chunks < 1024 && NP / (chunks * 2) >= min_chunk &&
+               (NP / (chunks * 2)) * KK >= (cg * N1) / 2)
+            chunks *= 2;
+        int64_t chunk_len = (NP + chunks - 1) / chunks;
+        chunk_len = (chunk_len + 15) / 16 * 16;  // keeps 16-byte alignment of chunk starts
+        chunks = (NP + chunk_len - 1) / chunk_len;
+        if (gy > 65535 || chunks > TK_MAX_I32)
+            return TK3D_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((gather_lds_kernel<T, KK, HAS_W, V, NT>),
+                           dim3((unsigned)chunks, (unsigned)gy, (unsigned)B), dim3(NT),
+                           (size_t)(cg * row_bytes), s, in, idx, w, out, (int)C, (int)N1, NP, cg,
+                           chunk_len, vec_ok);
+        return tk_launch_status();
+    }
+
     const int64_t tiles = (NP + (int64_t)GS_BLOCK * V - 1) / ((int64_t)GS_BLOCK * V);
     // Channels per workgroup: enough to amortise the index reads, few enough to
     // keep at least ~2k workgroups in flight.
@@ -230,8 +578,6 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
     const int64_t gy = (C + cg - 1) / cg;
     if (tiles > TK_MAX_I32 || gy > 65535)
         return TK3D_ERR_UNSUPPORTED;
-    // 16-byte stores need every output row to start on a 16-byte boundary.
-    const int vec_ok = (((uintptr_t)out & 15) == 0) && ((NP * (int64_t)sizeof(T)) % 16 == 0);
     hipLaunchKernelGGL((gather_kernel<T, KK, HAS_W, V>),
                        dim3((unsigned)tiles, (unsigned)gy, (unsigned)B), dim3(GS_BLOCK), 0, s,
                        in, idx, w, out, (int)C, (int)N1, NP, cg, vec_ok);
@@ -258,38 +604,94 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
         return tk_launch_status();
     }
 
+    if constexpr (sizeof(T) == 4) {
+        // fp32: 64-bit fixed-point accumulators, up to 128 KiB of LDS per workgroup.
+        constexpr int64_t FIXED_LDS = 128 * 1024;
+        constexpr int NT = 1024, V = 4, CGMAX = 8;
+        const int64_t acc_row = N1 * 8;
+        if (acc_row <= FIXED_LDS) {
+            const int vec_ok = (((uintptr_t)gout & 15) == 0) && ((NP * 4) % 16 == 0);
+            int cg = CGMAX;
+            while (cg > 1 && (cg * acc_row > FIXED_LDS || cg > C))
+                cg /= 2;
+            // Prefer more workgroups over wider channel groups until every CU has one.
+            while (cg > 2 && B * ((C + cg - 1) / cg) < 256)
+                cg /= 2;
+            const int64_t gy = (C + cg - 1) / cg;
+            int64_t nseg = 1;
+            const int64_t groups = B * gy;
+            if (groups < 128) {
+                nseg = (256 + groups - 1) / groups;
+                const int64_t max_seg = (NP + 4 * NT * V - 1) / (4 * NT * V);
+                if (nseg > max_seg)
+                    nseg = max_seg;
+                if (nseg < 1)
+                    nseg = 1;
+            }
+            int64_t seg_len = (NP + nseg - 1) / nseg;
+            seg_len = (seg_len + 15) / 16 * 16;
+            nseg = (NP + seg_len - 1) / seg_len;
+            if (gy > 65535 || nseg > TK_MAX_I32)
+                return TK3D_ERR_UNSUPPORTED;
+            int log2_count = 1;
+            while (((int64_t)1 << log2_count) < seg_len * KK + 1)
+                ++log2_count;
+            auto kernel = scatter_fixed_kernel<KK, HAS_W, V, NT, CGMAX>;
+            static bool lds_opt_in = false;  // raising the limit is idempotent
+            if (!lds_opt_in) {
+                const hipError_t e = hipFuncSetAttribute(
+                    reinterpret_cast<const void *>(kernel),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)FIXED_LDS);
+                if (e != hipSuccess)
+                    return (int)e;
+                lds_opt_in = true;
+            }
+            if (nseg > 1)
+                hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
+                                   dim3(GS_BLOCK), 0, s, gin, out_elems);
+            hipLaunchKernelGGL(kernel, dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
+                               (size_t)(cg * acc_row), s, gout, idx, w, gin, (int)C, (int)N1, NP,
+                               cg, seg_len, nseg > 1 ? 1 : 0, vec_ok, log2_count);
+            return tk_launch_status();
+        }
+    }
+
     constexpr int64_t LDS_BUDGET = 64 * 1024;
     const int64_t row_bytes = N1 * (int64_t)sizeof(T);
     if (row_bytes <= LDS_BUDGET) {
         constexpr int NT = 512;
+        constexpr int V = (sizeof(T) == 4) ? 4 : 2;
+        const int vec_ok =
+            (((uintptr_t)gout & 15) == 0) && ((NP * (int64_t)sizeof(T)) % 16 == 0);
         int cg = 8;
         while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
             cg /= 2;
         // Prefer more workgroups over wider channel groups until the chip is full.
-        while (cg > 1 && B * ((C + cg - 1) / cg) < 512)
+        while (cg > 2 && B * ((C + cg - 1) / cg) < 512)
             cg /= 2;
         const int64_t gy = (C + cg - 1) / cg;
         int64_t nseg = 1;
         const int64_t groups = B * gy;
         if (groups < 256) {
             nseg = (512 + groups - 1) / groups;
-            const int64_t max_seg = (NP + 4 * NT - 1) / (4 * NT);  // >= 4 points per thread
+            const int64_t max_seg = (NP + 4 * NT * V - 1) / (4 * NT * V);  // >= 4 rounds per lane
             if (nseg > max_seg)
                 nseg = max_seg;
             if (nseg < 1)
                 nseg = 1;
         }
-        const int64_t seg_len = (NP + nseg - 1) / nseg;
+        int64_t seg_len = (NP + nseg - 1) / nseg;
+        seg_len = (seg_len + 15) / 16 * 16;  // keeps 16-byte alignment of segment starts
         nseg = (NP + seg_len - 1) / seg_len;
         if (gy > 65535 || nseg > TK_MAX_I32)
             return TK3D_ERR_UNSUPPORTED;
         if (nseg > 1)
             hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
                                dim3(GS_BLOCK), 0, s, gin, out_elems);
-        hipLaunchKernelGGL((scatter_lds_kernel<T, KK, HAS_W, NT>),
+        hipLaunchKernelGGL((scatter_lds_kernel<T, KK, HAS_W, V, NT>),
                            dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
                            (size_t)(cg * row_bytes), s, gout, idx, w, gin, (int)C, (int)N1, NP,
-                           cg, seg_len, nseg > 1 ? 1 : 0);
+                           cg, seg_len, nseg > 1 ? 1 : 0, vec_ok);
         return tk_launch_status();
     }
 
