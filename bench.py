@@ -130,6 +130,14 @@ def secondary_metrics(dev, steps, warmup):
     g4 = torch.randn(32, 128, 8192, generator=g).to(dev)
     out["interpolate_bwd_ms"] = gpu_time_ms(
         lambda: _C.interpolate_backward_cuda(g4, kidx, w, 2048), steps, warmup)
+    g = torch.Generator().manual_seed(5)
+    a = sphere_cloud(g, 32, 16384).to(dev)
+    c = sphere_cloud(g, 32, 16384).to(dev)
+    _, i1, _, i2 = _C.chamfer_distance_forward_cuda(a, c)
+    gd1 = torch.randn(32, 16384, generator=g).to(dev)
+    gd2 = torch.randn(32, 16384, generator=g).to(dev)
+    out["chamfer_bwd_B32_N16384_ms"] = gpu_time_ms(
+        lambda: _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2), steps, warmup)
     return {k: round(v, 5) for k, v in out.items()}
 
 
