@@ -213,6 +213,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
 // Tuning builds only: [0] queries with two candidate tiles, [1] queries sent to the
 // exact wave scan, [2] queries.
 __device__ unsigned long long tk3d_chamfer_stats[4];
+__device__ long long tk3d_chamfer_stamps[16];
 #endif
 
 __device__ __forceinline__ float wave_reduce_min(float v)
@@ -665,6 +666,238 @@ __global__ __launch_bounds__(256) void chamfer_backward_scatter_kernel(
     }
 }
 
+// fp32 backward without global atomics, in one launch. A workgroup owns a range of
+// R points of one cloud X in one batch and produces their gradients completely:
+//   grad_X[j] = 2 gX[j] (x_j - y_{idxX[j]})                     the point's own term
+//             - sum_{i : idxY[i] = j} 2 gY[i] (y_i - x_j)       terms sent by cloud Y
+// It scans all of cloud Y's matches, accumulates those that land in its range in
+// 64-bit fixed-point LDS accumulators (integer LDS atomics run an order of
+// magnitude faster than floating-point ones on this GPU, and make the sum
+// independent of arrival order), adds the own term and stores each gradient once.
+// Scale: a power of two chosen from a bound on |term| taken over a sample of the
+// senders times 64; a term above the bound raises a flag and the workgroup repeats
+// with the bound over all senders. Non-finite input takes the floating-point path.
+template <int R, int NT>
+__global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
+    const float *__restrict__ gd1, const float *__restrict__ gd2,
+    const float *__restrict__ xyz1, const float *__restrict__ xyz2,
+    const int64_t *__restrict__ idx1, const int64_t *__restrict__ idx2, int n1, int n2,
+    int ranges1, int ranges2, int nblocks1, float *__restrict__ gx1, float *__restrict__ gx2)
+{
+    extern __shared__ __align__(16) unsigned long long acc[];  // [R * 3]
+    __shared__ unsigned s_max;
+    __shared__ int s_exceeded;
+    const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+
+    // Decode: the first nblocks1 workgroups produce grad_xyz1, the rest grad_xyz2.
+    int lb = blockIdx.x;
+    const bool second = lb >= nblocks1;
+    if (second)
+        lb -= nblocks1;
+    const int ranges = second ? ranges2 : ranges1;
+    const int b = lb / ranges;
+    const int j0 = (lb - b * ranges) * R;
+    const int nx = second ? n2 : n1, ny = second ? n1 : n2;
+    const float *__restrict__ X = (second ? xyz2 : xyz1) + (int64_t)b * nx * 3;
+    const float *__restrict__ Y = (second ? xyz1 : xyz2) + (int64_t)b * ny * 3;
+    const float *__restrict__ gX = (second ? gd2 : gd1) + (int64_t)b * nx;
+    const float *__restrict__ gY = (second ? gd1 : gd2) + (int64_t)b * ny;
+    const int64_t *__restrict__ iX = (second ? idx2 : idx1) + (int64_t)b * nx;
+    const int64_t *__restrict__ iY = (second ? idx1 : idx2) + (int64_t)b * ny;
+    float *__restrict__ out = (second ? gx2 : gx1) + (int64_t)b * nx * 3;
+    const int j1 = (j0 + R < nx) ? j0 + R : nx;
+
+#ifdef TK3D_CHAMFER_STATS
+#define TK3D_STAMP(n) do { if (blockIdx.x == 0 && threadIdx.x == 0) tk3d_chamfer_stamps[n] = wall_clock64(); } while (0)
+#else
+#define TK3D_STAMP(n) do { } while (0)
+#endif
+    TK3D_STAMP(0);
+    bool use_float = false;
+    for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
+        __syncthreads();
+        for (int t = threadIdx.x; t < R * 3; t += NT)
+            acc[t] = 0ull;
+        if (threadIdx.x == 0) {
+            s_max = 0u;
+            s_exceeded = 0;
+        }
+        __syncthreads();
+        // bound on |term| over the senders: every 8th run of 64 consecutive senders on
+        // the first attempt (coalesced), all of them on the second. The match indices
+        // of U senders are fetched together so their latencies overlap.
+        constexpr int U = 8;
+        unsigned m = 0u;
+        const int nsample = attempt == 0 ? (ny + 7) / 8 : ny;
+        for (int s0 = threadIdx.x; s0 < nsample; s0 += NT * U) {
+            int64_t jj[U];
+            int ii[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int sidx = s0 + u * NT;
+                const int i = attempt == 0 ? (sidx >> 6) * 512 + (sidx & 63) : sidx;
+                ii[u] = (sidx < nsample && i < ny) ? i : -1;
+                jj[u] = ii[u] >= 0 ? iY[ii[u]] : -1;
+            }
+            float g[U], y[U][3], x[U][3];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool ok = jj[u] >= 0 && jj[u] < nx;
+                const int is = ok ? ii[u] : 0;
+                g[u] = ok ? gY[is] * 2 : 0.0f;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    y[u][a] = Y[(int64_t)is * 3 + a];
+                    x[u][a] = X[(ok ? jj[u] : 0) * 3 + a];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (jj[u] < 0 || jj[u] >= nx)
+                    continue;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    const float v = g[u] * (y[u][a] - x[u][a]);
+                    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7fffffffu;
+                    m = bits > m ? bits : m;
+                }
+            }
+        }
+        if (m != 0u)
+            atomicMax(&s_max, m);
+        __syncthreads();
+        TK3D_STAMP(1 + attempt * 4);
+        const float bound = __builtin_bit_cast(float, s_max) * (attempt == 0 ? 64.0f : 1.000001f);
+        if (!(bound < 3.0e38f)) {  // NaN or inf
+            use_float = true;
+            break;
+        }
+        int e = 0;
+        (void)__builtin_frexpf(bound, &e);
+        // a term below 2^50, and up to 2^12 of them (more senders than that on one
+        // point lower the scale further below)
+        int log2_count = 1;
+        while ((1 << log2_count) < ny + 1)
+            ++log2_count;
+        const int kexp = (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
+        const double scale = __builtin_ldexp(1.0, kexp);
+
+        bool exceeded = false;
+        for (int i0 = threadIdx.x; i0 < ny; i0 += NT * U) {
+            // Everything a sender needs is requested before anything is used: U
+            // match indices, then U gradients and 2U points, all in flight together.
+            int64_t jj[U];
+            float g[U], y[U][3], x[U][3];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u * NT;
+                jj[u] = i < ny ? iY[i] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u * NT;
+                // Senders that match outside the range read one fixed element instead
+                // (a broadcast), so only the index stream is paid for per range.
+                const bool in = jj[u] >= j0 && jj[u] < j1;
+                const int64_t js = in ? jj[u] : (int64_t)j0;
+                const int is = in ? i : 0;
+                g[u] = gY[is] * 2;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    y[u][a] = Y[(int64_t)is * 3 + a];
+                    x[u][a] = X[js * 3 + a];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (jj[u] < j0 || jj[u] >= j1)
+                    continue;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    const float v = -(g[u] * (y[u][a] - x[u][a]));
+                    exceeded = exceeded || !(__builtin_fabsf(v) <= bound);
+                    const double d = __builtin_fma((double)v, scale, MAGIC);
+                    atomicAdd(&acc[(jj[u] - j0) * 3 + a],
+                              __builtin_bit_cast(unsigned long long, d) -
+                                  __builtin_bit_cast(unsigned long long, MAGIC));
+                }
+            }
+        }
+        if (exceeded)
+            s_exceeded = 1;
+        __syncthreads();
+        TK3D_STAMP(2 + attempt * 4);
+        if (!s_exceeded) {
+            // own terms: a lane takes whole points, F of them per round, with the
+            // match indices and then the matched points fetched together
+            constexpr int F = 4;
+            for (int p0 = threadIdx.x; p0 < j1 - j0; p0 += NT * F) {
+                int64_t mj[F];
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    const int p = p0 + f * NT;
+                    mj[f] = p < j1 - j0 ? iX[j0 + p] : -1;
+                }
+                float gg[F], xs[F][3], ys[F][3];
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    const int p = p0 + f * NT;
+                    const int j = j0 + (p < j1 - j0 ? p : 0);
+                    const bool ok = mj[f] >= 0 && mj[f] < ny;
+                    gg[f] = ok ? gX[j] * 2 : 0.0f;
+#pragma unroll
+                    for (int a = 0; a < 3; ++a) {
+                        xs[f][a] = X[(int64_t)j * 3 + a];
+                        ys[f][a] = Y[(ok ? mj[f] : 0) * 3 + a];
+                    }
+                }
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    const int p = p0 + f * NT;
+                    if (p >= j1 - j0)
+                        continue;
+                    const bool ok = mj[f] >= 0 && mj[f] < ny;
+#pragma unroll
+                    for (int a = 0; a < 3; ++a) {
+                        const float own = ok ? gg[f] * (xs[f][a] - ys[f][a]) : 0.0f;
+                        const float sent =
+                            (float)__builtin_ldexp((double)(long long)acc[p * 3 + a], -kexp);
+                        out[(int64_t)(j0 + p) * 3 + a] = own + sent;
+                    }
+                }
+            }
+            TK3D_STAMP(3 + attempt * 4);
+            return;
+        }
+    }
+    (void)use_float;
+
+    // Non-finite gradients or coordinates: floating-point LDS accumulation.
+    float *facc = reinterpret_cast<float *>(acc);
+    __syncthreads();
+    for (int t = threadIdx.x; t < R * 3; t += NT)
+        facc[t] = 0.0f;
+    __syncthreads();
+    for (int i = threadIdx.x; i < ny; i += NT) {
+        const int64_t j = iY[i];
+        if (j < j0 || j >= j1)
+            continue;
+        const float g = gY[i] * 2;
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+            atomicAdd(&facc[(j - j0) * 3 + a], -(g * (Y[(int64_t)i * 3 + a] - X[j * 3 + a])));
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < (j1 - j0) * 3; t += NT) {
+        const int j = j0 + t / 3, a = t - (t / 3) * 3;
+        const int64_t jj = iX[j];
+        float own = 0.0f;
+        if (jj >= 0 && jj < ny)
+            own = (gX[j] * 2) * (X[(int64_t)j * 3 + a] - Y[jj * 3 + a]);
+        out[(int64_t)j * 3 + a] = own + facc[t];
+    }
+}
+
 template <typename T, int QPL, int BLOCK = 256, int TILE = 32, int STAGE = 1024>
 int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
                            int64_t N2, T *dist1, int64_t *idx1, T *dist2,
@@ -764,6 +997,29 @@ int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
     if (t1 + t2 == 0)
         return TK3D_OK;
     hipStream_t s = (hipStream_t)stream;
+    if constexpr (sizeof(T) == 4) {
+        // Every range scans all senders of its batch, so ranges are as long as LDS
+        // allows: 4096 points x 3 x 8 bytes = 96 KiB.
+        constexpr int R = 4096, NT = 1024;
+        const int64_t r1 = (N1 + R - 1) / R, r2 = (N2 + R - 1) / R;
+        if (B * (r1 + r2) <= TK_MAX_I32) {
+            auto kernel = chamfer_backward_fixed_kernel<R, NT>;
+            constexpr size_t lds = (size_t)R * 3 * sizeof(unsigned long long);
+            static bool lds_opt_in = false;  // raising the limit is idempotent
+            if (!lds_opt_in) {
+                const hipError_t e = hipFuncSetAttribute(
+                    reinterpret_cast<const void *>(kernel),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (e != hipSuccess)
+                    return (int)e;
+                lds_opt_in = true;
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(B * (r1 + r2))), dim3(NT), lds, s, gd1,
+                               gd2, xyz1, xyz2, idx1, idx2, (int)N1, (int)N2, (int)r1, (int)r2,
+                               (int)(B * r1), gx1, gx2);
+            return tk_launch_status();
+        }
+    }
     int64_t blocks = (t1 + t2 + 255) / 256;
     if (blocks > 65536)
         blocks = 65536;
