@@ -187,14 +187,19 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
 //
 // d2(q,k) = s + |q'|^2 up to rounding. For one query the additive |q'|^2 is common to
 // all keys, so minima of s locate minima of d2 up to the rounding error of both
-// expressions. With u = 2^-24:
-//     |canonical d2 - true d2|  <= 5.01 u d2                (3 rounded differences,
-//                                                            1 product, 2 fmas)
-//     |s + |q'|^2 - true d2|    <= 8.1 u (|k'|+|q'|)^2      (centring 2 u, |k'|^2 3 u,
-//                                                            3 fmas 3 u)
-// hence |s + |q'|^2 - canonical d2| <= E = 13.2 u R, R = (max|k'| + |q'|)^2, and any
+// expressions. With u = 2^-24, rho = |k'| + |q'| and d the true distance:
+//     canonical d2: three rounded differences, one product, two fmas, all terms
+//         non-negative                      |canonical - d^2| <= 5.01 u d^2 <= 5.01 u rho^2
+//     centring: k' and q' carry one rounding each, so k'-q' is off by at most
+//         u rho and its squared norm by     2.01 u rho^2
+//     |k'|^2: three non-negative rounded terms                   3 u |k'|^2
+//     the three fmas of s: each rounds a partial sum of magnitude at most rho^2
+//                                                                3.01 u rho^2
+// hence |s + |q'|^2 - canonical d2| <= E = 13.1 u R with R = (max|k'| + |q'|)^2, and any
 // key whose canonical distance equals the minimum has s <= min(s) + 2E. The kernel
-// uses slack = 64 u R (> 2E plus the rounding of the comparison itself).
+// compares against min(s) + slack with slack = 32 u R: 26.2 u R for 2E, 1 u R for the
+// rounding of that sum, the rest margin (max|k'| and |q'| are inflated by 1e-6 to
+// cover their own rounding; 1e-37 is added against underflow).
 //
 // Sweep: per tile of TILE keys only min(s) is formed (3 fma + half a min3 per
 // pair), and each query keeps the three smallest tile minima v0<=v1<=v2 with the
