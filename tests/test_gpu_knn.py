@@ -59,7 +59,9 @@ def test_interpolation_config_fp32(cuda, k):
 @pytest.mark.parametrize("b,n1,n2,k", [(2, 300, 2048, 1), (2, 100, 500, 4), (2, 77, 130, 5),
                                         (2, 100, 500, 8), (1, 200, 3000, 17), (2, 100, 500, 64),
                                         (1, 50, 300, 100), (2, 33, 40, 40), (2, 10, 5, 5),
-                                        (1, 1000, 1025, 33)])
+                                        (1, 1000, 1025, 33), (2, 300, 1000, 65),
+                                        (2, 200, 700, 128), (1, 100, 400, 129),
+                                        (4, 1000, 4096, 32)])
 def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
     g = gen(k)
     q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
@@ -70,8 +72,24 @@ def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
 def test_lattice_ties_follow_mink_eviction_order(cuda):
     g = gen(9)
     q, key = lattice_cloud(g, 2, 400, 4), lattice_cloud(g, 2, 1500, 4)
-    for k in (3, 6, 16, 33):
+    for k in (3, 6, 16, 33, 64, 100):
         check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("k", [3, 8, 16, 24, 64])
+def test_non_finite_keys_follow_mink(cuda, k):
+    # MinK compares with '<' and '>' only: a NaN distance taken during the fill is never
+    # the maximum unless it sits in slot 0, where it blocks every later insertion; an
+    # infinite distance is an ordinary large value.
+    g = gen(11)
+    q, key = uniform_cloud(g, 4, 200), uniform_cloud(g, 4, 600)
+    key[0, 0, 1] = float("nan")        # slot 0 of every query in cloud 0
+    key[1, 2, 0] = float("nan")        # a later fill slot
+    key[1, 300, 2] = float("nan")      # beyond the fill: never inserted
+    key[2, 1, 0] = float("inf")        # infinite distance inside the fill
+    key[2, 400, 1] = -float("inf")
+    key[3, 0, 0] = float("inf")
+    check_raw(q, key, k, cuda)
 
 
 def test_k1_equals_chamfer_argmin(cuda):

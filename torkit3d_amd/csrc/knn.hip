@@ -127,6 +127,11 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
 // largest number of candidates any lane has, instead of the number of distinct
 // candidate keys across all lanes. The sequence of insertions seen by one lane is
 // exactly MinK's, so the slot order is unchanged.
+#ifdef TK3D_KNN_STATS
+__device__ unsigned long long knn_stats[1 << 16];  // per wave: t0, t1, sweep cycles, rounds
+#define KNN_CLOCK() __builtin_readcyclecounter()
+#endif
+
 template <int KMAX>
 __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
@@ -134,6 +139,7 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     int n2, int k)
 {
     constexpr int CHUNK = 32;
+    static_assert(KNN_STAGE % CHUNK == 0, "a chunk must not straddle stages");
     __shared__ __align__(16) float skey[KNN_STAGE * 4];
     const int tid = threadIdx.x;
     const int b = blockIdx.x / blocks_per_batch;
@@ -152,6 +158,7 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     int ki[KMAX];
     float max_key = 0.0f;
     int max_idx = 0;
+    bool fill_nan = false;
     // Fill phase: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots stay at
     // -inf so the rescan never selects them.
 #pragma unroll
@@ -162,12 +169,22 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             const float d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
             kd[s] = d;
             ki[s] = s;
+            fill_nan |= d != d;
             if (s == 0 || d > max_key) {
                 max_key = d;
                 max_idx = s;
             }
         }
     }
+    // The rescan below orders the slots by their bit patterns, which is the float order
+    // for everything a squared distance can be except NaN. A NaN can only enter during
+    // the fill (later keys must compare below the maximum); a wave that has one rescans
+    // with float compares instead.
+    const bool float_rescan = __builtin_amdgcn_ballot_w64(fill_nan) != 0;
+#ifdef TK3D_KNN_STATS
+    const unsigned long long st_t0 = KNN_CLOCK();
+    unsigned long long st_sweep = 0, st_rounds = 0;
+#endif
 
     for (int stage0 = 0; stage0 < n2; stage0 += KNN_STAGE) {
         __syncthreads();
@@ -187,31 +204,58 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
         for (int c0 = 0; c0 < cnt; c0 += CHUNK) {
             // ---- sweep: bit (31 - i) of `mask` <=> key c0+i is below the maximum ----
             const int maxbits = __builtin_bit_cast(int, max_key);
-            unsigned mask = 0u;
             const float4 *ck = reinterpret_cast<const float4 *>(skey) + c0;
+            const int first = stage0 + c0;  // global index of bit 31
+#ifdef TK3D_KNN_STATS
+            const unsigned long long st_a = KNN_CLOCK();
+#endif
+            unsigned mask = 0u;
+            if (c0 + CHUNK <= cnt) {
+                // A full chunk comes straight from global memory: the addresses are the
+                // same for the whole wave, so the loads are scalar and the coordinates are
+                // scalar operands of the vector arithmetic - no LDS traffic in the sweep.
+                const float *__restrict__ g = K + (int64_t)first * 3;
 #pragma unroll
-            for (int i = 0; i < CHUNK; ++i) {
-                const float4 e = ck[i];
-                const float d = tk_dist2<float>(e.x, e.y, e.z, qx, qy, qz);
-                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
-                mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | (diff >> 31)
+                for (int i = 0; i < CHUNK; ++i) {
+                    const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2],
+                                                    qx, qy, qz);
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
+                }
+            } else {
+#pragma unroll 4
+                for (int i = 0; i < CHUNK; ++i) {
+                    const float4 e = ck[i];  // zero padding beyond the last key
+                    const float d = tk_dist2<float>(e.x, e.y, e.z, qx, qy, qz);
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                }
             }
-            // Keys that do not exist, or that the fill phase already took, are no candidates.
-            const int first = stage0 + c0;               // global index of bit 31
-            int lo = k - first;                          // keys below k were used for filling
+            // Keys that do not exist, or that the fill phase took, are no candidates.
+            int lo = k - first;                          // keys below k filled the slots
             lo = lo < 0 ? 0 : (lo > CHUNK ? CHUNK : lo);
             int hi = cnt - c0;                           // keys at or beyond hi are padding
             hi = hi > CHUNK ? CHUNK : hi;
             unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
             valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
             mask &= valid;
+#ifdef TK3D_KNN_STATS
+            st_sweep += KNN_CLOCK() - st_a;
+#endif
 
-            // ---- insertion rounds ----
-            while (__builtin_amdgcn_ballot_w64(mask != 0u)) {  // wave-uniform
-                const bool has = mask != 0u;
-                const int i = has ? __builtin_clz(mask) : 0;
-                mask &= ~(0x80000000u >> i);
-                const float4 e = ck[i];
+            // ---- insertion rounds; the next candidate's key is fetched from LDS while the
+            // current one is inserted ----
+            bool has = mask != 0u;
+            int i = has ? __builtin_clz(mask) : 0;
+            float4 e = ck[i];
+            while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+#ifdef TK3D_KNN_STATS
+                ++st_rounds;
+#endif
+                mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
+                const bool has_next = mask != 0u;
+                const int i_next = has_next ? __builtin_clz(mask) : 0;
+                const float4 e_next = ck[i_next];
                 const float d = tk_dist2<float>(e.x, e.y, e.z, qx, qy, qz);
                 if (has && d < max_key) {
                     const int kj = first + i;
@@ -221,18 +265,78 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
                         kd[s] = here ? d : kd[s];
                         ki[s] = here ? kj : ki[s];
                     }
-                    max_key = d;
+                    if (float_rescan) {
+                        max_key = d;
 #pragma unroll
-                    for (int s = 0; s < KMAX; ++s) {
-                        const bool up = kd[s] > max_key;
-                        max_key = up ? kd[s] : max_key;
-                        max_idx = up ? s : max_idx;
+                        for (int s = 0; s < KMAX; ++s) {
+                            const bool up = kd[s] > max_key;
+                            max_key = up ? kd[s] : max_key;
+                            max_idx = up ? s : max_idx;
+                        }
+                    } else {
+                        // New maximum = largest bit pattern. MinK starts its rescan from the
+                        // inserted key, so the maximum stays in the inserted slot when nothing
+                        // is strictly above it; otherwise it is the first slot that holds the
+                        // largest pattern: (top - 1 - bits) is negative exactly there, and
+                        // the sign bits shifted together put slot 0 in the highest position.
+                        // Both steps are written as short independent chains: with few waves
+                        // per SIMD the round is bound by its dependent latency.
+                        int t[KMAX];
+#pragma unroll
+                        for (int s = 0; s < KMAX; ++s)
+                            t[s] = __builtin_bit_cast(int, kd[s]);
+#pragma unroll
+                        for (int n = KMAX; n > 1; n = (n + 2) / 3) {
+#pragma unroll
+                            for (int j = 0; 3 * j < n; ++j) {
+                                int v = t[3 * j];
+                                if (3 * j + 1 < n)
+                                    v = t[3 * j + 1] > v ? t[3 * j + 1] : v;
+                                if (3 * j + 2 < n)
+                                    v = t[3 * j + 2] > v ? t[3 * j + 2] : v;
+                                t[j] = v;
+                            }
+                        }
+                        const int top = t[0];
+                        const unsigned below = (unsigned)top - 1u;
+                        constexpr int GS = KMAX <= 16 ? 4 : 8;  // slots per independent chain
+                        unsigned eq[(KMAX + 31) / 32] = {};
+#pragma unroll
+                        for (int g0 = 0; g0 < KMAX; g0 += GS) {
+                            unsigned part = 0u;
+#pragma unroll
+                            for (int s = g0; s < g0 + GS; ++s)
+                                part = __builtin_amdgcn_alignbit(
+                                    part, below - __builtin_bit_cast(unsigned, kd[s]), 31);
+                            eq[g0 / 32] = (eq[g0 / 32] << GS) | part;
+                        }
+                        max_key = __builtin_bit_cast(float, top);
+                        int first_top;
+                        if constexpr (KMAX <= 32)
+                            first_top = __builtin_clz(eq[0]) - (32 - KMAX);
+                        else
+                            first_top = eq[0] ? __builtin_clz(eq[0]) : 32 + __builtin_clz(eq[1]);
+                        max_idx = top != __builtin_bit_cast(int, d) ? first_top : max_idx;
                     }
                 }
+                has = has_next;
+                i = i_next;
+                e = e_next;
             }
         }
     }
 
+#ifdef TK3D_KNN_STATS
+    if ((tid & 63) == 0) {
+        const unsigned wv = (blockIdx.x * (KNN_BLOCK / 64) + (tid >> 6)) & 0x3fff;
+        unsigned hw;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+        knn_stats[wv * 4 + 0] = st_t0;
+        knn_stats[wv * 4 + 1] = KNN_CLOCK();
+        knn_stats[wv * 4 + 2] = st_sweep;
+        knn_stats[wv * 4 + 3] = (st_rounds << 32) | hw;
+    }
+#endif
     if (active) {
         float *od = distance + ((int64_t)b * n1 + qi) * k;
         int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
@@ -244,6 +348,235 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             }
         }
     }
+}
+
+// fp32 variant for larger k: the slots live in LDS as a per-lane tournament tree.
+//
+// With the slots in registers every insertion pays O(k) selects and compares, because
+// registers cannot be indexed per lane. LDS can: a lane keeps, in columns of its own
+// (row r of an array at [r * 64 + lane], conflict-free whatever r each lane uses),
+//   leaf[s]  distance in slot s           kidx[s]  key index in slot s
+//   ival[n]  largest distance below node n of a binary tree over the slots (heap
+//            numbering, node 1 the root, the leaves of slot s at KMAX + s)
+//   iarg[n]  the first slot that holds ival[n]
+// An insertion overwrites the leaf of the current maximum and replays the log2(KMAX)
+// matches on the way to the root. The other side of each of those matches is known up
+// front, so all of them are fetched at once and the path costs one LDS round trip plus
+// three vector instructions per level. A right child wins a match only when strictly
+// greater, so a node reports the first slot holding its maximum - MinK's rescan order
+// (mink.cuh:74-87); MinK starts that rescan from the inserted key, hence the maximum
+// stays in the inserted slot when the root is not strictly above it.
+//
+// The sweep takes its keys through scalar loads (the address is the same for every
+// lane) and the rounds fetch their candidates straight from global memory, one round
+// ahead; a block is one wave and never synchronises.
+//
+// NaN distances can only enter during the fill (a later key must compare below the
+// maximum). MinK never selects such a slot as maximum unless it is slot 0, in which
+// case it never inserts again. Here a NaN in slot 0 freezes the lane; a NaN elsewhere
+// plays the tournament as -inf and is recomputed when the results are written.
+template <int KMAX>
+__global__ __launch_bounds__(64) void knn_tree_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
+    int n2, int k)
+{
+    constexpr int CHUNK = 32;
+    constexpr int NT = 64;
+    constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : KMAX == 64 ? 6 : 7;
+    static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 128");
+    extern __shared__ __align__(16) unsigned char knn_tree_lds[];
+    const int lane = threadIdx.x;
+    float *const leaf = reinterpret_cast<float *>(knn_tree_lds) + lane;
+    int *const kidx = reinterpret_cast<int *>(knn_tree_lds) + KMAX * NT + lane;
+    float *const ival = reinterpret_cast<float *>(knn_tree_lds) + 2 * KMAX * NT + lane;
+    unsigned char *const iarg = knn_tree_lds + 12 * KMAX * NT + lane;
+
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
+    const bool active = qi < n1;
+    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
+    float qx = 0, qy = 0, qz = 0;
+    if (active) {
+        const float *q = query + ((int64_t)b * n1 + qi) * 3;
+        qx = q[0];
+        qy = q[1];
+        qz = q[2];
+    }
+
+    // Fill phase: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots hold -inf.
+    bool frozen = false;
+    for (int s = 0; s < KMAX; ++s) {
+        float d = -__builtin_huge_valf();
+        if (s < k) {
+            d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            if (d != d) {
+                frozen |= s == 0;
+                d = -__builtin_huge_valf();  // marks the slot: no real distance is -inf
+            }
+        }
+        leaf[s * NT] = d;
+        kidx[s * NT] = s;
+    }
+    for (int n = KMAX - 1; n >= 1; --n) {
+        const int l = 2 * n, r = 2 * n + 1;
+        float lv, rv;
+        int la, ra;
+        if (l >= KMAX) {
+            lv = leaf[(l - KMAX) * NT];
+            rv = leaf[(r - KMAX) * NT];
+            la = l - KMAX;
+            ra = r - KMAX;
+        } else {
+            lv = ival[l * NT];
+            rv = ival[r * NT];
+            la = iarg[l * NT];
+            ra = iarg[r * NT];
+        }
+        const bool right = rv > lv;
+        ival[n * NT] = right ? rv : lv;
+        iarg[n * NT] = (unsigned char)(right ? ra : la);
+    }
+    float max_key = frozen ? -__builtin_huge_valf() : ival[NT];
+    int max_idx = iarg[NT];
+
+#ifdef TK3D_KNN_STATS
+    const unsigned long long st_t0 = KNN_CLOCK();
+    unsigned long long st_sweep = 0, st_rounds = 0;
+#endif
+    for (int first = 0; first < n2; first += CHUNK) {  // `first` = key index of bit 31
+        // ---- sweep: bit (31 - i) of `mask` <=> key first+i is below the maximum ----
+        const int maxbits = __builtin_bit_cast(int, max_key);
+#ifdef TK3D_KNN_STATS
+        const unsigned long long st_a = KNN_CLOCK();
+#endif
+        unsigned mask = 0u;
+        if (first + CHUNK <= n2) {
+            const float *__restrict__ g = K + (int64_t)first * 3;
+#pragma unroll
+            for (int i = 0; i < CHUNK; ++i) {
+                const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
+                                                qy, qz);
+                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
+            }
+        } else {
+            for (int i = 0; i < CHUNK; ++i) {
+                const int j = first + i < n2 ? first + i : n2 - 1;  // clamped, masked below
+                const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
+                                                K[(int64_t)j * 3 + 2], qx, qy, qz);
+                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+            }
+        }
+        // Keys that do not exist, or that the fill phase took, are no candidates.
+        int lo = k - first;                          // keys below k filled the slots
+        lo = lo < 0 ? 0 : (lo > CHUNK ? CHUNK : lo);
+        int hi = n2 - first;                         // keys at or beyond hi do not exist
+        hi = hi > CHUNK ? CHUNK : hi;
+        unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
+        valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
+        mask &= valid;
+#ifdef TK3D_KNN_STATS
+        st_sweep += KNN_CLOCK() - st_a;
+#endif
+
+        // ---- insertion rounds, the next candidate's key in flight during the current ----
+        const float *__restrict__ ck = K + (int64_t)first * 3;
+        bool has = mask != 0u;
+        int i = has ? __builtin_clz(mask) : 0;
+        float ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
+        while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+#ifdef TK3D_KNN_STATS
+            ++st_rounds;
+#endif
+            mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
+            const bool has_next = mask != 0u;
+            const int i_next = has_next ? __builtin_clz(mask) : 0;
+            const float nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
+                        nz = ck[3 * i_next + 2];
+            const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+            if (has && d < max_key) {
+                const int p = max_idx;
+                leaf[p * NT] = d;
+                kidx[p * NT] = first + i;
+                float sv[LEVELS];
+                int sa[LEVELS];
+                sv[0] = leaf[(p ^ 1) * NT];
+                sa[0] = p ^ 1;
+#pragma unroll
+                for (int l = 1; l < LEVELS; ++l) {
+                    const int sib = ((KMAX + p) >> l) ^ 1;
+                    sv[l] = ival[sib * NT];
+                    sa[l] = iarg[sib * NT];
+                }
+                float v = d;
+                int a = p;
+#pragma unroll
+                for (int l = 0; l < LEVELS; ++l) {
+                    const int node = (KMAX + p) >> l;
+                    // the other side wins from the right only when strictly greater
+                    const bool take = (node & 1) ? !(v > sv[l]) : (sv[l] > v);
+                    v = take ? sv[l] : v;
+                    a = take ? sa[l] : a;
+                    if (l + 1 < LEVELS) {  // the root lives in max_key / max_idx
+                        ival[(node >> 1) * NT] = v;
+                        iarg[(node >> 1) * NT] = (unsigned char)a;
+                    }
+                }
+                max_key = v;
+                max_idx = v != d ? a : p;
+            }
+            has = has_next;
+            i = i_next;
+            ex = nx;
+            ey = ny;
+            ez = nz;
+        }
+    }
+
+#ifdef TK3D_KNN_STATS
+    if (lane == 0) {
+        const unsigned wv = blockIdx.x & 0x3fff;
+        knn_stats[wv * 4 + 0] = st_t0;
+        knn_stats[wv * 4 + 1] = KNN_CLOCK();
+        knn_stats[wv * 4 + 2] = st_sweep;
+        knn_stats[wv * 4 + 3] = st_rounds << 32;
+    }
+#endif
+    if (active) {
+        float *od = distance + ((int64_t)b * n1 + qi) * k;
+        int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
+        for (int s = 0; s < k; ++s) {
+            float d = leaf[s * NT];
+            if (d == -__builtin_huge_valf())  // a NaN of the fill phase, still in its slot
+                d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            od[s] = d;
+            oi[s] = (int64_t)kidx[s * NT];
+        }
+    }
+}
+
+template <int KMAX>
+int knn_tree_launch(const float *query, const float *key, float *distance, int64_t *index,
+                    int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    constexpr int LDS_BYTES = 13 * KMAX * 64;
+    static bool raised = false;  // per process; the attribute is sticky
+    if (LDS_BYTES > 48 * 1024 && !raised) {
+        const hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&knn_tree_kernel_f32<KMAX>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess)
+            return (int)e;
+        raised = true;
+    }
+    const int64_t bpb = ((int64_t)n1 + 63) / 64;
+    if (B * bpb > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((knn_tree_kernel_f32<KMAX>), dim3((unsigned)(B * bpb)), dim3(64),
+                       LDS_BYTES, s, query, key, distance, index, (int)bpb, n1, n2, k);
+    return tk_launch_status();
 }
 
 // Any k: the structure lives in the output rows in global memory.
@@ -360,13 +693,26 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
     else if (k <= 16)
         knn_launch<T, 16>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else if (k <= 32)
-        knn_launch<T, 32>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else if (k <= 64)
-        knn_launch<T, 64>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else
+    else if constexpr (sizeof(T) == 4) {
+        // fp32: slots in LDS as a tournament tree up to k = 128
+        if (k <= 32)
+            return knn_tree_launch<32>(query, key, distance, index, B, n1, n2, kk, s);
+        if (k <= 64)
+            return knn_tree_launch<64>(query, key, distance, index, B, n1, n2, kk, s);
+        if (k <= 128)
+            return knn_tree_launch<128>(query, key, distance, index, B, n1, n2, kk, s);
         hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)), dim3(KNN_BLOCK),
                            0, s, query, key, distance, index, (int)bpb, n1, n2, kk);
+    } else {
+        if (k <= 32)
+            knn_launch<T, 32>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+        else if (k <= 64)
+            knn_launch<T, 64>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+        else
+            hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)),
+                               dim3(KNN_BLOCK), 0, s, query, key, distance, index, (int)bpb,
+                               n1, n2, kk);
+    }
     return tk_launch_status();
 }
 
