@@ -768,7 +768,13 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
                 }
             }
         }
-        if (m != 0u)
+        // one LDS atomic per wave: 64 lanes on one address would be served one by one
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned t = (unsigned)__shfl_xor((int)m, o);
+            m = t > m ? t : m;
+        }
+        if ((threadIdx.x & 63) == 0 && m != 0u)
             atomicMax(&s_max, m);
         __syncthreads();
         TK3D_STAMP(1 + attempt * 4);

@@ -301,9 +301,9 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
 // atomics run at the rate of a plain LDS write, 13 times faster. So each
 // contribution g*w (rounded to fp32 as the reference rounds it) is converted to an
 // integer at a per-row power-of-two scale and added with ds_add_u64:
-//   * magnitudes: the workgroup samples one 16-byte group in eight of its share of
-//     gout for max|g| per row (and reads all of w for max|w|), and allows 64 times
-//     that as the bound B_c of a row;
+//   * magnitudes: the workgroup samples an eighth of its share of gout for max|g| per
+//     row and an eighth of w for max|w| (runs of 64 consecutive loads, one run in
+//     eight), and allows 64 times their product as the bound B_c of a row;
 //   * scale: 2^k with k the largest integer keeping B_c * 2^k below 2^50 and
 //     count * B_c * 2^k below 2^62, i.e. a resolution of 2^-40 of the row maximum
 //     or better for up to 2^16 terms per row; fp32 accumulation resolves 2^-24;
@@ -314,6 +314,26 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
 // Integer addition is associative, so unlike the reference the result does not
 // depend on the order in which the contributions arrive. A row holding NaN or inf
 // has no usable scale; the workgroup then takes the floating-point path.
+// Largest value of a wave, in every lane. Called by whole waves only.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned t = (unsigned)__shfl_xor((int)v, o);
+        v = t > v ? t : v;
+    }
+    return v;
+}
+
+#ifdef TK3D_SCATTER_STATS
+__device__ unsigned long long scatter_stats[1 << 16];
+#define SC_STAMP(i)                                                                      \
+    if (threadIdx.x == 0)                                                                \
+    scatter_stats[((blockIdx.z * gridDim.y + blockIdx.y) & 0x1fff) * 8 + (i)] = __builtin_readcyclecounter()
+#else
+#define SC_STAMP(i)
+#endif
+
 template <int KK, bool HAS_W, int V, int NT, int CGMAX>
 __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     const float *__restrict__ gout, const int64_t *__restrict__ idx,
@@ -335,20 +355,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
 
-    if (threadIdx.x == 0)
-        s_maxw = HAS_W ? 0u : 0x3f800000u;
-    if (HAS_W) {
-        __syncthreads();
-        unsigned mw = 0u;
-        for (int64_t e = ps * KK + threadIdx.x; e < pe * KK; e += NT) {
-            const unsigned bits =
-                __builtin_bit_cast(unsigned, w[(int64_t)b * np * KK + e]) & 0x7fffffffu;
-            mw = bits > mw ? bits : mw;
-        }
-        if (mw != 0u)
-            atomicMax(&s_maxw, mw);
-    }
-
+    SC_STAMP(0);
     for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
         __syncthreads();
         for (int i = threadIdx.x; i < nc * n1; i += NT)
@@ -358,17 +365,40 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         if (threadIdx.x == 0) {
             s_finite = 1;
             s_exceeded = 0;
+            s_maxw = HAS_W ? 0u : 0x3f800000u;
         }
         __syncthreads();
+        SC_STAMP(1);
 
         // ---- magnitudes: every 8th group first, everything on the second attempt ----
+        if (HAS_W) {
+            // first attempt: one run of 64 consecutive weights in every 512
+            unsigned mw = 0u;
+            const int64_t ne = (pe - ps) * KK;
+            for (int64_t t = threadIdx.x;; t += NT) {
+                const int64_t e = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
+                if (e >= ne)
+                    break;
+                const unsigned bits =
+                    __builtin_bit_cast(unsigned, w[((int64_t)b * np + ps) * KK + e]) & 0x7fffffffu;
+                mw = bits > mw ? bits : mw;
+            }
+            // one LDS atomic per wave: 64 lanes on one address would be served one by one
+            mw = wave_max_u32(mw);
+            if ((threadIdx.x & 63) == 0 && mw != 0u)
+                atomicMax(&s_maxw, mw);
+        }
         {
-            const int64_t stride = (int64_t)NT * V * (attempt == 0 ? 8 : 1);
+            // first attempt: one run of 64 consecutive 16-byte groups in every 512
             unsigned mg[CGMAX];
 #pragma unroll
             for (int c = 0; c < CGMAX; ++c)
                 mg[c] = 0u;
-            for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += stride) {
+            for (int64_t t = threadIdx.x;; t += NT) {
+                const int64_t gi = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
+                const int64_t p0 = ps + gi * V;
+                if (p0 >= pe)
+                    break;
                 const bool full = (p0 + V <= pe);
 #pragma unroll
                 for (int c = 0; c < CGMAX; ++c) {
@@ -395,11 +425,16 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                 }
             }
 #pragma unroll
-            for (int c = 0; c < CGMAX; ++c)
-                if (c < nc && mg[c] != 0u)
-                    atomicMax(&s_maxg[c], mg[c]);
+            for (int c = 0; c < CGMAX; ++c) {
+                if (c >= nc)  // uniform
+                    break;
+                const unsigned m = wave_max_u32(mg[c]);
+                if ((threadIdx.x & 63) == 0 && m != 0u)
+                    atomicMax(&s_maxg[c], m);
+            }
         }
         __syncthreads();
+        SC_STAMP(2);
 
         // ---- bounds and scales: lane c < CGMAX works out row c ----
         if (threadIdx.x < CGMAX) {
@@ -420,6 +455,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         if (!s_finite)
             break;
 
+        SC_STAMP(3);
         struct RowScale {
             double scale;
             float bound;
@@ -443,7 +479,9 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             });
         if (exceeded)
             s_exceeded = 1;
+        SC_STAMP(4);
         __syncthreads();
+        SC_STAMP(5);
         if (!s_exceeded) {
             float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
             for (int i = threadIdx.x; i < nc * n1; i += NT) {
@@ -456,6 +494,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                     dstrows[i] = v;
                 }
             }
+            SC_STAMP(6);
             return;
         }
     }
