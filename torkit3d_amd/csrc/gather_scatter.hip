@@ -105,10 +105,25 @@ __global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
     }
 }
 
+#ifdef TK3D_GATHER_STATS
+__device__ unsigned long long gather_stats[1 << 16];
+#define GA_STAMP(i)                                                                      \
+    if (threadIdx.x == 0)                                                                \
+    gather_stats[((blockIdx.z * gridDim.y + blockIdx.y) & 0x1fff) * 8 + (i)] = __builtin_readcyclecounter()
+#else
+#define GA_STAMP(i)
+#endif
+
 // Same gather with the source rows staged in LDS. Row gathers through the vector
 // cache cost one cache line per lane (64 lanes -> 64 lines per load instruction),
 // which caps the plain kernel near 2 TB/s of output; LDS serves the same random
 // reads at bank rate. grid = (point chunks, channel groups, B); LDS = cg*n1 elements.
+//
+// A wave covers 64*V consecutive points and lane l takes points l, l+64, ... of that
+// span: every index, weight and output access of the wave is then a run of
+// consecutive elements (indices: 24-byte stride for three neighbours), instead of
+// each lane walking its own 96 bytes of the index array, which costs the vector
+// cache one line lookup per lane and load.
 template <typename T, int KK, bool HAS_W, int V, int NT>
 __global__ __launch_bounds__(NT) void gather_lds_kernel(
     const T *__restrict__ in, const int64_t *__restrict__ idx, const T *__restrict__ w,
@@ -120,70 +135,92 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
     const int c0 = blockIdx.y * cg;
     const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
     const T *__restrict__ src_rows = in + ((int64_t)b * c_total + c0) * n1;
-    for (int i = threadIdx.x; i < nc * n1; i += NT)
-        rows[i] = src_rows[i];
-    __syncthreads();
-
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
     const int64_t ps = (int64_t)blockIdx.x * chunk_len;
     const int64_t pe = (ps + chunk_len < np) ? ps + chunk_len : np;
-    for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += (int64_t)NT * V) {
+
+    // Indices and weights are fetched one iteration ahead (the first set while the rows
+    // are staged) and only decoded when their iteration starts.
+    int64_t jn[V][KK];
+    T wn[V][KK];
+    auto fetch = [&](int64_t p0) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+#pragma unroll
+            for (int i = 0; i < KK; ++i) {
+                const int64_t p = p0 + v * 64;
+                jn[v][i] = -1;
+                wn[v][i] = (T)0;
+                if (p < pe) {
+                    jn[v][i] = idx[((int64_t)b * np + p) * KK + i];
+                    if (HAS_W)
+                        wn[v][i] = w[((int64_t)b * np + p) * KK + i];
+                }
+            }
+        }
+    };
+    const int64_t pfirst = ps + (int64_t)wave * (64 * V) + lane;
+    fetch(pfirst);
+
+    GA_STAMP(0);
+    {
+        // the staged rows are contiguous in global memory: 16-byte copies when aligned
+        constexpr int E = 16 / (int)sizeof(T);
+        const int total = nc * n1;
+        const bool wide = ((uintptr_t)src_rows & 15) == 0;
+        const int nwide = wide ? total / E : 0;
+        const float4 *__restrict__ s4 = reinterpret_cast<const float4 *>(src_rows);
+        float4 *d4 = reinterpret_cast<float4 *>(rows);
+#pragma unroll 4
+        for (int i = threadIdx.x; i < nwide; i += NT)
+            d4[i] = s4[i];
+        for (int i = nwide * E + threadIdx.x; i < total; i += NT)
+            rows[i] = src_rows[i];
+    }
+    GA_STAMP(1);
+    __syncthreads();
+    GA_STAMP(2);
+
+    for (int64_t p0 = pfirst; p0 < pe; p0 += (int64_t)NT * V) {
         int src[V][KK];
         T wt[V][KK];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
 #pragma unroll
             for (int i = 0; i < KK; ++i) {
-                const int64_t p = p0 + v;
-                int64_t j = -1;
-                T ww = (T)0;
-                if (p < pe) {
-                    j = idx[((int64_t)b * np + p) * KK + i];
-                    if (HAS_W)
-                        ww = w[((int64_t)b * np + p) * KK + i];
-                }
+                const int64_t j = jn[v][i];
                 src[v][i] = (j >= 0 && j < n1) ? (int)j : -1;
-                wt[v][i] = ww;
+                wt[v][i] = wn[v][i];
             }
         }
-        const bool full = (p0 + V <= pe);
+        if (p0 + (int64_t)NT * V < pe)
+            fetch(p0 + (int64_t)NT * V);
 #pragma unroll 4
         for (int c = 0; c < nc; ++c) {
             const T *row = rows + c * n1;
             T *__restrict__ orow = out + ((int64_t)b * c_total + c0 + c) * np;
-            T val[V];
 #pragma unroll
             for (int v = 0; v < V; ++v) {
+                T val;
                 if (HAS_W) {
+                    // out = 0; out = fma(in, w, out) per neighbour, in slot order
+                    // (interpolate_kernel.cu:31-42 under default contraction).
                     T acc = (T)0;
 #pragma unroll
                     for (int i = 0; i < KK; ++i)
                         if (src[v][i] >= 0)
                             acc = tk_fma<T>(row[src[v][i]], wt[v][i], acc);
-                    val[v] = acc;
+                    val = acc;
                 } else {
-                    val[v] = src[v][0] >= 0 ? row[src[v][0]] : (T)0;
+                    val = src[v][0] >= 0 ? row[src[v][0]] : (T)0;
                 }
-            }
-            if (full && vec_ok && V == 4 && sizeof(T) == 4) {
-                float4 pack;
-                pack.x = (float)val[0];
-                pack.y = (float)val[1 % V];
-                pack.z = (float)val[2 % V];
-                pack.w = (float)val[3 % V];
-                *reinterpret_cast<float4 *>(orow + p0) = pack;
-            } else if (full && vec_ok && V == 2 && sizeof(T) == 8) {
-                double2 pack;
-                pack.x = (double)val[0];
-                pack.y = (double)val[1 % V];
-                *reinterpret_cast<double2 *>(orow + p0) = pack;
-            } else {
-#pragma unroll
-                for (int v = 0; v < V; ++v)
-                    if (p0 + v < pe)
-                        orow[p0 + v] = val[v];
+                if (p0 + v * 64 < pe)
+                    __builtin_nontemporal_store(val, &orow[p0 + v * 64]);
             }
         }
     }
+    GA_STAMP(3);
 }
 
 // ---- scatter ---------------------------------------------------------------------
@@ -198,9 +235,8 @@ __global__ __launch_bounds__(GS_BLOCK) void fill_zero_kernel(T *__restrict__ p, 
 
 // Streams the points [ps, pe) of one batch for `nc` channels starting at c0 and hands
 // every contribution to `sink(ctx, c, dst, value, weight)`, where `ctx = prep(c)` is
-// evaluated once per channel and lane iteration. A lane takes V consecutive
-// points so that the streamed operand is read with 16-byte loads, and the channel
-// loop is unrolled to keep several of them in flight.
+// evaluated once per channel and lane iteration. A lane takes V points 64 apart,
+// and the channel loop is unrolled to keep several loads in flight.
 template <typename T, int KK, bool HAS_W, int V, int NT, typename Prep, typename Sink>
 __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
                                                const int64_t *__restrict__ idx,
@@ -208,44 +244,38 @@ __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
                                                int c0, int nc, int n1, int64_t np, int64_t ps,
                                                int64_t pe, int vec_ok, Prep prep, Sink sink)
 {
-    for (int64_t p0 = ps + (int64_t)threadIdx.x * V; p0 < pe; p0 += (int64_t)NT * V) {
+    (void)vec_ok;
+    // A wave covers 64*V consecutive points, lane l the points l, l+64, ...: every load
+    // of the wave is a run of consecutive elements (24-byte stride for the indices of
+    // three neighbours).
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    for (int64_t p0 = ps + (int64_t)wave * (64 * V) + lane; p0 < pe; p0 += (int64_t)NT * V) {
         int dst[V][KK];
         T wt[V][KK];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
 #pragma unroll
             for (int i = 0; i < KK; ++i) {
+                const int64_t p = p0 + v * 64;
                 int64_t j = -1;
                 T ww = (T)1;
-                if (p0 + v < pe) {
-                    j = idx[((int64_t)b * np + p0 + v) * KK + i];
+                if (p < pe) {
+                    j = idx[((int64_t)b * np + p) * KK + i];
                     if (HAS_W)
-                        ww = w[((int64_t)b * np + p0 + v) * KK + i];
+                        ww = w[((int64_t)b * np + p) * KK + i];
                 }
                 dst[v][i] = (j >= 0 && j < n1) ? (int)j : -1;
                 wt[v][i] = ww;
             }
         }
-        const bool full = (p0 + V <= pe);
 #pragma unroll 4
         for (int c = 0; c < nc; ++c) {
             const T *__restrict__ grow = gout + ((int64_t)b * c_total + c0 + c) * np;
             T g[V];
-            if (full && vec_ok && V == 4 && sizeof(T) == 4) {
-                const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
-                g[0] = (T)pack.x;
-                g[1 % V] = (T)pack.y;
-                g[2 % V] = (T)pack.z;
-                g[3 % V] = (T)pack.w;
-            } else if (full && vec_ok && V == 2 && sizeof(T) == 8) {
-                const double2 pack = *reinterpret_cast<const double2 *>(grow + p0);
-                g[0] = (T)pack.x;
-                g[1 % V] = (T)pack.y;
-            } else {
 #pragma unroll
-                for (int v = 0; v < V; ++v)
-                    g[v] = (p0 + v < pe) ? grow[p0 + v] : (T)0;
-            }
+            for (int v = 0; v < V; ++v)
+                g[v] = (p0 + v * 64 < pe) ? grow[p0 + v * 64] : (T)0;
             const auto ctx = prep(c);
 #pragma unroll
             for (int v = 0; v < V; ++v)
@@ -588,6 +618,10 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         int cg = 8;
         while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
             cg /= 2;
+#ifdef TK3D_GATHER_STATS
+        if (getenv("TK3D_CG"))
+            cg = atoi(getenv("TK3D_CG"));
+#endif
         const int64_t gy = (C + cg - 1) / cg;
         // Split the points until the chip is full; every chunk re-stages its rows, so
         // keep a chunk well above the staged size.
@@ -596,6 +630,10 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         while (B * gy * chunks < 1024 && NP / (chunks * 2) >= min_chunk &&
                (NP / (chunks * 2)) * KK >= (cg * N1) / 2)
             chunks *= 2;
+#ifdef TK3D_GATHER_STATS
+        if (getenv("TK3D_CHUNKS"))
+            chunks = atoi(getenv("TK3D_CHUNKS"));
+#endif
         int64_t chunk_len = (NP + chunks - 1) / chunks;
         chunk_len = (chunk_len + 15) / 16 * 16;  // keeps 16-byte alignment of chunk starts
         chunks = (NP + chunk_len - 1) / chunk_len;
