@@ -15,7 +15,9 @@ already resident in HBM. The headline value is pair-distances per second,
                 timed on this box's host cores on a bounded sample of the same
                 workload;
   secondary     milliseconds for farthest point sampling, ball query, group
-                points (B=16, N=4096) and the KNN / interpolation configuration.
+                points (B=16, N=4096), the KNN / interpolation configuration and the
+                set-abstraction chain of the stress configuration, with the CPU
+                oracle's time for the same ops beside them.
 
 Everything runs on one GPU; --gpus above 1 is refused.
 """
@@ -85,14 +87,28 @@ def cpu_baseline_chamfer(a, c, budget_s=12.0):
     }
 
 
-def secondary_metrics(dev, steps, warmup):
-    """ms per call for the other ops at their benchmark shapes (events, same stream)."""
+def cpu_ms(fn, scale):
+    """Wall milliseconds of one oracle call, scaled from its batch sample to the full batch."""
+    t0 = time.perf_counter()
+    fn()
+    return round((time.perf_counter() - t0) * 1e3 * scale, 3)
+
+
+def secondary_metrics(dev, steps, warmup, cpu):
+    """ms per call for the other ops at their benchmark shapes (events, same stream).
+
+    With `cpu`, the oracle is timed on the first clouds of each configuration and the
+    figure scaled to the full batch (every op is independent across the batch).
+    """
     import torch
 
     from torkit3d_amd import _C
     from torkit3d_amd.ops.interpolate_feature import three_nn_weights
 
     out = {}
+    cpu_out = {}
+    if cpu:
+        import oracle
     g = torch.Generator().manual_seed(2)
     centres = torch.rand(16, 8, 3, generator=g) * 2 - 1
     comp = torch.randint(0, 8, (16, 4096), generator=g)
@@ -100,6 +116,10 @@ def secondary_metrics(dev, steps, warmup):
            + 0.1 * torch.randn(16, 4096, 3, generator=g)).to(dev)
     out["fps_B16_N4096_K1024_ms"] = gpu_time_ms(
         lambda: _C.sample_farthest_points_cuda(pts, 1024), steps, warmup)
+    if cpu:
+        sample = pts[:4].cpu().numpy()
+        cpu_out["fps_B16_N4096_K1024_ms"] = cpu_ms(
+            lambda: oracle.sample_farthest_points(sample, 1024), 16 / 4)
 
     g = torch.Generator().manual_seed(3)
     xyz = torch.rand(16, 4096, 3, generator=g).to(dev)
@@ -109,11 +129,21 @@ def secondary_metrics(dev, steps, warmup):
         lambda: _C.ball_query_cuda(ctr, xyz, 0.2, 32), steps, warmup)
     nbr = _C.ball_query_cuda(ctr, xyz, 0.2, 32)
     feat = torch.randn(16, 64, 4096, generator=g).to(dev)
+    if cpu:
+        cq, ck = ctr[:4].cpu().numpy(), xyz[:4].cpu().numpy()
+        cpu_out["ball_query_B16_N1024x4096_r0.2_k32_ms"] = cpu_ms(
+            lambda: oracle.ball_query(cq, ck, 0.2, 32), 16 / 4)
+        cf, ci = feat[:4].cpu().numpy(), nbr[:4].cpu().numpy()
+        cpu_out["group_fwd_B16_C64_N4096_to_1024x32_ms"] = cpu_ms(
+            lambda: oracle.group_forward(cf, ci), 16 / 4)
     out["group_fwd_B16_C64_N4096_to_1024x32_ms"] = gpu_time_ms(
         lambda: _C.group_points_forward_cuda(feat, nbr), steps, warmup)
     go = torch.randn(16, 64, 1024, 32, generator=g).to(dev)
     out["group_bwd_ms"] = gpu_time_ms(
         lambda: _C.group_points_backward_cuda(go, nbr, 4096), steps, warmup)
+    if cpu:
+        cgo = go[:4].cpu().numpy()
+        cpu_out["group_bwd_ms"] = cpu_ms(lambda: oracle.group_backward(cgo, ci, 4096), 16 / 4)
 
     g = torch.Generator().manual_seed(4)
     q = (torch.rand(32, 8192, 3, generator=g) * 2 - 1).to(dev)
@@ -122,6 +152,10 @@ def secondary_metrics(dev, steps, warmup):
         lambda: _C.knn_distance_cuda(q, key, 16, 1), steps, warmup)
     out["knn_B32_N8192_M2048_k3_ms"] = gpu_time_ms(
         lambda: _C.knn_distance_cuda(q, key, 3, 1), steps, warmup)
+    if cpu:
+        cq, ck = q[:2].cpu().numpy(), key[:2].cpu().numpy()
+        cpu_out["knn_B32_N8192_M2048_k16_ms"] = cpu_ms(lambda: oracle.knn(cq, ck, 16), 32 / 2)
+        cpu_out["knn_B32_N8192_M2048_k3_ms"] = cpu_ms(lambda: oracle.knn(cq, ck, 3), 32 / 2)
     d2, kidx = _C.knn_distance_cuda(q, key, 3, 1)
     w = three_nn_weights(d2)
     f4 = torch.randn(32, 128, 2048, generator=g).to(dev)
@@ -130,6 +164,13 @@ def secondary_metrics(dev, steps, warmup):
     g4 = torch.randn(32, 128, 8192, generator=g).to(dev)
     out["interpolate_bwd_ms"] = gpu_time_ms(
         lambda: _C.interpolate_backward_cuda(g4, kidx, w, 2048), steps, warmup)
+    if cpu:
+        cf, ci, cw = f4[:4].cpu().numpy(), kidx[:4].cpu().numpy(), w[:4].cpu().numpy()
+        cpu_out["interpolate_fwd_B32_C128_ms"] = cpu_ms(
+            lambda: oracle.interpolate_forward(cf, ci, cw), 32 / 4)
+        cg = g4[:4].cpu().numpy()
+        cpu_out["interpolate_bwd_ms"] = cpu_ms(
+            lambda: oracle.interpolate_backward(cg, ci, cw, 2048), 32 / 4)
     g = torch.Generator().manual_seed(5)
     a = sphere_cloud(g, 32, 16384).to(dev)
     c = sphere_cloud(g, 32, 16384).to(dev)
@@ -138,7 +179,42 @@ def secondary_metrics(dev, steps, warmup):
     gd2 = torch.randn(32, 16384, generator=g).to(dev)
     out["chamfer_bwd_B32_N16384_ms"] = gpu_time_ms(
         lambda: _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2), steps, warmup)
-    return {k: round(v, 5) for k, v in out.items()}
+    if cpu:
+        ca, cc = a[:4].cpu().numpy(), c[:4].cpu().numpy()
+        cg1, cg2 = gd1[:4].cpu().numpy(), gd2[:4].cpu().numpy()
+        ci1, ci2 = i1[:4].cpu().numpy(), i2[:4].cpu().numpy()
+        cpu_out["chamfer_bwd_B32_N16384_ms"] = cpu_ms(
+            lambda: oracle.chamfer_backward(cg1, cg2, ca, cc, ci1, ci2), 32 / 4)
+
+    # Set-abstraction chain of the stress configuration: B=8, three levels of farthest
+    # point sampling, ball query and grouping, each level on the previous level's picks.
+    g = torch.Generator().manual_seed(5)
+    level = torch.rand(8, 16384, 3, generator=g).to(dev)
+    feats = {16384: torch.randn(8, 32, 16384, generator=g).to(dev),
+             4096: torch.randn(8, 64, 4096, generator=g).to(dev),
+             1024: torch.randn(8, 128, 1024, generator=g).to(dev)}
+    chain = []
+    for n_out, radius, nsample in ((4096, 0.1, 32), (1024, 0.2, 32), (256, 0.4, 64)):
+        sel = _C.sample_farthest_points_cuda(level, n_out)
+        centres = torch.gather(level, 1, sel[:, :, None].expand(-1, -1, 3)).contiguous()
+        chain.append((level, centres, n_out, radius, nsample, feats[level.shape[1]]))
+        level = centres
+
+    def run_chain():
+        for support, centres, n_out, radius, nsample, feat in chain:
+            _C.sample_farthest_points_cuda(support, n_out)
+            nb = _C.ball_query_cuda(centres, support, radius, nsample)
+            _C.group_points_forward_cuda(feat, nb)
+
+    out["sa_chain_B8_16384_4096_1024_256_ms"] = gpu_time_ms(run_chain, max(3, steps // 10), 2)
+    out["fps_B8_N16384_K4096_ms"] = gpu_time_ms(
+        lambda: _C.sample_farthest_points_cuda(chain[0][0], 4096), max(3, steps // 10), 1)
+    res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()}}
+    if cpu:
+        res["cpu_oracle_ms"] = cpu_out
+        res["cpu_oracle_note"] = ("OpenMP oracle on %d threads, timed on the first 2-4 clouds of each "
+                                  "configuration and scaled to the full batch" % oracle.num_threads())
+    return res
 
 
 def main():
@@ -236,7 +312,8 @@ def main():
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_chamfer(a_cpu, c_cpu)
     if not args.no_secondary:
-        line["secondary"] = secondary_metrics(dev, max(5, args.steps // 2), args.warmup)
+        line["secondary"] = secondary_metrics(dev, max(5, args.steps // 2), args.warmup,
+                                              not args.no_cpu_baseline)
     print(json.dumps(line))
 
 
