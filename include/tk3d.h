@@ -101,6 +101,21 @@ int tk3d_knn_distance_f64(const double *query, const double *key, int64_t B,
                           int64_t N1, int64_t N2, int64_t k, int version,
                           double *distance, int64_t *index, void *stream);
 
+/* 3 nearest neighbours and their interpolation weights in one launch. Fuses what
+ * FeatureInterpolator.forward does in Python (torkit3d/layers/pointnet2.py:125-130):
+ * knn_points(query, key, 3), then 1/clamp(d2, min=eps), a sum and a division as
+ * four torch kernels. distance and index are exactly tk3d_knn_distance_* with k = 3
+ * (squared distances, MinK slot order); weight[b,i,s] = inv[s] / (inv[0]+inv[1]+inv[2])
+ * with inv[s] = 1 / max(distance[b,i,s], eps), eps rounded to the data type.
+ * channels_first = 0: query [B,N1,3], key [B,N2,3]; 1: query [B,3,N1], key [B,3,N2]
+ * (the reference's models hold [B,3,N]). Outputs are [B,N1,3]. Requires N2 >= 3. */
+int tk3d_three_nn_f32(const float *query, const float *key, int channels_first,
+                      int64_t B, int64_t N1, int64_t N2, double eps, float *distance,
+                      int64_t *index, float *weight, void *stream);
+int tk3d_three_nn_f64(const double *query, const double *key, int channels_first,
+                      int64_t B, int64_t N1, int64_t N2, double eps,
+                      double *distance, int64_t *index, double *weight, void *stream);
+
 /* ---- ball query --------------------------------------------------------------
  * Replaces ball_query_cuda
  * (torkit3d/csrc/include/ball_query.h:6-10, cuda/ball_query_kernel.cu:105-173).
@@ -113,6 +128,17 @@ int tk3d_ball_query_f32(const float *query, const float *key, int64_t B,
 int tk3d_ball_query_f64(const double *query, const double *key, int64_t B,
                         int64_t N1, int64_t N2, float radius,
                         int64_t max_neighbors, int64_t *index, void *stream);
+
+/* Ball query on [B,3,N] clouds (query [B,3,N1], key [B,3,N2]), the layout the
+ * reference's models hold: ball_query(..., transpose=True) is the Python default and
+ * copies both clouds to [B,N,3] before the call (torkit3d/ops/ball_query.py:17-38).
+ * Same result as tk3d_ball_query_* on the transposed clouds, without the copies. */
+int tk3d_ball_query_bcn_f32(const float *query, const float *key, int64_t B,
+                            int64_t N1, int64_t N2, float radius,
+                            int64_t max_neighbors, int64_t *index, void *stream);
+int tk3d_ball_query_bcn_f64(const double *query, const double *key, int64_t B,
+                            int64_t N1, int64_t N2, float radius,
+                            int64_t max_neighbors, int64_t *index, void *stream);
 
 /* ---- farthest point sampling ---------------------------------------------------
  * Replaces sample_farthest_points_cuda
@@ -137,6 +163,26 @@ int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
                                     void *workspace, size_t workspace_bytes,
                                     void *stream);
 
+/* Farthest point sampling on either point layout, optionally returning the sampled
+ * coordinates as well. Fuses what the reference's models do around the op in
+ * Python: sample_farthest_points(points, K, transpose=True) copies a [B,3,N] cloud
+ * to [B,N,3] first (torkit3d/ops/sample_farthest_points.py:28-30) and
+ * batch_index_select(points, index, dim=2) gathers the picks afterwards
+ * (torkit3d/nn/functional.py:34-69, models/segmentation/pointnet2.py:89-90).
+ * channels_first = 0: points [B,N,3], sampled [B,K,3];
+ * channels_first = 1: points [B,3,N], sampled [B,3,K].
+ * `sampled` may be NULL. `index` is identical to tk3d_sample_farthest_points_*. */
+int tk3d_sample_farthest_points_gather_f32(const float *points, int channels_first,
+                                           int64_t B, int64_t N,
+                                           int64_t num_samples, int64_t *index,
+                                           float *sampled, void *workspace,
+                                           size_t workspace_bytes, void *stream);
+int tk3d_sample_farthest_points_gather_f64(const double *points, int channels_first,
+                                           int64_t B, int64_t N,
+                                           int64_t num_samples, int64_t *index,
+                                           double *sampled, void *workspace,
+                                           size_t workspace_bytes, void *stream);
+
 /* ---- group points (gather) -------------------------------------------------------
  * Replaces group_points_forward_cuda / group_points_backward_cuda
  * (torkit3d/csrc/include/group_points.h:6-13, cuda/group_points_kernel.cu:8-114).
@@ -157,6 +203,34 @@ int tk3d_group_points_backward_f64(const double *grad_output,
                                    const int64_t *index, int64_t B, int64_t C,
                                    int64_t N1, int64_t N2, int64_t K,
                                    double *grad_input, void *stream);
+
+/* Grouping for a PointNet++ set-abstraction layer in one output tensor. Fuses what
+ * SetAbstraction.forward does in Python (torkit3d/layers/pointnet2.py:46-58):
+ * group_points(feature), group_points(xyz), subtract the centre, torch.cat - the
+ * concatenation alone re-reads and re-writes the grouped features.
+ *   output[b, c,   m, s] = feature[b, c, index[b,m,s]]              c < C
+ *   output[b, C+a, m, s] = xyz[b, a, index[b,m,s]] - centre[b,a,m]  a < 3
+ * feature [B,C,N1] (may be NULL when C == 0), xyz [B,3,N1], centre [B,3,N2],
+ * index [B,N2,K], output [B,C+3,N2,K].
+ * backward: grad_feature[b,c,j] = sum of grad_output[b,c,m,s] over index[b,m,s] == j,
+ * grad_xyz the same over channels C..C+2; either may be NULL (not wanted). The
+ * gradient of `centre` is minus the sum of channels C..C+2 over s. */
+int tk3d_group_points_concat_forward_f32(const float *feature, const float *xyz,
+                                         const float *centre, const int64_t *index,
+                                         int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                         int64_t K, float *output, void *stream);
+int tk3d_group_points_concat_forward_f64(const double *feature, const double *xyz,
+                                         const double *centre, const int64_t *index,
+                                         int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                         int64_t K, double *output, void *stream);
+int tk3d_group_points_concat_backward_f32(const float *grad_output, const int64_t *index,
+                                          int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                          int64_t K, float *grad_feature,
+                                          float *grad_xyz, void *stream);
+int tk3d_group_points_concat_backward_f64(const double *grad_output, const int64_t *index,
+                                          int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                          int64_t K, double *grad_feature,
+                                          double *grad_xyz, void *stream);
 
 /* ---- feature interpolation ----------------------------------------------------------
  * Replaces interpolate_forward_cuda / interpolate_backward_cuda

@@ -13,7 +13,8 @@
 
 namespace {
 
-template <typename T, int QW, int UNROLL>
+// SOA: clouds are [B,3,N] (coordinate planes) instead of [B,N,3].
+template <typename T, int QW, int UNROLL, bool SOA>
 __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ query,
                                                          const T *__restrict__ key,
                                                          int64_t *__restrict__ index,
@@ -27,8 +28,10 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
         return;
     const int b = (int)(gw / waves_per_batch);
     const int q0 = (int)(gw - (int64_t)b * waves_per_batch) * QW;
-    const T *__restrict__ Q = query + ((int64_t)b * n1 + q0) * 3;
+    const T *__restrict__ Q = query + (int64_t)b * n1 * 3 + (SOA ? q0 : q0 * 3);
     const T *__restrict__ K = key + (int64_t)b * n2 * 3;
+    const int qps = SOA ? 1 : 3, qcs = SOA ? n1 : 1;  // point / coordinate strides
+    const int kps = SOA ? 1 : 3, kcs = SOA ? n2 : 1;
     int64_t *__restrict__ out = index + ((int64_t)b * n1 + q0) * k;
 
     T qx[QW], qy[QW], qz[QW];
@@ -38,9 +41,9 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
 #pragma unroll
     for (int q = 0; q < QW; ++q) {
         const bool ok = q < nq;
-        qx[q] = ok ? Q[q * 3 + 0] : (T)0;
-        qy[q] = ok ? Q[q * 3 + 1] : (T)0;
-        qz[q] = ok ? Q[q * 3 + 2] : (T)0;
+        qx[q] = ok ? Q[q * qps] : (T)0;
+        qy[q] = ok ? Q[q * qps + qcs] : (T)0;
+        qz[q] = ok ? Q[q * qps + 2 * qcs] : (T)0;
         cnt[q] = ok ? 0 : k;  // absent queries count as finished
         first[q] = -1;
     }
@@ -51,9 +54,9 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
         for (int u = 0; u < UNROLL; ++u) {
             const int j = j0 + u * TK_WAVE + lane;
             const bool ok = j < n2;
-            kx[u] = ok ? K[(int64_t)j * 3 + 0] : (T)0;
-            ky[u] = ok ? K[(int64_t)j * 3 + 1] : (T)0;
-            kz[u] = ok ? K[(int64_t)j * 3 + 2] : (T)0;
+            kx[u] = ok ? K[(int64_t)j * kps] : (T)0;
+            ky[u] = ok ? K[(int64_t)j * kps + kcs] : (T)0;
+            kz[u] = ok ? K[(int64_t)j * kps + 2 * kcs] : (T)0;
         }
         bool all_done = true;
 #pragma unroll
@@ -93,8 +96,8 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
 }
 
 template <typename T>
-int ball_query(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2,
-               float radius, int64_t k, int64_t *index, void *stream)
+int ball_query(const T *query, const T *key, bool channels_first, int64_t B, int64_t N1,
+               int64_t N2, float radius, int64_t k, int64_t *index, void *stream)
 {
     if (B < 0 || N1 < 0 || N2 < 0)
         return TK3D_ERR_BAD_SIZE;
@@ -117,9 +120,14 @@ int ball_query(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2,
     // (ball_query.h:9, ball_query_kernel.cu:19,26).
     const T r = (T)radius;
     const T r2 = r * r;
-    hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL>), dim3((unsigned)blocks), dim3(256),
-                       0, (hipStream_t)stream, query, key, index, waves, (int)wpb, (int)N1,
-                       (int)N2, r2, (int)k);
+    if (channels_first)
+        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, true>), dim3((unsigned)blocks),
+                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
+                           (int)N1, (int)N2, r2, (int)k);
+    else
+        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, false>), dim3((unsigned)blocks),
+                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
+                           (int)N1, (int)N2, r2, (int)k);
     return tk_launch_status();
 }
 
@@ -131,14 +139,32 @@ int tk3d_ball_query_f32(const float *query, const float *key, int64_t B, int64_t
                         int64_t N2, float radius, int64_t max_neighbors, int64_t *index,
                         void *stream)
 {
-    return ball_query<float>(query, key, B, N1, N2, radius, max_neighbors, index, stream);
+    return ball_query<float>(query, key, false, B, N1, N2, radius, max_neighbors, index,
+                             stream);
 }
 
 int tk3d_ball_query_f64(const double *query, const double *key, int64_t B, int64_t N1,
                         int64_t N2, float radius, int64_t max_neighbors, int64_t *index,
                         void *stream)
 {
-    return ball_query<double>(query, key, B, N1, N2, radius, max_neighbors, index, stream);
+    return ball_query<double>(query, key, false, B, N1, N2, radius, max_neighbors, index,
+                              stream);
+}
+
+int tk3d_ball_query_bcn_f32(const float *query, const float *key, int64_t B, int64_t N1,
+                            int64_t N2, float radius, int64_t max_neighbors,
+                            int64_t *index, void *stream)
+{
+    return ball_query<float>(query, key, true, B, N1, N2, radius, max_neighbors, index,
+                             stream);
+}
+
+int tk3d_ball_query_bcn_f64(const double *query, const double *key, int64_t B, int64_t N1,
+                            int64_t N2, float radius, int64_t max_neighbors,
+                            int64_t *index, void *stream)
+{
+    return ball_query<double>(query, key, true, B, N1, N2, radius, max_neighbors, index,
+                              stream);
 }
 
 }  // extern "C"

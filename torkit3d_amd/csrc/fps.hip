@@ -82,6 +82,10 @@ struct FpsLayout {
     int log2_bs;
     int c;        // ceil(n / bs): points per reference thread
     float inv_c;  // 1 / c
+    // Element strides of the coordinate arrays: point j, axis a sits at j*ps + a*cs.
+    // [B,N,3] clouds have (3, 1), [B,3,N] clouds (1, N); a batch is n*3 elements in both.
+    int ps, cs;    // input cloud
+    int ops, ocs;  // optional output of the sampled coordinates ([B,K,3] or [B,3,K])
 };
 
 // Point index of a position in the priority order described at the top.
@@ -99,6 +103,7 @@ __device__ __forceinline__ int fps_point_of_position(int pos, const FpsLayout &L
 template <typename T, int P, int NT>
 __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ points,
                                                           int64_t *__restrict__ index,
+                                                          T *__restrict__ sampled,
                                                           FpsLayout L)
 {
     constexpr int NW = NT / TK_WAVE;
@@ -118,17 +123,24 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
         const int pos = tid * P + p;
         const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
         const bool ok = j < L.n;
-        x[p] = ok ? pts[(int64_t)j * 3 + 0] : (T)0;
-        y[p] = ok ? pts[(int64_t)j * 3 + 1] : (T)0;
-        z[p] = ok ? pts[(int64_t)j * 3 + 2] : (T)0;
+        x[p] = ok ? pts[(int64_t)j * L.ps] : (T)0;
+        y[p] = ok ? pts[(int64_t)j * L.ps + L.cs] : (T)0;
+        z[p] = ok ? pts[(int64_t)j * L.ps + 2 * L.cs] : (T)0;
         // Unused slots sit at -1: min() keeps them there and they never exceed 0.
         md[p] = ok ? tk_inf<T>() : (T)-1;
     }
 
     int sel_j = 0;
-    T cx = pts[0], cy = pts[1], cz = pts[2];
-    if (tid == 0)
+    T cx = pts[0], cy = pts[L.cs], cz = pts[2 * L.cs];
+    T *__restrict__ so = sampled ? sampled + (int64_t)blockIdx.x * L.k * 3 : nullptr;
+    if (tid == 0) {
         out[0] = 0;
+        if (so) {
+            so[0] = cx;
+            so[L.ocs] = cy;
+            so[2 * L.ocs] = cz;
+        }
+    }
 
     for (int it = 1; it < L.k; ++it) {
         // Lane-local update and first maximum above zero (strict '>' from zero, as
@@ -183,8 +195,14 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
         }
         // gmax == 0: no point lies away from the chosen set; the previous choice
         // is emitted again, as the reference does.
-        if (tid == 0)
+        if (tid == 0) {
             out[it] = (int64_t)sel_j;
+            if (so) {
+                so[(int64_t)it * L.ops] = cx;
+                so[(int64_t)it * L.ops + L.ocs] = cy;
+                so[(int64_t)it * L.ops + 2 * L.ocs] = cz;
+            }
+        }
     }
 }
 
@@ -267,6 +285,7 @@ template <int P, int NODE> struct FpsWalk {
 template <int P, int NT>
 __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__restrict__ points,
                                                               int64_t *__restrict__ index,
+                                                              float *__restrict__ sampled,
                                                               FpsLayout L)
 {
     static_assert((P & (P - 1)) == 0, "P must be a power of two");
@@ -290,18 +309,25 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
         const int pos = tid * P + p;
         const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
         const bool ok = j < L.n;
-        x[p] = ok ? pts[(int64_t)j * 3 + 0] : 0.0f;
-        y[p] = ok ? pts[(int64_t)j * 3 + 1] : 0.0f;
-        z[p] = ok ? pts[(int64_t)j * 3 + 2] : 0.0f;
+        x[p] = ok ? pts[(int64_t)j * L.ps] : 0.0f;
+        y[p] = ok ? pts[(int64_t)j * L.ps + L.cs] : 0.0f;
+        z[p] = ok ? pts[(int64_t)j * L.ps + 2 * L.cs] : 0.0f;
         jv[p] = j;
         t[P + p] = ok ? F32_INF : F32_NEG1;
     }
     t[0] = 0;
 
     int sel_j = 0;
-    float cx = pts[0], cy = pts[1], cz = pts[2];
-    if (tid == 0)
+    float cx = pts[0], cy = pts[L.cs], cz = pts[2 * L.cs];
+    float *__restrict__ so = sampled ? sampled + (int64_t)blockIdx.x * L.k * 3 : nullptr;
+    if (tid == 0) {
         out[0] = 0;
+        if (so) {
+            so[0] = cx;
+            so[L.ocs] = cy;
+            so[2 * L.ocs] = cz;
+        }
+    }
 
     for (int it = 1; it < L.k; ++it) {
 #pragma unroll
@@ -342,8 +368,14 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
             cy = read_lane(mine.y, gl);
             cz = read_lane(mine.z, gl);
         }
-        if (tid == 0)
+        if (tid == 0) {
             out[it] = (int64_t)sel_j;
+            if (so) {
+                so[(int64_t)it * L.ops] = cx;
+                so[(int64_t)it * L.ops + L.ocs] = cy;
+                so[(int64_t)it * L.ops + 2 * L.ocs] = cz;
+            }
+        }
     }
 }
 
@@ -353,6 +385,7 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
 template <typename T, int NT>
 __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__ points,
                                                            int64_t *__restrict__ index,
+                                                           T *__restrict__ sampled,
                                                            T *__restrict__ min_dist,
                                                            FpsLayout L)
 {
@@ -379,8 +412,14 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
     if (tid == 0)
         out[0] = 0;
     for (int it = 1; it < L.k; ++it) {
-        const T cx = pts[(int64_t)sel_j * 3 + 0], cy = pts[(int64_t)sel_j * 3 + 1],
-                cz = pts[(int64_t)sel_j * 3 + 2];
+        const T cx = pts[(int64_t)sel_j * L.ps], cy = pts[(int64_t)sel_j * L.ps + L.cs],
+                cz = pts[(int64_t)sel_j * L.ps + 2 * L.cs];
+        if (tid == 0 && sampled) {  // coordinates of sample it-1
+            T *so = sampled + (int64_t)blockIdx.x * L.k * 3 + (int64_t)(it - 1) * L.ops;
+            so[0] = cx;
+            so[L.ocs] = cy;
+            so[2 * L.ocs] = cz;
+        }
         T best = (T)0;
         int bpos = 0;
         for (int pos = p0; pos < p1; ++pos) {
@@ -388,8 +427,8 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
             if (m < (T)0)
                 continue;
             const int j = fps_point_of_position(pos, L);
-            const T d = tk_dist2<T>(pts[(int64_t)j * 3 + 0], pts[(int64_t)j * 3 + 1],
-                                    pts[(int64_t)j * 3 + 2], cx, cy, cz);
+            const T d = tk_dist2<T>(pts[(int64_t)j * L.ps], pts[(int64_t)j * L.ps + L.cs],
+                                    pts[(int64_t)j * L.ps + 2 * L.cs], cx, cy, cz);
             const T nm = tk_min<T>(m, d);
             md[pos] = nm;
             if (nm > best) {
@@ -416,13 +455,23 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
         if (tid == 0)
             out[it] = (int64_t)sel_j;
     }
+    if (tid == 0 && sampled) {  // coordinates of the last sample
+        T *so = sampled + (int64_t)blockIdx.x * L.k * 3 + (int64_t)(L.k - 1) * L.ops;
+        so[0] = pts[(int64_t)sel_j * L.ps];
+        so[L.ocs] = pts[(int64_t)sel_j * L.ps + L.cs];
+        so[2 * L.ocs] = pts[(int64_t)sel_j * L.ps + 2 * L.cs];
+    }
 }
 
-FpsLayout fps_layout(int64_t n, int64_t k)
+FpsLayout fps_layout(int64_t n, int64_t k, bool channels_first = false)
 {
     FpsLayout L;
     L.n = (int)n;
     L.k = (int)k;
+    L.ps = channels_first ? 1 : 3;
+    L.cs = channels_first ? (int)n : 1;
+    L.ops = channels_first ? 1 : 3;
+    L.ocs = channels_first ? (int)k : 1;
     int bs = 1, lg = 0;
     // Block size of the reference: smallest power of two >= n, capped at 512
     // (sample_farthest_points_kernel.cu:132-133); its switch runs 32 threads for
@@ -446,46 +495,46 @@ FpsLayout fps_layout(int64_t n, int64_t k)
 int64_t fps_register_capacity(size_t es) { return es == 4 ? 1024 * 16 : 1024 * 8; }
 
 template <typename T, int P, int NT>
-void fps_launch(const T *points, int64_t B, int64_t *index, const FpsLayout &L,
+void fps_launch(const T *points, int64_t B, int64_t *index, T *sampled, const FpsLayout &L,
                 hipStream_t s)
 {
     hipLaunchKernelGGL((fps_register_kernel<T, P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
-                       points, index, L);
+                       points, index, sampled, L);
 }
 
 template <int P, int NT>
-void fps_launch_f32(const float *points, int64_t B, int64_t *index, const FpsLayout &L,
-                    hipStream_t s)
+void fps_launch_f32(const float *points, int64_t B, int64_t *index, float *sampled,
+                    const FpsLayout &L, hipStream_t s)
 {
     hipLaunchKernelGGL((fps_register_kernel_f32<P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
-                       points, index, L);
+                       points, index, sampled, L);
 }
 
 // fp32: (points per lane, lanes) by cloud size, from timing every shape on an
 // MI355X: two waves per SIMD (512 lanes) hide each other's reduction latency; more
 // waves only repeat the per-wave reduction.
-void fps_dispatch_f32(const float *points, int64_t B, int64_t *index, const FpsLayout &L,
-                      int64_t npos, hipStream_t s)
+void fps_dispatch_f32(const float *points, int64_t B, int64_t *index, float *sampled,
+                      const FpsLayout &L, int64_t npos, hipStream_t s)
 {
     if (npos <= 64 * 2)
-        fps_launch_f32<2, 64>(points, B, index, L, s);
+        fps_launch_f32<2, 64>(points, B, index, sampled, L, s);
     else if (npos <= 256 * 2)
-        fps_launch_f32<2, 256>(points, B, index, L, s);
+        fps_launch_f32<2, 256>(points, B, index, sampled, L, s);
     else if (npos <= 512 * 2)
-        fps_launch_f32<2, 512>(points, B, index, L, s);
+        fps_launch_f32<2, 512>(points, B, index, sampled, L, s);
     else if (npos <= 512 * 4)
-        fps_launch_f32<4, 512>(points, B, index, L, s);
+        fps_launch_f32<4, 512>(points, B, index, sampled, L, s);
     else if (npos <= 512 * 8)
-        fps_launch_f32<8, 512>(points, B, index, L, s);
+        fps_launch_f32<8, 512>(points, B, index, sampled, L, s);
     else if (npos <= 512 * 16)
-        fps_launch_f32<16, 512>(points, B, index, L, s);
+        fps_launch_f32<16, 512>(points, B, index, sampled, L, s);
     else
-        fps_launch_f32<32, 512>(points, B, index, L, s);
+        fps_launch_f32<32, 512>(points, B, index, sampled, L, s);
 }
 
 template <typename T>
-int fps(const T *points, int64_t B, int64_t N, int64_t K, int64_t *index, void *workspace,
-        size_t workspace_bytes, void *stream)
+int fps(const T *points, bool channels_first, int64_t B, int64_t N, int64_t K, int64_t *index,
+        T *sampled, void *workspace, size_t workspace_bytes, void *stream)
 {
     if (B < 0 || N < 0)
         return TK3D_ERR_BAD_SIZE;
@@ -498,35 +547,35 @@ int fps(const T *points, int64_t B, int64_t N, int64_t K, int64_t *index, void *
     if (!points || !index)
         return TK3D_ERR_NULL_POINTER;
     hipStream_t s = (hipStream_t)stream;
-    const FpsLayout L = fps_layout(N, K);
+    const FpsLayout L = fps_layout(N, K, channels_first);
     const int64_t npos = (int64_t)L.bs * L.c;
     if (npos <= fps_register_capacity(sizeof(T))) {
         if constexpr (sizeof(T) == 4) {
-            fps_dispatch_f32(points, B, index, L, npos, s);
+            fps_dispatch_f32(points, B, index, sampled, L, npos, s);
             return tk_launch_status();
         }
         // Fewest points per lane that still covers the cloud: short serial chains.
         if (npos <= 256 * 1)
-            fps_launch<T, 1, 256>(points, B, index, L, s);
+            fps_launch<T, 1, 256>(points, B, index, sampled, L, s);
         else if (npos <= 256 * 2)
-            fps_launch<T, 2, 256>(points, B, index, L, s);
+            fps_launch<T, 2, 256>(points, B, index, sampled, L, s);
         else if (npos <= 512 * 2)
-            fps_launch<T, 2, 512>(points, B, index, L, s);
+            fps_launch<T, 2, 512>(points, B, index, sampled, L, s);
         else if (npos <= 1024 * 2)
-            fps_launch<T, 2, 1024>(points, B, index, L, s);
+            fps_launch<T, 2, 1024>(points, B, index, sampled, L, s);
         else if (npos <= 1024 * 4)
-            fps_launch<T, 4, 1024>(points, B, index, L, s);
+            fps_launch<T, 4, 1024>(points, B, index, sampled, L, s);
         else if (npos <= 1024 * 8)
-            fps_launch<T, 8, 1024>(points, B, index, L, s);
+            fps_launch<T, 8, 1024>(points, B, index, sampled, L, s);
         else if constexpr (sizeof(T) == 4)
-            fps_launch<T, 16, 1024>(points, B, index, L, s);
+            fps_launch<T, 16, 1024>(points, B, index, sampled, L, s);
         return tk_launch_status();
     }
     const size_t need = (size_t)B * (size_t)npos * sizeof(T);
     if (!workspace || workspace_bytes < need)
         return TK3D_ERR_WORKSPACE;
     hipLaunchKernelGGL((fps_streaming_kernel<T, 1024>), dim3((unsigned)B), dim3(1024), 0, s,
-                       points, index, (T *)workspace, L);
+                       points, index, sampled, (T *)workspace, L);
     return tk_launch_status();
 }
 
@@ -549,15 +598,34 @@ int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,
                                     int64_t num_samples, int64_t *index, void *workspace,
                                     size_t workspace_bytes, void *stream)
 {
-    return fps<float>(points, B, N, num_samples, index, workspace, workspace_bytes, stream);
+    return fps<float>(points, false, B, N, num_samples, index, nullptr, workspace,
+                      workspace_bytes, stream);
 }
 
 int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
                                     int64_t num_samples, int64_t *index, void *workspace,
                                     size_t workspace_bytes, void *stream)
 {
-    return fps<double>(points, B, N, num_samples, index, workspace, workspace_bytes,
-                       stream);
+    return fps<double>(points, false, B, N, num_samples, index, nullptr, workspace,
+                       workspace_bytes, stream);
+}
+
+int tk3d_sample_farthest_points_gather_f32(const float *points, int channels_first,
+                                           int64_t B, int64_t N, int64_t num_samples,
+                                           int64_t *index, float *sampled, void *workspace,
+                                           size_t workspace_bytes, void *stream)
+{
+    return fps<float>(points, channels_first != 0, B, N, num_samples, index, sampled,
+                      workspace, workspace_bytes, stream);
+}
+
+int tk3d_sample_farthest_points_gather_f64(const double *points, int channels_first,
+                                           int64_t B, int64_t N, int64_t num_samples,
+                                           int64_t *index, double *sampled, void *workspace,
+                                           size_t workspace_bytes, void *stream)
+{
+    return fps<double>(points, channels_first != 0, B, N, num_samples, index, sampled,
+                       workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

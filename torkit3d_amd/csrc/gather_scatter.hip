@@ -35,7 +35,7 @@ constexpr int GS_BLOCK = 256;
 template <typename T, int KK, bool HAS_W, int V>
 __global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
     const T *__restrict__ in, const int64_t *__restrict__ idx, const T *__restrict__ w,
-    T *__restrict__ out, int c_total, int n1, int64_t np, int cg, int vec_ok)
+    T *__restrict__ out, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg, int vec_ok)
 {
     const int b = blockIdx.z;
     const int c0 = blockIdx.y * cg;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
     const bool full = (p0 + V <= np);
     for (int c = c0; c < c1; ++c) {
         const T *__restrict__ row = in + ((int64_t)b * c_total + c) * n1;
-        T *__restrict__ orow = out + ((int64_t)b * c_total + c) * np;
+        T *__restrict__ orow = out + ((int64_t)b * wc_total + wc_off + c) * np;
         T val[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
@@ -127,7 +127,7 @@ __device__ unsigned long long gather_stats[1 << 16];
 template <typename T, int KK, bool HAS_W, int V, int NT>
 __global__ __launch_bounds__(NT) void gather_lds_kernel(
     const T *__restrict__ in, const int64_t *__restrict__ idx, const T *__restrict__ w,
-    T *__restrict__ out, int c_total, int n1, int64_t np, int cg, int64_t chunk_len, int vec_ok)
+    T *__restrict__ out, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg, int64_t chunk_len, int vec_ok)
 {
     extern __shared__ __align__(16) unsigned char gather_smem[];
     T *rows = reinterpret_cast<T *>(gather_smem);  // [cg][n1]
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
 #pragma unroll 4
         for (int c = 0; c < nc; ++c) {
             const T *row = rows + c * n1;
-            T *__restrict__ orow = out + ((int64_t)b * c_total + c0 + c) * np;
+            T *__restrict__ orow = out + ((int64_t)b * wc_total + wc_off + c0 + c) * np;
 #pragma unroll
             for (int v = 0; v < V; ++v) {
                 T val;
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(GS_BLOCK) void fill_zero_kernel(T *__restrict__ p, 
 template <typename T, int KK, bool HAS_W, int V, int NT, typename Prep, typename Sink>
 __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
                                                const int64_t *__restrict__ idx,
-                                               const T *__restrict__ w, int b, int c_total,
+                                               const T *__restrict__ w, int b, int wc_total,
                                                int c0, int nc, int n1, int64_t np, int64_t ps,
                                                int64_t pe, int vec_ok, Prep prep, Sink sink)
 {
@@ -271,7 +271,7 @@ __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
         }
 #pragma unroll 4
         for (int c = 0; c < nc; ++c) {
-            const T *__restrict__ grow = gout + ((int64_t)b * c_total + c0 + c) * np;
+            const T *__restrict__ grow = gout + ((int64_t)b * wc_total + c0 + c) * np;
             T g[V];
 #pragma unroll
             for (int v = 0; v < V; ++v)
@@ -292,7 +292,7 @@ __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
 template <typename T, int KK, bool HAS_W, int V, int NT>
 __global__ __launch_bounds__(NT) void scatter_lds_kernel(
     const T *__restrict__ gout, const int64_t *__restrict__ idx, const T *__restrict__ w,
-    T *__restrict__ gin, int c_total, int n1, int64_t np, int cg, int64_t seg_len,
+    T *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg, int64_t seg_len,
     int merge_with_atomics, int vec_ok)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
         rows[i] = (T)0;
     __syncthreads();
     scatter_stream<T, KK, HAS_W, V, NT>(
-        gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
         [&](int, int c, int dst, T g, T ww) { atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g); });
     __syncthreads();
 
@@ -367,7 +367,7 @@ __device__ unsigned long long scatter_stats[1 << 16];
 template <int KK, bool HAS_W, int V, int NT, int CGMAX>
 __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     const float *__restrict__ gout, const int64_t *__restrict__ idx,
-    const float *__restrict__ w, float *__restrict__ gin, int c_total, int n1, int64_t np, int cg,
+    const float *__restrict__ w, float *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg,
     int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                 for (int c = 0; c < CGMAX; ++c) {
                     if (c >= nc)
                         break;
-                    const float *__restrict__ grow = gout + ((int64_t)b * c_total + c0 + c) * np;
+                    const float *__restrict__ grow = gout + ((int64_t)b * wc_total + wc_off + c0 + c) * np;
                     float g[V];
                     if (full && vec_ok && V == 4) {
                         const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         };
         bool exceeded = false;
         scatter_stream<float, KK, HAS_W, V, NT>(
-            gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok,
+            gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok,
             [&](int c) {
                 RowScale r;
                 r.scale = s_scale[c];
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         rows[i] = 0.0f;
     __syncthreads();
     scatter_stream<float, KK, HAS_W, V, NT>(
-        gout, idx, w, b, c_total, c0, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
         [&](int, int c, int dst, float g, float ww) {
             atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g);
         });
@@ -558,7 +558,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
 template <typename T, int KK, bool HAS_W>
 __global__ __launch_bounds__(GS_BLOCK) void scatter_global_kernel(
     const T *__restrict__ gout, const int64_t *__restrict__ idx, const T *__restrict__ w,
-    T *__restrict__ gin, int c_total, int n1, int64_t np, int cg)
+    T *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg)
 {
     const int b = blockIdx.z;
     const int c0 = blockIdx.y * cg;
@@ -575,7 +575,7 @@ __global__ __launch_bounds__(GS_BLOCK) void scatter_global_kernel(
         wt[i] = HAS_W ? w[((int64_t)b * np + p) * KK + i] : (T)1;
     }
     for (int c = c0; c < c1; ++c) {
-        const T g = gout[((int64_t)b * c_total + c) * np + p];
+        const T g = gout[((int64_t)b * wc_total + wc_off + c) * np + p];
         T *row = gin + ((int64_t)b * c_total + c) * n1;
 #pragma unroll
         for (int i = 0; i < KK; ++i)
@@ -599,8 +599,12 @@ int check_shape(int64_t B, int64_t C, int64_t N1, int64_t NP, int64_t KK)
 
 template <typename T, int KK, bool HAS_W>
 int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, int64_t N1,
-           int64_t NP, T *out, hipStream_t s)
+           int64_t NP, T *out, hipStream_t s, int64_t wc_total = -1, int64_t wc_off = 0)
 {
+    // The output may be a channel slice [wc_off, wc_off + C) of a tensor with wc_total
+    // channels (same B and NP); by default it is exactly [B, C, NP].
+    if (wc_total < 0)
+        wc_total = C;
     if (B * C * NP == 0)
         return TK3D_OK;
     if (!in && N1 > 0)
@@ -641,7 +645,7 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
             return TK3D_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((gather_lds_kernel<T, KK, HAS_W, V, NT>),
                            dim3((unsigned)chunks, (unsigned)gy, (unsigned)B), dim3(NT),
-                           (size_t)(cg * row_bytes), s, in, idx, w, out, (int)C, (int)N1, NP, cg,
+                           (size_t)(cg * row_bytes), s, in, idx, w, out, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP, cg,
                            chunk_len, vec_ok);
         return tk_launch_status();
     }
@@ -657,14 +661,18 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gather_kernel<T, KK, HAS_W, V>),
                        dim3((unsigned)tiles, (unsigned)gy, (unsigned)B), dim3(GS_BLOCK), 0, s,
-                       in, idx, w, out, (int)C, (int)N1, NP, cg, vec_ok);
+                       in, idx, w, out, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP, cg, vec_ok);
     return tk_launch_status();
 }
 
 template <typename T, int KK, bool HAS_W>
 int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C, int64_t N1,
-            int64_t NP, T *gin, hipStream_t s)
+            int64_t NP, T *gin, hipStream_t s, int64_t wc_total = -1, int64_t wc_off = 0)
 {
+    // gout may be a channel slice [wc_off, wc_off + C) of a tensor with wc_total
+    // channels (same B and NP); by default it is exactly [B, C, NP].
+    if (wc_total < 0)
+        wc_total = C;
     const int64_t out_elems = B * C * N1;
     if (out_elems == 0)
         return TK3D_OK;
@@ -727,7 +735,7 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
                 hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
                                    dim3(GS_BLOCK), 0, s, gin, out_elems);
             hipLaunchKernelGGL(kernel, dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
-                               (size_t)(cg * acc_row), s, gout, idx, w, gin, (int)C, (int)N1, NP,
+                               (size_t)(cg * acc_row), s, gout, idx, w, gin, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP,
                                cg, seg_len, nseg > 1 ? 1 : 0, vec_ok, log2_count);
             return tk_launch_status();
         }
@@ -767,7 +775,7 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
                                dim3(GS_BLOCK), 0, s, gin, out_elems);
         hipLaunchKernelGGL((scatter_lds_kernel<T, KK, HAS_W, V, NT>),
                            dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
-                           (size_t)(cg * row_bytes), s, gout, idx, w, gin, (int)C, (int)N1, NP,
+                           (size_t)(cg * row_bytes), s, gout, idx, w, gin, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP,
                            cg, seg_len, nseg > 1 ? 1 : 0, vec_ok);
         return tk_launch_status();
     }
@@ -783,7 +791,7 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((scatter_global_kernel<T, KK, HAS_W>),
                        dim3((unsigned)tiles, (unsigned)gy, (unsigned)B), dim3(GS_BLOCK), 0, s,
-                       gout, idx, w, gin, (int)C, (int)N1, NP, cg);
+                       gout, idx, w, gin, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP, cg);
     return tk_launch_status();
 }
 
@@ -854,9 +862,116 @@ int group_backward(const T *gout, const int64_t *idx, int64_t B, int64_t C, int6
                                 (hipStream_t)stream);
 }
 
+// Grouped coordinates relative to their centre, written into the last three channels
+// of a [B, wc_total, N2, K] tensor: out[b, wc_off+a, m, s] = xyz[b,a,idx[b,m,s]] -
+// centre[b,a,m] (torkit3d/layers/pointnet2.py:55-58). The clouds are [B,3,N]; they
+// are small (12 bytes per point), so the gathers hit in cache.
+template <typename T>
+__global__ __launch_bounds__(GS_BLOCK) void group_xyz_kernel(
+    const T *__restrict__ xyz, const T *__restrict__ centre, const int64_t *__restrict__ idx,
+    T *__restrict__ out, int wc_total, int wc_off, int n1, int n2, int k)
+{
+    const int b = blockIdx.y;
+    const int64_t np = (int64_t)n2 * k;
+    const int64_t p = (int64_t)blockIdx.x * GS_BLOCK + threadIdx.x;
+    if (p >= np)
+        return;
+    const int64_t j = idx[(int64_t)b * np + p];
+    const bool ok = j >= 0 && j < n1;
+    const int m = (int)(p / k);
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const T v = ok ? xyz[((int64_t)b * 3 + a) * n1 + j] : (T)0;
+        out[((int64_t)b * wc_total + wc_off + a) * np + p] =
+            v - centre[((int64_t)b * 3 + a) * n2 + m];
+    }
+}
+
+template <typename T>
+int group_concat_forward(const T *feat, const T *xyz, const T *centre, const int64_t *idx,
+                         int64_t B, int64_t C, int64_t N1, int64_t N2, int64_t K, T *out,
+                         void *stream)
+{
+    if (N2 < 0 || K < 0 || !tk_fits(TK_MAX_ELEMS, N2, K))
+        return N2 < 0 || K < 0 ? TK3D_ERR_BAD_SIZE : TK3D_ERR_UNSUPPORTED;
+    const int rc = check_shape(B, C + 3, N1, N2 * K, 1);
+    if (rc != TK3D_OK)
+        return rc;
+    if (B * N2 * K == 0)
+        return TK3D_OK;
+    if (!xyz || !centre || !idx || !out || (C > 0 && !feat))
+        return TK3D_ERR_NULL_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    if (C > 0) {
+        const int g = gather<T, 1, false>(feat, idx, nullptr, B, C, N1, N2 * K, out, s, C + 3, 0);
+        if (g != TK3D_OK)
+            return g;
+    }
+    const int64_t tiles = (N2 * K + GS_BLOCK - 1) / GS_BLOCK;
+    if (tiles > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((group_xyz_kernel<T>), dim3((unsigned)tiles, (unsigned)B), dim3(GS_BLOCK),
+                       0, s, xyz, centre, idx, out, (int)(C + 3), (int)C, (int)N1, (int)N2,
+                       (int)K);
+    return tk_launch_status();
+}
+
+template <typename T>
+int group_concat_backward(const T *gout, const int64_t *idx, int64_t B, int64_t C, int64_t N1,
+                          int64_t N2, int64_t K, T *gfeat, T *gxyz, void *stream)
+{
+    if (N2 < 0 || K < 0 || !tk_fits(TK_MAX_ELEMS, N2, K))
+        return N2 < 0 || K < 0 ? TK3D_ERR_BAD_SIZE : TK3D_ERR_UNSUPPORTED;
+    const int rc = check_shape(B, C + 3, N1, N2 * K, 1);
+    if (rc != TK3D_OK)
+        return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (C > 0 && gfeat) {
+        const int g = scatter<T, 1, false>(gout, idx, nullptr, B, C, N1, N2 * K, gfeat, s, C + 3, 0);
+        if (g != TK3D_OK)
+            return g;
+    }
+    if (gxyz)
+        return scatter<T, 1, false>(gout, idx, nullptr, B, 3, N1, N2 * K, gxyz, s, C + 3, C);
+    return TK3D_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int tk3d_group_points_concat_forward_f32(const float *feature, const float *xyz,
+                                         const float *centre, const int64_t *index, int64_t B,
+                                         int64_t C, int64_t N1, int64_t N2, int64_t K,
+                                         float *output, void *stream)
+{
+    return group_concat_forward<float>(feature, xyz, centre, index, B, C, N1, N2, K, output,
+                                       stream);
+}
+int tk3d_group_points_concat_forward_f64(const double *feature, const double *xyz,
+                                         const double *centre, const int64_t *index,
+                                         int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                         int64_t K, double *output, void *stream)
+{
+    return group_concat_forward<double>(feature, xyz, centre, index, B, C, N1, N2, K, output,
+                                        stream);
+}
+int tk3d_group_points_concat_backward_f32(const float *grad_output, const int64_t *index,
+                                          int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                          int64_t K, float *grad_feature, float *grad_xyz,
+                                          void *stream)
+{
+    return group_concat_backward<float>(grad_output, index, B, C, N1, N2, K, grad_feature,
+                                        grad_xyz, stream);
+}
+int tk3d_group_points_concat_backward_f64(const double *grad_output, const int64_t *index,
+                                          int64_t B, int64_t C, int64_t N1, int64_t N2,
+                                          int64_t K, double *grad_feature, double *grad_xyz,
+                                          void *stream)
+{
+    return group_concat_backward<double>(grad_output, index, B, C, N1, N2, K, grad_feature,
+                                         grad_xyz, stream);
+}
 
 int tk3d_group_points_forward_f32(const float *input, const int64_t *index, int64_t B,
                                   int64_t C, int64_t N1, int64_t N2, int64_t K,

@@ -20,10 +20,35 @@ namespace {
 constexpr int KNN_BLOCK = 256;
 constexpr int KNN_STAGE = 1024;
 
-template <typename T, int KMAX>
+// Coordinate `a` of point `j` of an n-point cloud: [n,3] rows, or with SOA three planes
+// [3,n] (the layout the reference's models keep their clouds in).
+template <bool SOA, typename T>
+__device__ __forceinline__ T knn_coord(const T *__restrict__ cloud, int n, int j, int a)
+{
+    return SOA ? cloud[(int64_t)a * n + j] : cloud[(int64_t)j * 3 + a];
+}
+
+// Inverse-squared-distance weights of the three neighbours, as FeatureInterpolator
+// forms them with torch ops (torkit3d/layers/pointnet2.py:128-130):
+// inv = 1 / clamp(d, min=eps); w = inv / (inv0 + inv1 + inv2).
+template <typename T>
+__device__ __forceinline__ void knn_three_weights(const T (&d)[3], T eps, T *__restrict__ w)
+{
+    T inv[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+        inv[i] = (T)1 / (d[i] < eps ? eps : d[i]);  // a NaN stays a NaN, as in clamp
+    const T norm = (inv[0] + inv[1]) + inv[2];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+        w[i] = inv[i] / norm;
+}
+
+template <typename T, int KMAX, bool SOA, bool WEIGHTS>
 __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
     const T *__restrict__ query, const T *__restrict__ key, T *__restrict__ distance,
-    int64_t *__restrict__ index, int blocks_per_batch, int n1, int n2, int k)
+    int64_t *__restrict__ index, T *__restrict__ weight, T eps, int blocks_per_batch, int n1,
+    int n2, int k)
 {
     __shared__ T skey[KNN_STAGE * 4];
     const int tid = threadIdx.x;
@@ -33,10 +58,10 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
     const T *__restrict__ K = key + (int64_t)b * n2 * 3;
     T qx = 0, qy = 0, qz = 0;
     if (active) {
-        const T *q = query + ((int64_t)b * n1 + qi) * 3;
-        qx = q[0];
-        qy = q[1];
-        qz = q[2];
+        const T *__restrict__ Q = query + (int64_t)b * n1 * 3;
+        qx = knn_coord<SOA>(Q, n1, qi, 0);
+        qy = knn_coord<SOA>(Q, n1, qi, 1);
+        qz = knn_coord<SOA>(Q, n1, qi, 2);
     }
 
     T kd[KMAX];
@@ -51,7 +76,8 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
         kd[s] = -tk_inf<T>();
         ki[s] = 0;
         if (s < k) {  // uniform
-            const T d = tk_dist2<T>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            const T d = tk_dist2<T>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                                       knn_coord<SOA>(K, n2, s, 2), qx, qy, qz);
             kd[s] = d;
             ki[s] = s;
             if (s == 0 || d > max_key) {
@@ -67,9 +93,9 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
             const int kj = stage0 + j;
             T x = 0, y = 0, z = 0;
             if (kj < n2) {
-                x = K[(int64_t)kj * 3 + 0];
-                y = K[(int64_t)kj * 3 + 1];
-                z = K[(int64_t)kj * 3 + 2];
+                x = knn_coord<SOA>(K, n2, kj, 0);
+                y = knn_coord<SOA>(K, n2, kj, 1);
+                z = knn_coord<SOA>(K, n2, kj, 2);
             }
             skey[j * 4 + 0] = x;
             skey[j * 4 + 1] = y;
@@ -112,6 +138,10 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
                 oi[s] = (int64_t)ki[s];
             }
         }
+        if constexpr (WEIGHTS && KMAX >= 3) {  // k == 3
+            const T d3[3] = {kd[0], kd[1], kd[2]};
+            knn_three_weights<T>(d3, eps, weight + ((int64_t)b * n1 + qi) * 3);
+        }
     }
 }
 
@@ -132,11 +162,11 @@ __device__ unsigned long long knn_stats[1 << 16];  // per wave: t0, t1, sweep cy
 #define KNN_CLOCK() __builtin_readcyclecounter()
 #endif
 
-template <int KMAX>
+template <int KMAX, bool SOA, bool WEIGHTS>
 __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
-    float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
-    int n2, int k)
+    float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
+    float eps, int blocks_per_batch, int n1, int n2, int k)
 {
     constexpr int CHUNK = 32;
     static_assert(KNN_STAGE % CHUNK == 0, "a chunk must not straddle stages");
@@ -148,10 +178,10 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     const float *__restrict__ K = key + (int64_t)b * n2 * 3;
     float qx = 0, qy = 0, qz = 0;
     if (active) {
-        const float *q = query + ((int64_t)b * n1 + qi) * 3;
-        qx = q[0];
-        qy = q[1];
-        qz = q[2];
+        const float *__restrict__ Q = query + (int64_t)b * n1 * 3;
+        qx = knn_coord<SOA>(Q, n1, qi, 0);
+        qy = knn_coord<SOA>(Q, n1, qi, 1);
+        qz = knn_coord<SOA>(Q, n1, qi, 2);
     }
 
     float kd[KMAX];
@@ -166,7 +196,8 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
         kd[s] = -__builtin_huge_valf();
         ki[s] = 0;
         if (s < k) {  // uniform
-            const float d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                                       knn_coord<SOA>(K, n2, s, 2), qx, qy, qz);
             kd[s] = d;
             ki[s] = s;
             fill_nan |= d != d;
@@ -192,9 +223,9 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             const int kj = stage0 + j;
             float4 e = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (kj < n2) {
-                e.x = K[(int64_t)kj * 3 + 0];
-                e.y = K[(int64_t)kj * 3 + 1];
-                e.z = K[(int64_t)kj * 3 + 2];
+                e.x = knn_coord<SOA>(K, n2, kj, 0);
+                e.y = knn_coord<SOA>(K, n2, kj, 1);
+                e.z = knn_coord<SOA>(K, n2, kj, 2);
             }
             reinterpret_cast<float4 *>(skey)[j] = e;
         }
@@ -214,11 +245,12 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
                 // A full chunk comes straight from global memory: the addresses are the
                 // same for the whole wave, so the loads are scalar and the coordinates are
                 // scalar operands of the vector arithmetic - no LDS traffic in the sweep.
-                const float *__restrict__ g = K + (int64_t)first * 3;
 #pragma unroll
                 for (int i = 0; i < CHUNK; ++i) {
-                    const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2],
-                                                    qx, qy, qz);
+                    const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, first + i, 0),
+                                                    knn_coord<SOA>(K, n2, first + i, 1),
+                                                    knn_coord<SOA>(K, n2, first + i, 2), qx, qy,
+                                                    qz);
                     const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
                     mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
                 }
@@ -346,6 +378,10 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
                 od[s] = kd[s];
                 oi[s] = (int64_t)ki[s];
             }
+        }
+        if constexpr (WEIGHTS && KMAX >= 3) {  // k == 3
+            const float d3[3] = {kd[0], kd[1], kd[2]};
+            knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + qi) * 3);
         }
     }
 }
@@ -653,16 +689,19 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_global_kernel(
     }
 }
 
-template <typename T, int KMAX>
+template <typename T, int KMAX, bool SOA = false, bool WEIGHTS = false>
 void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64_t B,
-                int bpb, int n1, int n2, int k, hipStream_t s)
+                int bpb, int n1, int n2, int k, hipStream_t s, T *weight = nullptr,
+                T eps = (T)0)
 {
     if constexpr (sizeof(T) == 4)
-        hipLaunchKernelGGL((knn_batched_kernel_f32<KMAX>), dim3((unsigned)(B * bpb)),
-                           dim3(KNN_BLOCK), 0, s, query, key, distance, index, bpb, n1, n2, k);
+        hipLaunchKernelGGL((knn_batched_kernel_f32<KMAX, SOA, WEIGHTS>),
+                           dim3((unsigned)(B * bpb)), dim3(KNN_BLOCK), 0, s, query, key, distance,
+                           index, weight, eps, bpb, n1, n2, k);
     else
-        hipLaunchKernelGGL((knn_register_kernel<T, KMAX>), dim3((unsigned)(B * bpb)),
-                           dim3(KNN_BLOCK), 0, s, query, key, distance, index, bpb, n1, n2, k);
+        hipLaunchKernelGGL((knn_register_kernel<T, KMAX, SOA, WEIGHTS>),
+                           dim3((unsigned)(B * bpb)), dim3(KNN_BLOCK), 0, s, query, key, distance,
+                           index, weight, eps, bpb, n1, n2, k);
 }
 
 template <typename T>
@@ -716,9 +755,54 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
     return tk_launch_status();
 }
 
+// 3 nearest neighbours with the interpolation weights formed in the same kernel.
+template <typename T>
+int three_nn(const T *query, const T *key, bool channels_first, int64_t B, int64_t N1,
+             int64_t N2, double eps, T *distance, int64_t *index, T *weight, void *stream)
+{
+    if (B < 0 || N1 < 0 || N2 < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (N2 < 3)
+        return TK3D_ERR_BAD_K;
+    if (N1 > TK_MAX_I32 / 4 || N2 > TK_MAX_I32 / 4 || !tk_fits(TK_MAX_ELEMS, B, N1, 3) ||
+        !tk_fits(TK_MAX_ELEMS, B, N2, 3))
+        return TK3D_ERR_UNSUPPORTED;
+    if (B * N1 == 0)
+        return TK3D_OK;
+    if (!query || !key || !distance || !index || !weight)
+        return TK3D_ERR_NULL_POINTER;
+    const int64_t bpb = (N1 + KNN_BLOCK - 1) / KNN_BLOCK;
+    if (B * bpb > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (channels_first)
+        knn_launch<T, 4, true, true>(query, key, distance, index, B, (int)bpb, (int)N1, (int)N2,
+                                     3, s, weight, (T)eps);
+    else
+        knn_launch<T, 4, false, true>(query, key, distance, index, B, (int)bpb, (int)N1,
+                                      (int)N2, 3, s, weight, (T)eps);
+    return tk_launch_status();
+}
+
 }  // namespace
 
 extern "C" {
+
+int tk3d_three_nn_f32(const float *query, const float *key, int channels_first, int64_t B,
+                      int64_t N1, int64_t N2, double eps, float *distance, int64_t *index,
+                      float *weight, void *stream)
+{
+    return three_nn<float>(query, key, channels_first != 0, B, N1, N2, eps, distance, index,
+                           weight, stream);
+}
+
+int tk3d_three_nn_f64(const double *query, const double *key, int channels_first, int64_t B,
+                      int64_t N1, int64_t N2, double eps, double *distance, int64_t *index,
+                      double *weight, void *stream)
+{
+    return three_nn<double>(query, key, channels_first != 0, B, N1, N2, eps, distance, index,
+                            weight, stream);
+}
 
 int tk3d_knn_distance_f32(const float *query, const float *key, int64_t B, int64_t N1,
                           int64_t N2, int64_t k, int version, float *distance,

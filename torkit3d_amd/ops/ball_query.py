@@ -1,21 +1,25 @@
 """Ball query (API of torkit3d/ops/ball_query.py)."""
 import torch
 
-from .. import _C
+from .. import _C, _fused
 
 
 class BallQueryFunction(torch.autograd.Function):
-    """Not differentiable (torkit3d/ops/ball_query.py:6-14)."""
+    """Not differentiable (torkit3d/ops/ball_query.py:6-14). ``channels_first``
+    (not in the reference) says the clouds are [B, 3, N]."""
 
     @staticmethod
-    def forward(ctx, query, key, radius, max_neighbors):
-        index = _C.ball_query_cuda(query, key, radius, max_neighbors)
+    def forward(ctx, query, key, radius, max_neighbors, channels_first=False):
+        if channels_first:
+            index = _fused.ball_query_bcn(query, key, radius, max_neighbors)
+        else:
+            index = _C.ball_query_cuda(query, key, radius, max_neighbors)
         ctx.mark_non_differentiable(index)
         return index
 
     @staticmethod
     def backward(ctx, *grad_outputs):
-        return (None,) * 4
+        return (None,) * 5
 
 
 def ball_query(query, key, radius, max_neighbors, transpose=True):
@@ -28,7 +32,6 @@ def ball_query(query, key, radius, max_neighbors, transpose=True):
         index [B, N1, max_neighbors] int64: the first hits in key order, padded with
         the first hit; all -1 where nothing lies within the radius.
     """
-    if transpose:
-        query, key = query.transpose(1, 2), key.transpose(1, 2)
+    # The reference copies [B, 3, N] clouds to [B, N, 3] here; the kernel reads either.
     query, key = query.contiguous(), key.contiguous()
-    return BallQueryFunction.apply(query, key, radius, max_neighbors)
+    return BallQueryFunction.apply(query, key, radius, max_neighbors, bool(transpose))

@@ -1,7 +1,7 @@
 """Weighted feature interpolation (API of torkit3d/ops/interpolate_feature.py)."""
 import torch
 
-from .. import _C
+from .. import _C, _fused
 
 
 class InterpolateFeature(torch.autograd.Function):
@@ -35,3 +35,19 @@ def three_nn_weights(distance, eps=1e-10):
     squared distance returned by ``knn_points``."""
     inv_distance = 1.0 / torch.clamp(distance, min=eps)
     return inv_distance / torch.sum(inv_distance, dim=2, keepdim=True)
+
+
+def three_nn_interpolation(query_xyz, key_xyz, transpose=False, eps=1e-10):
+    """Index and weight of the reference's FeatureInterpolator in one kernel:
+    ``knn_points(query, key, 3)`` followed by ``three_nn_weights``
+    (torkit3d/layers/pointnet2.py:125-130).
+
+    Args:
+        query_xyz: [B, N1, 3] ([B, 3, N1] if ``transpose``); key_xyz likewise.
+
+    Returns:
+        distance [B, N1, 3] (squared, MinK slot order), index [B, N1, 3] int64,
+        weight [B, N1, 3]. Not differentiable, as in the reference (``no_grad``).
+    """
+    with torch.no_grad():
+        return _fused.three_nn(query_xyz.contiguous(), key_xyz.contiguous(), bool(transpose), eps)

@@ -1,21 +1,26 @@
 """Farthest point sampling (API of torkit3d/ops/sample_farthest_points.py)."""
 import torch
 
-from .. import _C
+from .. import _C, _fused
 
 
 class SampleFarthestPointsFunction(torch.autograd.Function):
-    """Not differentiable (torkit3d/ops/sample_farthest_points.py:6-14)."""
+    """Not differentiable (torkit3d/ops/sample_farthest_points.py:6-14).
+    ``channels_first`` (not in the reference) says the cloud is [B, 3, N]."""
 
     @staticmethod
-    def forward(ctx, points, num_samples):
-        index = _C.sample_farthest_points_cuda(points, num_samples)
+    def forward(ctx, points, num_samples, channels_first=False):
+        if channels_first:
+            index, _ = _fused.sample_farthest_points_gather(points, num_samples, True,
+                                                            want_xyz=False)
+        else:
+            index = _C.sample_farthest_points_cuda(points, num_samples)
         ctx.mark_non_differentiable(index)
         return index
 
     @staticmethod
     def backward(ctx, *grad_outputs):
-        return (None,) * 2
+        return (None,) * 3
 
 
 def sample_farthest_points(points, num_samples, transpose=False):
@@ -27,7 +32,19 @@ def sample_farthest_points(points, num_samples, transpose=False):
     Returns:
         index [B, num_samples] int64.
     """
-    if transpose:
-        points = points.transpose(1, 2)
-    points = points.contiguous()
-    return SampleFarthestPointsFunction.apply(points, num_samples)
+    # The reference copies a [B, 3, N] cloud to [B, N, 3] here; the kernel reads either.
+    return SampleFarthestPointsFunction.apply(points.contiguous(), num_samples, bool(transpose))
+
+
+def sample_farthest_points_gather(points, num_samples, transpose=False):
+    """``sample_farthest_points`` plus the coordinates of the picks, from the same
+    kernel (the reference's models follow the op with
+    ``batch_index_select(points, index, dim=2)``, models/segmentation/pointnet2.py:89-90).
+
+    Returns:
+        index [B, num_samples] int64, sampled [B, num_samples, 3]
+        ([B, 3, num_samples] if ``transpose``). Not differentiable.
+    """
+    with torch.no_grad():
+        return _fused.sample_farthest_points_gather(points.contiguous(), num_samples,
+                                                    bool(transpose))
