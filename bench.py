@@ -209,7 +209,37 @@ def secondary_metrics(dev, steps, warmup, cpu):
     out["sa_chain_B8_16384_4096_1024_256_ms"] = gpu_time_ms(run_chain, max(3, steps // 10), 2)
     out["fps_B8_N16384_K4096_ms"] = gpu_time_ms(
         lambda: _C.sample_farthest_points_cuda(chain[0][0], 4096), max(3, steps // 10), 1)
-    res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()}}
+    # Fused callers against the composition of ops the reference's layers run.
+    from torkit3d_amd import _fused
+    from torkit3d_amd.ops.interpolate_feature import three_nn_weights as weights_of
+
+    fused = {}
+    xyz_bcn = xyz.transpose(1, 2).contiguous()
+    ctr_bcn = ctr.transpose(1, 2).contiguous()
+
+    def unfused_grouping():
+        grouped_xyz = _C.group_points_forward_cuda(xyz_bcn, nbr) - ctr_bcn.unsqueeze(-1)
+        return torch.cat([_C.group_points_forward_cuda(feat, nbr), grouped_xyz], dim=1)
+
+    fused["sa_grouping_C64_unfused_ms"] = gpu_time_ms(unfused_grouping, steps, 3)
+    fused["sa_grouping_C64_fused_ms"] = gpu_time_ms(
+        lambda: _fused.group_points_concat_forward(feat, xyz_bcn, ctr_bcn, nbr), steps, 3)
+    fused["ball_query_from_bcn_unfused_ms"] = gpu_time_ms(
+        lambda: _C.ball_query_cuda(ctr_bcn.transpose(1, 2).contiguous(),
+                                   xyz_bcn.transpose(1, 2).contiguous(), 0.2, 32), steps, 3)
+    fused["ball_query_from_bcn_fused_ms"] = gpu_time_ms(
+        lambda: _fused.ball_query_bcn(ctr_bcn, xyz_bcn, 0.2, 32), steps, 3)
+
+    def unfused_three_nn():
+        d2_, i_ = _C.knn_distance_cuda(q, key, 3, 1)
+        return i_, weights_of(d2_)
+
+    fused["three_nn_weights_unfused_ms"] = gpu_time_ms(unfused_three_nn, steps, 3)
+    fused["three_nn_weights_fused_ms"] = gpu_time_ms(
+        lambda: _fused.three_nn(q, key, False), steps, 3)
+
+    res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()},
+           "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()}}
     if cpu:
         res["cpu_oracle_ms"] = cpu_out
         res["cpu_oracle_note"] = ("OpenMP oracle on %d threads, timed on the first 2-4 clouds of each "

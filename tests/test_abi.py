@@ -84,6 +84,23 @@ def test_argument_errors_are_reported_without_launching(lib):
         assert interp(FAKE, FAKE, FAKE, i64(1), i64(2), i64(4), i64(4), i64(9), FAKE, NULL) == -3
         group = getattr(lib, "tk3d_group_points_backward" + sfx)
         assert group(FAKE, FAKE, i64(1), i64(-2), i64(4), i64(4), i64(2), FAKE, NULL) == -2
+        # entry points that fuse Python-side steps of the reference
+        ball = getattr(lib, "tk3d_ball_query_bcn" + sfx)
+        assert ball(FAKE, FAKE, i64(1), i64(4), i64(4), ctypes.c_float(0.1), i64(-1), FAKE, NULL) == -3
+        assert ball(NULL, FAKE, i64(1), i64(4), i64(4), ctypes.c_float(0.1), i64(2), FAKE, NULL) == -1
+        fps = getattr(lib, "tk3d_sample_farthest_points_gather" + sfx)
+        assert fps(FAKE, 1, i64(1), i64(10), i64(11), FAKE, NULL, NULL, ctypes.c_size_t(0), NULL) == -3
+        assert fps(NULL, 0, i64(1), i64(10), i64(5), FAKE, NULL, NULL, ctypes.c_size_t(0), NULL) == -1
+        nn3 = getattr(lib, "tk3d_three_nn" + sfx)
+        eps = ctypes.c_double(1e-10)
+        assert nn3(FAKE, FAKE, 0, i64(1), i64(8), i64(2), eps, FAKE, FAKE, FAKE, NULL) == -3
+        assert nn3(FAKE, FAKE, 1, i64(1), i64(8), i64(4), eps, FAKE, FAKE, NULL, NULL) == -1
+        assert nn3(NULL, NULL, 1, i64(0), i64(8), i64(4), eps, NULL, NULL, NULL, NULL) == 0
+        cat = getattr(lib, "tk3d_group_points_concat_forward" + sfx)
+        assert cat(NULL, FAKE, FAKE, FAKE, i64(1), i64(2), i64(4), i64(4), i64(2), FAKE, NULL) == -1
+        assert cat(NULL, FAKE, FAKE, FAKE, i64(1), i64(0), i64(4), i64(-4), i64(2), FAKE, NULL) == -2
+        cat = getattr(lib, "tk3d_group_points_concat_backward" + sfx)
+        assert cat(FAKE, FAKE, i64(1), i64(2), i64(4), i64(4), i64(2), NULL, NULL, NULL) == 0
 
 
 def test_fps_workspace_size(lib):

@@ -97,3 +97,56 @@ def test_three_nn_weights_matches_reference_recipe():
     w = interpolate_feature.three_nn_weights(d2)
     inv = 1.0 / torch.clamp(d2, min=1e-10)
     assert torch.equal(w, inv / inv.sum(2, keepdim=True))
+
+
+def test_layers_keep_the_reference_constructors():
+    # torkit3d/layers/pointnet2.py:16, :72, :91, :109 and the sub-module names its
+    # checkpoints are keyed by (torkit3d/nn/modules/conv.py:18-23)
+    from torkit3d_amd.layers import pointnet2
+
+    assert params(pointnet2.SetAbstraction.__init__)[1:] == [
+        ("in_channels", E), ("mlp_channels", E), ("query_neighbor", E), ("use_xyz", E)]
+    assert params(pointnet2.BallQuery.__init__)[1:] == [("radius", E), ("max_neighbors", E)]
+    assert params(pointnet2.FeaturePropagation.__init__)[1:] == [
+        ("in_channels", E), ("mlp_channels", E)]
+    assert params(pointnet2.FeatureInterpolator.__init__)[1:] == [
+        ("num_neighbors", 3), ("eps", 1e-10)]
+    assert params(pointnet2.SetAbstraction.forward)[1:] == [
+        ("in_xyz", E), ("out_xyz", E), ("in_feature", E)]
+    assert params(pointnet2.FeaturePropagation.forward)[1:] == [
+        ("in_xyz", E), ("in_feature", E), ("out_xyz", E), ("out_feature", None)]
+    sa = pointnet2.SetAbstraction(4, [8, 16], pointnet2.BallQuery(0.2, 8), True)
+    assert sorted(sa.state_dict()) == sorted(
+        ["mlp.%d.%s" % (i, k) for i in range(2) for k in (
+            "conv.weight", "bn.weight", "bn.bias", "bn.running_mean", "bn.running_var",
+            "bn.num_batches_tracked")])
+    assert sa.mlp[0].conv.in_channels == 7 and sa.out_channels == 16
+    fp = pointnet2.FeaturePropagation(10, [6])
+    assert "mlp.0.conv.weight" in fp.state_dict() and fp.mlp[0].conv.kernel_size == (1,)
+
+
+def test_batch_index_select_is_a_batched_gather():
+    from torkit3d_amd.nn import batch_index_select
+
+    x = torch.arange(2 * 3 * 5.0).reshape(2, 3, 5)
+    idx = torch.tensor([[4, 0], [1, 1]])
+    out = batch_index_select(x, idx, dim=2)
+    assert out.shape == (2, 3, 2)
+    assert torch.equal(out[0], x[0][:, [4, 0]]) and torch.equal(out[1], x[1][:, [1, 1]])
+    assert torch.equal(batch_index_select(x, torch.tensor([2, 0]), dim=1),
+                       torch.stack([x[0, 2], x[1, 0]]))
+
+
+def test_fused_entry_points_reject_cpu_tensors():
+    from torkit3d_amd import _fused
+
+    x = torch.zeros(1, 3, 8)
+    idx = torch.zeros(1, 8, 2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _fused.ball_query_bcn(x, x, 0.1, 2)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _fused.sample_farthest_points_gather(x, 2, True)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _fused.three_nn(x, x, True)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _fused.group_points_concat_forward(None, x, x, idx)

@@ -75,6 +75,14 @@ template <typename T> __device__ __forceinline__ T wave_max(T v)
     return read_lane(v, 63);
 }
 
+// Coordinate `a` of point `j`: clouds are [n,3] rows, or with SOA three planes [3,n]
+// (the layout the reference's models keep their clouds in).
+template <bool SOA, typename T>
+__device__ __forceinline__ T fps_coord(const T *__restrict__ pts, int n, int64_t j, int a)
+{
+    return SOA ? pts[(int64_t)a * n + j] : pts[j * 3 + a];
+}
+
 struct FpsLayout {
     int n;        // points per cloud
     int k;        // samples per cloud
@@ -82,10 +90,6 @@ struct FpsLayout {
     int log2_bs;
     int c;        // ceil(n / bs): points per reference thread
     float inv_c;  // 1 / c
-    // Element strides of the coordinate arrays: point j, axis a sits at j*ps + a*cs.
-    // [B,N,3] clouds have (3, 1), [B,3,N] clouds (1, N); a batch is n*3 elements in both.
-    int ps, cs;    // input cloud
-    int ops, ocs;  // optional output of the sampled coordinates ([B,K,3] or [B,3,K])
 };
 
 // Point index of a position in the priority order described at the top.
@@ -100,10 +104,9 @@ __device__ __forceinline__ int fps_point_of_position(int pos, const FpsLayout &L
     return t + cc * L.bs;
 }
 
-template <typename T, int P, int NT>
+template <typename T, int P, int NT, bool SOA>
 __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ points,
                                                           int64_t *__restrict__ index,
-                                                          T *__restrict__ sampled,
                                                           FpsLayout L)
 {
     constexpr int NW = NT / TK_WAVE;
@@ -123,24 +126,18 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
         const int pos = tid * P + p;
         const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
         const bool ok = j < L.n;
-        x[p] = ok ? pts[(int64_t)j * L.ps] : (T)0;
-        y[p] = ok ? pts[(int64_t)j * L.ps + L.cs] : (T)0;
-        z[p] = ok ? pts[(int64_t)j * L.ps + 2 * L.cs] : (T)0;
+        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : (T)0;
+        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : (T)0;
+        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : (T)0;
         // Unused slots sit at -1: min() keeps them there and they never exceed 0.
         md[p] = ok ? tk_inf<T>() : (T)-1;
     }
 
     int sel_j = 0;
-    T cx = pts[0], cy = pts[L.cs], cz = pts[2 * L.cs];
-    T *__restrict__ so = sampled ? sampled + (int64_t)blockIdx.x * L.k * 3 : nullptr;
-    if (tid == 0) {
+    T cx = fps_coord<SOA>(pts, L.n, 0, 0), cy = fps_coord<SOA>(pts, L.n, 0, 1),
+      cz = fps_coord<SOA>(pts, L.n, 0, 2);
+    if (tid == 0)
         out[0] = 0;
-        if (so) {
-            so[0] = cx;
-            so[L.ocs] = cy;
-            so[2 * L.ocs] = cz;
-        }
-    }
 
     for (int it = 1; it < L.k; ++it) {
         // Lane-local update and first maximum above zero (strict '>' from zero, as
@@ -195,14 +192,8 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
         }
         // gmax == 0: no point lies away from the chosen set; the previous choice
         // is emitted again, as the reference does.
-        if (tid == 0) {
+        if (tid == 0)
             out[it] = (int64_t)sel_j;
-            if (so) {
-                so[(int64_t)it * L.ops] = cx;
-                so[(int64_t)it * L.ops + L.ocs] = cy;
-                so[(int64_t)it * L.ops + 2 * L.ocs] = cz;
-            }
-        }
     }
 }
 
@@ -282,10 +273,9 @@ template <int P, int NODE> struct FpsWalk {
     }
 };
 
-template <int P, int NT>
+template <int P, int NT, bool SOA>
 __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__restrict__ points,
                                                               int64_t *__restrict__ index,
-                                                              float *__restrict__ sampled,
                                                               FpsLayout L)
 {
     static_assert((P & (P - 1)) == 0, "P must be a power of two");
@@ -309,25 +299,19 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
         const int pos = tid * P + p;
         const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
         const bool ok = j < L.n;
-        x[p] = ok ? pts[(int64_t)j * L.ps] : 0.0f;
-        y[p] = ok ? pts[(int64_t)j * L.ps + L.cs] : 0.0f;
-        z[p] = ok ? pts[(int64_t)j * L.ps + 2 * L.cs] : 0.0f;
+        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : 0.0f;
+        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : 0.0f;
+        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : 0.0f;
         jv[p] = j;
         t[P + p] = ok ? F32_INF : F32_NEG1;
     }
     t[0] = 0;
 
     int sel_j = 0;
-    float cx = pts[0], cy = pts[L.cs], cz = pts[2 * L.cs];
-    float *__restrict__ so = sampled ? sampled + (int64_t)blockIdx.x * L.k * 3 : nullptr;
-    if (tid == 0) {
+    float cx = fps_coord<SOA>(pts, L.n, 0, 0), cy = fps_coord<SOA>(pts, L.n, 0, 1),
+          cz = fps_coord<SOA>(pts, L.n, 0, 2);
+    if (tid == 0)
         out[0] = 0;
-        if (so) {
-            so[0] = cx;
-            so[L.ocs] = cy;
-            so[2 * L.ocs] = cz;
-        }
-    }
 
     for (int it = 1; it < L.k; ++it) {
 #pragma unroll
@@ -368,24 +352,17 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
             cy = read_lane(mine.y, gl);
             cz = read_lane(mine.z, gl);
         }
-        if (tid == 0) {
+        if (tid == 0)
             out[it] = (int64_t)sel_j;
-            if (so) {
-                so[(int64_t)it * L.ops] = cx;
-                so[(int64_t)it * L.ops + L.ocs] = cy;
-                so[(int64_t)it * L.ops + 2 * L.ocs] = cz;
-            }
-        }
     }
 }
 
 // Clouds that do not fit in registers: minimum distances live in a global
 // workspace, coordinates are re-read every step (they stay in L2). Same selection
 // rule; positions are visited in priority order so the tie rule is unchanged.
-template <typename T, int NT>
+template <typename T, int NT, bool SOA>
 __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__ points,
                                                            int64_t *__restrict__ index,
-                                                           T *__restrict__ sampled,
                                                            T *__restrict__ min_dist,
                                                            FpsLayout L)
 {
@@ -412,14 +389,8 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
     if (tid == 0)
         out[0] = 0;
     for (int it = 1; it < L.k; ++it) {
-        const T cx = pts[(int64_t)sel_j * L.ps], cy = pts[(int64_t)sel_j * L.ps + L.cs],
-                cz = pts[(int64_t)sel_j * L.ps + 2 * L.cs];
-        if (tid == 0 && sampled) {  // coordinates of sample it-1
-            T *so = sampled + (int64_t)blockIdx.x * L.k * 3 + (int64_t)(it - 1) * L.ops;
-            so[0] = cx;
-            so[L.ocs] = cy;
-            so[2 * L.ocs] = cz;
-        }
+        const T cx = fps_coord<SOA>(pts, L.n, sel_j, 0), cy = fps_coord<SOA>(pts, L.n, sel_j, 1),
+                cz = fps_coord<SOA>(pts, L.n, sel_j, 2);
         T best = (T)0;
         int bpos = 0;
         for (int pos = p0; pos < p1; ++pos) {
@@ -427,8 +398,8 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
             if (m < (T)0)
                 continue;
             const int j = fps_point_of_position(pos, L);
-            const T d = tk_dist2<T>(pts[(int64_t)j * L.ps], pts[(int64_t)j * L.ps + L.cs],
-                                    pts[(int64_t)j * L.ps + 2 * L.cs], cx, cy, cz);
+            const T d = tk_dist2<T>(fps_coord<SOA>(pts, L.n, j, 0), fps_coord<SOA>(pts, L.n, j, 1),
+                                    fps_coord<SOA>(pts, L.n, j, 2), cx, cy, cz);
             const T nm = tk_min<T>(m, d);
             md[pos] = nm;
             if (nm > best) {
@@ -455,23 +426,13 @@ __global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__
         if (tid == 0)
             out[it] = (int64_t)sel_j;
     }
-    if (tid == 0 && sampled) {  // coordinates of the last sample
-        T *so = sampled + (int64_t)blockIdx.x * L.k * 3 + (int64_t)(L.k - 1) * L.ops;
-        so[0] = pts[(int64_t)sel_j * L.ps];
-        so[L.ocs] = pts[(int64_t)sel_j * L.ps + L.cs];
-        so[2 * L.ocs] = pts[(int64_t)sel_j * L.ps + 2 * L.cs];
-    }
 }
 
-FpsLayout fps_layout(int64_t n, int64_t k, bool channels_first = false)
+FpsLayout fps_layout(int64_t n, int64_t k)
 {
     FpsLayout L;
     L.n = (int)n;
     L.k = (int)k;
-    L.ps = channels_first ? 1 : 3;
-    L.cs = channels_first ? (int)n : 1;
-    L.ops = channels_first ? 1 : 3;
-    L.ocs = channels_first ? (int)k : 1;
     int bs = 1, lg = 0;
     // Block size of the reference: smallest power of two >= n, capped at 512
     // (sample_farthest_points_kernel.cu:132-133); its switch runs 32 threads for
@@ -495,46 +456,99 @@ FpsLayout fps_layout(int64_t n, int64_t k, bool channels_first = false)
 int64_t fps_register_capacity(size_t es) { return es == 4 ? 1024 * 16 : 1024 * 8; }
 
 template <typename T, int P, int NT>
-void fps_launch(const T *points, int64_t B, int64_t *index, T *sampled, const FpsLayout &L,
+void fps_launch(const T *points, bool soa, int64_t B, int64_t *index, const FpsLayout &L,
                 hipStream_t s)
 {
-    hipLaunchKernelGGL((fps_register_kernel<T, P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
-                       points, index, sampled, L);
+    if (soa)
+        hipLaunchKernelGGL((fps_register_kernel<T, P, NT, true>), dim3((unsigned)B), dim3(NT), 0,
+                           s, points, index, L);
+    else
+        hipLaunchKernelGGL((fps_register_kernel<T, P, NT, false>), dim3((unsigned)B), dim3(NT),
+                           0, s, points, index, L);
 }
 
 template <int P, int NT>
-void fps_launch_f32(const float *points, int64_t B, int64_t *index, float *sampled,
+void fps_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
                     const FpsLayout &L, hipStream_t s)
 {
-    hipLaunchKernelGGL((fps_register_kernel_f32<P, NT>), dim3((unsigned)B), dim3(NT), 0, s,
-                       points, index, sampled, L);
+    if (soa)
+        hipLaunchKernelGGL((fps_register_kernel_f32<P, NT, true>), dim3((unsigned)B), dim3(NT),
+                           0, s, points, index, L);
+    else
+        hipLaunchKernelGGL((fps_register_kernel_f32<P, NT, false>), dim3((unsigned)B), dim3(NT),
+                           0, s, points, index, L);
 }
 
 // fp32: (points per lane, lanes) by cloud size, from timing every shape on an
 // MI355X: two waves per SIMD (512 lanes) hide each other's reduction latency; more
 // waves only repeat the per-wave reduction.
-void fps_dispatch_f32(const float *points, int64_t B, int64_t *index, float *sampled,
+void fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
                       const FpsLayout &L, int64_t npos, hipStream_t s)
 {
     if (npos <= 64 * 2)
-        fps_launch_f32<2, 64>(points, B, index, sampled, L, s);
+        fps_launch_f32<2, 64>(points, soa, B, index, L, s);
     else if (npos <= 256 * 2)
-        fps_launch_f32<2, 256>(points, B, index, sampled, L, s);
+        fps_launch_f32<2, 256>(points, soa, B, index, L, s);
     else if (npos <= 512 * 2)
-        fps_launch_f32<2, 512>(points, B, index, sampled, L, s);
+        fps_launch_f32<2, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 4)
-        fps_launch_f32<4, 512>(points, B, index, sampled, L, s);
+        fps_launch_f32<4, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 8)
-        fps_launch_f32<8, 512>(points, B, index, sampled, L, s);
+        fps_launch_f32<8, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 16)
-        fps_launch_f32<16, 512>(points, B, index, sampled, L, s);
+        fps_launch_f32<16, 512>(points, soa, B, index, L, s);
     else
-        fps_launch_f32<32, 512>(points, B, index, sampled, L, s);
+        fps_launch_f32<32, 512>(points, soa, B, index, L, s);
+}
+
+// Coordinates of the picks: sampled[b, i, :] = points[b, index[b, i], :] in the layout of
+// the input cloud ([B,K,3], or [B,3,K] with SOA). A launch of its own after the
+// selection kernel: storing the coordinates from the selection loop changed that loop's
+// register allocation and cost it 4-9 %, far more than this pass.
+template <typename T, bool SOA>
+__global__ __launch_bounds__(256) void fps_gather_kernel(const T *__restrict__ points,
+                                                         const int64_t *__restrict__ index,
+                                                         T *__restrict__ sampled, int n, int k)
+{
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= k)
+        return;
+    const T *__restrict__ pts = points + (int64_t)b * n * 3;
+    T *__restrict__ so = sampled + (int64_t)b * k * 3;
+    const int64_t j = index[(int64_t)b * k + i];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const T v = fps_coord<SOA>(pts, n, j, a);
+        if (SOA)
+            so[(int64_t)a * k + i] = v;
+        else
+            so[(int64_t)i * 3 + a] = v;
+    }
 }
 
 template <typename T>
-int fps(const T *points, bool channels_first, int64_t B, int64_t N, int64_t K, int64_t *index,
-        T *sampled, void *workspace, size_t workspace_bytes, void *stream)
+int fps_finish(const T *points, bool soa, int64_t B, int64_t N, int64_t K,
+               const int64_t *index, T *sampled, hipStream_t s)
+{
+    const int rc = tk_launch_status();
+    if (rc != TK3D_OK || !sampled)
+        return rc;
+    const dim3 grid((unsigned)((K + 255) / 256), (unsigned)B);
+    if (B > 65535)
+        return TK3D_ERR_UNSUPPORTED;
+    if (soa)
+        hipLaunchKernelGGL((fps_gather_kernel<T, true>), grid, dim3(256), 0, s, points, index,
+                           sampled, (int)N, (int)K);
+    else
+        hipLaunchKernelGGL((fps_gather_kernel<T, false>), grid, dim3(256), 0, s, points, index,
+                           sampled, (int)N, (int)K);
+    return tk_launch_status();
+}
+
+template <typename T>
+int fps(const T *points, bool soa, int64_t B, int64_t N, int64_t K, int64_t *index, T *sampled,
+        void *workspace, size_t workspace_bytes, void *stream)
 {
     if (B < 0 || N < 0)
         return TK3D_ERR_BAD_SIZE;
@@ -547,36 +561,40 @@ int fps(const T *points, bool channels_first, int64_t B, int64_t N, int64_t K, i
     if (!points || !index)
         return TK3D_ERR_NULL_POINTER;
     hipStream_t s = (hipStream_t)stream;
-    const FpsLayout L = fps_layout(N, K, channels_first);
+    const FpsLayout L = fps_layout(N, K);
     const int64_t npos = (int64_t)L.bs * L.c;
     if (npos <= fps_register_capacity(sizeof(T))) {
         if constexpr (sizeof(T) == 4) {
-            fps_dispatch_f32(points, B, index, sampled, L, npos, s);
-            return tk_launch_status();
+            fps_dispatch_f32(points, soa, B, index, L, npos, s);
+            return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
         }
         // Fewest points per lane that still covers the cloud: short serial chains.
         if (npos <= 256 * 1)
-            fps_launch<T, 1, 256>(points, B, index, sampled, L, s);
+            fps_launch<T, 1, 256>(points, soa, B, index, L, s);
         else if (npos <= 256 * 2)
-            fps_launch<T, 2, 256>(points, B, index, sampled, L, s);
+            fps_launch<T, 2, 256>(points, soa, B, index, L, s);
         else if (npos <= 512 * 2)
-            fps_launch<T, 2, 512>(points, B, index, sampled, L, s);
+            fps_launch<T, 2, 512>(points, soa, B, index, L, s);
         else if (npos <= 1024 * 2)
-            fps_launch<T, 2, 1024>(points, B, index, sampled, L, s);
+            fps_launch<T, 2, 1024>(points, soa, B, index, L, s);
         else if (npos <= 1024 * 4)
-            fps_launch<T, 4, 1024>(points, B, index, sampled, L, s);
+            fps_launch<T, 4, 1024>(points, soa, B, index, L, s);
         else if (npos <= 1024 * 8)
-            fps_launch<T, 8, 1024>(points, B, index, sampled, L, s);
+            fps_launch<T, 8, 1024>(points, soa, B, index, L, s);
         else if constexpr (sizeof(T) == 4)
-            fps_launch<T, 16, 1024>(points, B, index, sampled, L, s);
-        return tk_launch_status();
+            fps_launch<T, 16, 1024>(points, soa, B, index, L, s);
+        return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
     }
     const size_t need = (size_t)B * (size_t)npos * sizeof(T);
     if (!workspace || workspace_bytes < need)
         return TK3D_ERR_WORKSPACE;
-    hipLaunchKernelGGL((fps_streaming_kernel<T, 1024>), dim3((unsigned)B), dim3(1024), 0, s,
-                       points, index, sampled, (T *)workspace, L);
-    return tk_launch_status();
+    if (soa)
+        hipLaunchKernelGGL((fps_streaming_kernel<T, 1024, true>), dim3((unsigned)B), dim3(1024),
+                           0, s, points, index, (T *)workspace, L);
+    else
+        hipLaunchKernelGGL((fps_streaming_kernel<T, 1024, false>), dim3((unsigned)B), dim3(1024),
+                           0, s, points, index, (T *)workspace, L);
+    return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
 }
 
 }  // namespace
