@@ -148,3 +148,82 @@ def test_interpolate_only_k3_through_the_reference_interface(cuda):
         _C.interpolate_forward_cuda(feat, idx, w)
     with pytest.raises(RuntimeError, match="Only support k=3"):
         _C.interpolate_backward_cuda(torch.zeros(1, 2, 4, device=cuda), idx, w, 5)
+
+
+def test_fp32_backward_is_bit_reproducible(cuda):
+    # fp32 scatters accumulate in 64-bit fixed point: integer adds commute, so repeated
+    # calls give identical bits (the reference's float atomics do not)
+    from torkit3d_amd import _C
+
+    g = gen(21)
+    index = torch.randint(0, 2048, (8, 4096, 3), generator=g).to(cuda)
+    weight = torch.rand(8, 4096, 3, generator=g).to(cuda)
+    go = torch.randn(8, 64, 4096, generator=g).to(cuda)
+    first = _C.interpolate_backward_cuda(go, index, weight, 2048)
+    gindex = torch.randint(0, 4096, (8, 1024, 32), generator=g).to(cuda)
+    ggo = torch.randn(8, 32, 1024, 32, generator=g).to(cuda)
+    gfirst = _C.group_points_backward_cuda(ggo, gindex, 4096)
+    a = torch.randn(4, 5000, 3, generator=g).to(cuda)
+    c = torch.randn(4, 3000, 3, generator=g).to(cuda)
+    _, i1, _, i2 = _C.chamfer_distance_forward_cuda(a, c)
+    gd1 = torch.randn(4, 5000, generator=g).to(cuda)
+    gd2 = torch.randn(4, 3000, generator=g).to(cuda)
+    cfirst = _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2)
+    for _ in range(3):
+        assert torch.equal(_C.interpolate_backward_cuda(go, index, weight, 2048), first)
+        assert torch.equal(_C.group_points_backward_cuda(ggo, gindex, 4096), gfirst)
+        again = _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2)
+        assert torch.equal(again[0], cfirst[0]) and torch.equal(again[1], cfirst[1])
+
+
+@pytest.mark.parametrize("where", [100, 2500, 4095])
+def test_scatter_outlier_missed_by_the_magnitude_sample(cuda, where):
+    # The fixed-point scale comes from a 1-in-8 sample of the gradient; a term far above
+    # the sampled maximum must send the workgroup through its exact second pass.
+    from torkit3d_amd import _C
+
+    g = gen(22)
+    index = torch.randint(0, 512, (2, 4096, 3), generator=g)
+    weight = torch.rand(2, 4096, 3, generator=g)
+    go = torch.randn(2, 16, 4096, generator=g)
+    go[1, 5, where] = 3.0e7  # 2^25 times a typical term
+    got = _C.interpolate_backward_cuda(go.to(cuda), index.to(cuda), weight.to(cuda), 512)
+    want = oracle.interpolate_backward(go.numpy(), index.numpy(), weight.numpy(), 512)
+    got, want = got.cpu().numpy(), want
+    # the row with the outlier is resolved to 2^-40 of its largest term per sum, every
+    # other row to fp32 accuracy
+    np.testing.assert_allclose(got[1, 5], want[1, 5], rtol=RTOL, atol=3.0e7 * 2.0 ** -40)
+    got[1, 5] = want[1, 5]
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=2e-5)
+    gidx = torch.randint(0, 512, (2, 1024, 4), generator=g)
+    ggo = torch.randn(2, 16, 1024, 4, generator=g)
+    ggo.view(2, 16, -1)[0, 3, where] = -1.0e8
+    got = _C.group_points_backward_cuda(ggo.to(cuda), gidx.to(cuda), 512).cpu().numpy()
+    want = oracle.group_backward(ggo.numpy(), gidx.numpy(), 512)
+    np.testing.assert_allclose(got[0, 3], want[0, 3], rtol=RTOL, atol=1.0e8 * 2.0 ** -40)
+    got[0, 3] = want[0, 3]
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=2e-5)
+
+
+def test_scatter_non_finite_gradients_follow_float_arithmetic(cuda):
+    # inf and NaN have no fixed-point image: such a row falls back to float atomics and
+    # must give what float addition gives (inf stays inf, inf - inf and NaN give NaN)
+    from torkit3d_amd import _C
+
+    g = gen(23)
+    index = torch.randint(0, 256, (2, 2048, 3), generator=g)
+    weight = torch.rand(2, 2048, 3, generator=g) + 0.1
+    go = torch.randn(2, 8, 2048, generator=g)
+    go[0, 1, 7] = float("inf")
+    go[0, 2, 9] = float("nan")
+    go[1, 3, 11] = float("inf")
+    go[1, 3, 12] = -float("inf")
+    index[1, 12] = index[1, 11]  # +inf and -inf meet in the same rows
+    got = _C.interpolate_backward_cuda(go.to(cuda), index.to(cuda), weight.to(cuda), 256).cpu().numpy()
+    want = oracle.interpolate_backward(go.numpy(), index.numpy(), weight.numpy(), 256)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isposinf(got), np.isposinf(want))
+    assert np.array_equal(np.isneginf(got), np.isneginf(want))
+    finite = np.isfinite(want)
+    assert np.isnan(want).any() and np.isinf(want).any()
+    np.testing.assert_allclose(got[finite], want[finite], rtol=RTOL, atol=2e-5)

@@ -778,7 +778,7 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
             atomicMax(&s_max, m);
         __syncthreads();
         TK3D_STAMP(1 + attempt * 4);
-        const float bound = __builtin_bit_cast(float, s_max) * (attempt == 0 ? 64.0f : 1.000001f);
+        const float bound = __builtin_bit_cast(float, s_max) * (attempt == 0 ? 8.0f : 1.000001f);
         if (!(bound < 3.0e38f)) {  // NaN or inf
             use_float = true;
             break;
@@ -1014,17 +1014,11 @@ int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
         constexpr int R = 4096, NT = 1024;
         const int64_t r1 = (N1 + R - 1) / R, r2 = (N2 + R - 1) / R;
         if (B * (r1 + r2) <= TK_MAX_I32) {
-            auto kernel = chamfer_backward_fixed_kernel<R, NT>;
+            constexpr auto kernel = chamfer_backward_fixed_kernel<R, NT>;
             constexpr size_t lds = (size_t)R * 3 * sizeof(unsigned long long);
-            static bool lds_opt_in = false;  // raising the limit is idempotent
-            if (!lds_opt_in) {
-                const hipError_t e = hipFuncSetAttribute(
-                    reinterpret_cast<const void *>(kernel),
-                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                if (e != hipSuccess)
-                    return (int)e;
-                lds_opt_in = true;
-            }
+            const int allowed = tk_allow_dynamic_lds<kernel>((int)lds);
+            if (allowed != TK3D_OK)
+                return allowed;
             hipLaunchKernelGGL(kernel, dim3((unsigned)(B * (r1 + r2))), dim3(NT), lds, s, gd1,
                                gd2, xyz1, xyz2, idx1, idx2, (int)N1, (int)N2, (int)r1, (int)r2,
                                (int)(B * r1), gx1, gx2);

@@ -333,10 +333,12 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
 // integer at a per-row power-of-two scale and added with ds_add_u64:
 //   * magnitudes: the workgroup samples an eighth of its share of gout for max|g| per
 //     row and an eighth of w for max|w| (runs of 64 consecutive loads, one run in
-//     eight), and allows 64 times their product as the bound B_c of a row;
+//     eight), and allows 8 times their product as the bound B_c of a row;
 //   * scale: 2^k with k the largest integer keeping B_c * 2^k below 2^50 and
-//     count * B_c * 2^k below 2^62, i.e. a resolution of 2^-40 of the row maximum
-//     or better for up to 2^16 terms per row; fp32 accumulation resolves 2^-24;
+//     count * B_c * 2^k below 2^62, i.e. one term is resolved to 2^-43 of the row's
+//     largest term or better for up to 2^16 terms per row. The resolution is absolute
+//     within a row where fp32 accumulation's is relative to each sum: a row whose
+//     terms span more than 2^20 resolves its small sums worse than fp32 would;
 //   * conversion: fma(double(term), 2^k, 1.5 * 2^52) leaves the rounded integer in
 //     the low mantissa bits (one cvt, one fma, one 64-bit subtract);
 //   * a term above its row's bound (the sample missed an outlier) raises a flag;
@@ -469,7 +471,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         // ---- bounds and scales: lane c < CGMAX works out row c ----
         if (threadIdx.x < CGMAX) {
             const float maxw = __builtin_bit_cast(float, s_maxw);
-            const float headroom = attempt == 0 ? 64.0f : 1.000001f;
+            const float headroom = attempt == 0 ? 8.0f : 1.000001f;
             const float bound = __builtin_bit_cast(float, s_maxg[threadIdx.x]) * maxw * headroom;
             if (!(bound < 3.0e38f))  // NaN or inf (NaN has the largest bit pattern)
                 s_finite = 0;
@@ -721,16 +723,10 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
             int log2_count = 1;
             while (((int64_t)1 << log2_count) < seg_len * KK + 1)
                 ++log2_count;
-            auto kernel = scatter_fixed_kernel<KK, HAS_W, V, NT, CGMAX>;
-            static bool lds_opt_in = false;  // raising the limit is idempotent
-            if (!lds_opt_in) {
-                const hipError_t e = hipFuncSetAttribute(
-                    reinterpret_cast<const void *>(kernel),
-                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)FIXED_LDS);
-                if (e != hipSuccess)
-                    return (int)e;
-                lds_opt_in = true;
-            }
+            constexpr auto kernel = scatter_fixed_kernel<KK, HAS_W, V, NT, CGMAX>;
+            const int allowed = tk_allow_dynamic_lds<kernel>((int)FIXED_LDS);
+            if (allowed != TK3D_OK)
+                return allowed;
             if (nseg > 1)
                 hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
                                    dim3(GS_BLOCK), 0, s, gin, out_elems);

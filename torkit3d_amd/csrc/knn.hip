@@ -598,14 +598,10 @@ int knn_tree_launch(const float *query, const float *key, float *distance, int64
                     int64_t B, int n1, int n2, int k, hipStream_t s)
 {
     constexpr int LDS_BYTES = 13 * KMAX * 64;
-    static bool raised = false;  // per process; the attribute is sticky
-    if (LDS_BYTES > 48 * 1024 && !raised) {
-        const hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&knn_tree_kernel_f32<KMAX>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess)
-            return (int)e;
-        raised = true;
+    if (LDS_BYTES > 48 * 1024) {
+        const int allowed = tk_allow_dynamic_lds<knn_tree_kernel_f32<KMAX>>(LDS_BYTES);
+        if (allowed != TK3D_OK)
+            return allowed;
     }
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     if (B * bpb > TK_MAX_I32)

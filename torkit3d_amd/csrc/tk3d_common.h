@@ -2,6 +2,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include "tk3d.h"
@@ -67,6 +69,27 @@ static inline int tk_launch_status()
 {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? TK3D_OK : (int)e;
+}
+
+// Raises the dynamic LDS limit of `Kernel` to `bytes` on the current device; done once
+// per device and kernel (the attribute belongs to the device's copy of the code).
+// Returns TK3D_OK or the hipError_t.
+template <auto Kernel> static inline int tk_allow_dynamic_lds(int bytes)
+{
+    static std::atomic<unsigned long long> done{0};  // one bit per device ordinal
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return (int)e;
+    if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1ull))
+        return TK3D_OK;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess)
+        return (int)e;
+    if (dev >= 0 && dev < 64)
+        done.fetch_or(1ull << dev, std::memory_order_release);
+    return TK3D_OK;
 }
 
 // True when a*b*c... of non-negative sizes fits in int64 and is below `limit`.
