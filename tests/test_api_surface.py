@@ -150,3 +150,23 @@ def test_fused_entry_points_reject_cpu_tensors():
         _fused.three_nn(x, x, True)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         _fused.group_points_concat_forward(None, x, x, idx)
+
+
+def test_edge_conv_module_keeps_the_reference_api():
+    # torkit3d/ops/edge_conv.py:17, :48-50, :73-75, :96-97
+    from torkit3d_amd.ops import edge_conv
+
+    assert params(edge_conv.EdgeConvBlock.__init__)[1:] == [
+        ("in_channels", E), ("conv_channels", E), ("checkpoint", False)]
+    want = [("query_feature", E), ("key_feature", E), ("key_ind", E), ("include_query", True)]
+    assert params(edge_conv.get_edge_feature_builtin) == want
+    assert params(edge_conv.get_edge_feature_custom) == want
+    assert edge_conv.get_edge_feature is edge_conv.get_edge_feature_custom
+    block = edge_conv.EdgeConvBlock(3, [8])
+    assert "convs.0.conv.weight" in block.state_dict() and block.convs[0].conv.in_channels == 6
+    q = torch.randn(1, 3, 5)
+    idx = torch.tensor([[[0, 1], [1, 2], [2, 3], [3, 4], [4, 0]]])
+    edge = edge_conv.get_edge_feature_builtin(q, q, idx)
+    assert edge.shape == (1, 6, 5, 2)
+    assert torch.equal(edge[0, :3, 0, 1], q[0, :, 1] - q[0, :, 0])
+    assert torch.equal(edge[0, 3:, 2, 0], q[0, :, 2])

@@ -214,3 +214,30 @@ def test_errors(cuda):
         _fused.sample_farthest_points_gather(x, 9, True)
     with pytest.raises(RuntimeError):
         _fused.group_points_concat_forward(None, x, x, torch.zeros(2, 8, 2, device=cuda))
+
+
+def test_edge_features_match_the_gather_form(cuda):
+    # torkit3d/ops/edge_conv.py: the group_points form must equal the torch.gather form
+    from torkit3d_amd.ops.edge_conv import (EdgeConvBlock, get_edge_feature_builtin,
+                                            get_edge_feature_custom)
+    from torkit3d_amd.ops.knn_points import knn_points
+
+    g = gen(8)
+    feat = torch.randn(2, 6, 500, generator=g).to(cuda)
+    xyz = torch.rand(2, 500, 3, generator=g).to(cuda)
+    _, idx = knn_points(xyz, xyz, 8)
+    f1 = feat.clone().requires_grad_(True)
+    f2 = feat.clone().requires_grad_(True)
+    a = get_edge_feature_custom(f1, f1, idx)
+    b = get_edge_feature_builtin(f2, f2, idx)
+    assert a.shape == (2, 12, 500, 8) and torch.equal(a, b)
+    assert torch.equal(get_edge_feature_custom(feat, feat, idx, include_query=False), b[:, :6])
+    up = torch.randn(2, 12, 500, 8, generator=g).to(cuda)
+    a.backward(up)
+    b.backward(up)
+    torch.testing.assert_close(f1.grad, f2.grad, rtol=1e-5, atol=1e-5)
+    torch.manual_seed(0)
+    block = EdgeConvBlock(6, [16, 32], checkpoint=True).to(cuda)
+    out = block(f1, f1, idx)
+    assert out.shape == (2, 32, 500)
+    out.sum().backward()
