@@ -88,6 +88,48 @@ def test_ties_follow_the_reference_tree_order(cuda, n):
         assert not np.array_equal(want, oracle.sample_farthest_points(pts.numpy(), k, "lowest"))
 
 
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 64, 333])
+def test_every_sample_count_ends_on_the_right_step(cuda, k):
+    # the fp32 kernel takes several selection steps per exchange between its waves; the
+    # last exchange must stop exactly at num_samples
+    pts = torch.rand(3, 2000, 3, generator=gen(50 + k))
+    guard = torch.full((3, k + 8), -7, dtype=torch.int64, device=cuda)
+    from torkit3d_amd import _C
+
+    got = _C.sample_farthest_points_cuda(pts.to(cuda), k)
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.sample_farthest_points(pts.numpy(), k))
+    assert int(guard.min()) == -7
+
+
+@pytest.mark.parametrize("kind", ["clusters", "two_far_copies", "lattice_fine", "half_duplicates",
+                                  "line", "shell"])
+def test_multi_step_selection_on_adversarial_clouds(cuda, kind):
+    # clouds on which the candidates of different waves are close to each other, tie, or
+    # sit in the same wave: the shortcut must refuse exactly the steps it cannot prove
+    g = gen(60)
+    n = 4096
+    if kind == "clusters":      # 64 tight clusters: after 64 picks every candidate is tiny
+        centres = torch.rand(2, 64, 3, generator=g)
+        pts = centres[:, torch.randint(0, 64, (n,), generator=g)] + 1e-3 * torch.randn(2, n, 3, generator=g)
+    elif kind == "two_far_copies":  # every point twice: each maximum is held by two points
+        half = torch.rand(2, n // 2, 3, generator=g)
+        pts = torch.cat([half, half + torch.tensor([4.0, 0.0, 0.0])], dim=1)
+        pts = torch.cat([pts[:, ::2], pts[:, 1::2]], dim=1)
+    elif kind == "lattice_fine":
+        pts = lattice_cloud(g, 2, n, 3)
+    elif kind == "half_duplicates":
+        half = torch.rand(2, n // 2, 3, generator=g)
+        pts = torch.cat([half, half], dim=1)
+    elif kind == "line":         # points on a line: neighbours of a pick are the next picks
+        pts = torch.zeros(2, n, 3)
+        pts[:, :, 0] = torch.rand(2, n, generator=g)
+    else:                        # thin shell
+        u = torch.randn(2, n, 3, generator=g)
+        pts = u / u.norm(dim=2, keepdim=True)
+    k = 1500
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
+
+
 def test_duplicates_and_full_sample(cuda):
     ones = torch.ones(2, 500, 3)
     np.testing.assert_array_equal(run(ones, 20, cuda), np.zeros((2, 20), np.int64))

@@ -203,41 +203,21 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
 //     order like signed integers; integer min/max need no NaN canonicalisation
 //     and the -1.0f marker of unused slots (a negative integer) stays put;
 //   * a lane reduces its P minima through a binary tree of maxima kept in
-//     registers; the wave reduction is six v_max_i32 with DPP operands, written
-//     out because the compiler does not fold the lane moves into the max;
+//     registers; the wave reduction is a DPP scan written out by hand (the compiler
+//     does not fold the lane moves into the max) that carries the two largest values;
 //   * the winning lane comes from one ballot + scalar find-first; its winning
 //     point is found by walking the winner lane's tree with v_readlane and
 //     scalar branches (left child first = lowest position), and the leaf reached
 //     reads that point's coordinates from fixed registers - log2(P) steps, no
 //     per-point compares or select chains in the loop;
-//   * a wave publishes one 32-byte slot (value, point, xyz); after the single
-//     barrier every wave loads all slots at once and picks the winner with
-//     v_readlane, no second LDS round trip.
-__device__ __forceinline__ int wave_max_i32(int v)
-{
-    // VALU write -> DPP read of the same register needs two wait states (s_nop 1).
-    asm volatile("s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
-                 "s_nop 1\n\t"
-                 "v_max_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
-                 "s_nop 1"
-                 : "+v"(v));
-    return __builtin_amdgcn_readlane(v, 63);
-}
-
+//   * a wave publishes one 32-byte slot (value, runner-up, point, xyz); after the single
+//     barrier every wave loads the slots and decides by itself how many of the
+//     candidates are winners (see fps_multistep_kernel_f32).
 struct __align__(16) FpsSlot {
     int val;  // bit pattern of the wave's maximum
     int j;    // point index of the wave's candidate
     float x, y, z;
-    int pad[3];
+    int pad[3];  // pad[0]: the wave's second-largest minimum
 };
 
 struct FpsPick {
@@ -245,15 +225,44 @@ struct FpsPick {
     int j;
 };
 
-// Walks the tree of lane `wl` from NODE down to the first leaf equal to `wmax`.
-// t[1] is the root, t[2i] / t[2i+1] the children of t[i], t[P + p] the minimum of
-// point p. Every register index is a compile-time constant; the direction taken
-// at each node is wave-uniform, so the walk is scalar branches.
-template <int P, int NODE> struct FpsWalk {
+// Largest and second-largest of the 64 lanes' values (with multiplicity: two lanes
+// holding the maximum give second == first), both wave-uniform. The scan of
+// wave_max_i32 carrying a pair: every step merges two disjoint lane sets, for which
+// second = max(second_a, second_b, min(first_a, first_b)). The two chains fill each
+// other's DPP wait states. Lanes whose source lane does not exist skip a step's DPP
+// writes and re-apply a stale `t` that their `second` already contains.
+__device__ __forceinline__ void wave_top2_i32(int v, int &first, int &second)
+{
+    int m1 = v, m2 = 0, t = 0;  // values are >= 0
+#define TK3D_TOP2_STEP(CTRL, MASK)                                                         \
+    "s_nop 0\n\t"                                                                           \
+    "v_min_i32_dpp %2, %0, %0 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
+    "v_max_i32_dpp %1, %1, %1 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
+    "v_max_i32_dpp %0, %0, %0 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
+    "v_max_i32_dpp %1, %2, %1 quad_perm:[0,1,2,3] row_mask:" MASK " bank_mask:0xf\n\t"
+    asm volatile("s_nop 1\n\t"
+                 TK3D_TOP2_STEP("row_shr:1", "0xf")
+                 TK3D_TOP2_STEP("row_shr:2", "0xf")
+                 TK3D_TOP2_STEP("row_shr:4", "0xf")
+                 TK3D_TOP2_STEP("row_shr:8", "0xf")
+                 TK3D_TOP2_STEP("row_bcast:15", "0xa")
+                 TK3D_TOP2_STEP("row_bcast:31", "0xc")
+                 "s_nop 1"
+                 : "+v"(m1), "+v"(m2), "+v"(t));
+#undef TK3D_TOP2_STEP
+    first = __builtin_amdgcn_readlane(m1, 63);
+    second = __builtin_amdgcn_readlane(m2, 63);
+}
+
+// FpsWalk that also reports the largest value it passed by: the walk from the root to
+// the first leaf equal to `wmax` sees the sibling of every node on its path, and the
+// largest of those siblings is the lane's second-largest minimum (equal to `wmax` when
+// the lane holds the maximum twice).
+template <int P, int NODE> struct FpsWalk2 {
     static __device__ __forceinline__ void go(const int (&t)[2 * P], const float (&x)[P],
                                               const float (&y)[P], const float (&z)[P],
                                               const int (&jv)[P], int wl, int wmax,
-                                              FpsPick &out)
+                                              FpsPick &out, int &passed)
     {
         if constexpr (NODE >= P) {
             constexpr int p = NODE - P;
@@ -261,28 +270,48 @@ template <int P, int NODE> struct FpsWalk {
             out.y = read_lane(y[p], wl);
             out.z = read_lane(z[p], wl);
             out.j = read_lane(jv[p], wl);
-            // Keeps each leaf a block of its own (no flattening into selects).
             asm volatile("" ::"s"(out.j));
         } else {
             const int left = read_lane(t[2 * NODE], wl);
-            if (left == wmax)
-                FpsWalk<P, 2 * NODE>::go(t, x, y, z, jv, wl, wmax, out);
-            else
-                FpsWalk<P, 2 * NODE + 1>::go(t, x, y, z, jv, wl, wmax, out);
+            const int right = read_lane(t[2 * NODE + 1], wl);
+            if (left == wmax) {
+                passed = right > passed ? right : passed;
+                FpsWalk2<P, 2 * NODE>::go(t, x, y, z, jv, wl, wmax, out, passed);
+            } else {
+                passed = left > passed ? left : passed;
+                FpsWalk2<P, 2 * NODE + 1>::go(t, x, y, z, jv, wl, wmax, out, passed);
+            }
         }
     }
 };
 
-template <int P, int NT, bool SOA>
-__global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__restrict__ points,
-                                                              int64_t *__restrict__ index,
-                                                              FpsLayout L)
+// fp32 kernel that takes up to MAXM selection steps per cross-wave exchange.
+//
+// A step's fixed cost (wave reduction, slot exchange, barrier: about 1000 clocks) is
+// several times the cost of updating the minima for one more centre, so after the
+// exchange every wave checks, redundantly, whether the next winners are already known.
+// Let the waves' candidates be sorted by (value descending, wave ascending) - waves
+// hold ascending position ranges, so this is the reference's order - and let w1 be the
+// winner. The m-th candidate w_m (value V_m > 0) is the winner of the m-th following
+// step exactly when
+//   * no wave that already supplied a winner holds another point at or above V_m (each
+//     wave publishes its second-largest minimum for this; ties are refused), and
+//   * the canonical distance from w_m to every winner accepted so far is >= V_m, so the
+//     coming updates leave its minimum at V_m;
+// every other point is at or below V_m by the sort, minima only shrink, and the
+// accepted winners drop to zero. The chain stops at the first candidate that fails;
+// on uniform clouds about 2.7 steps are taken per exchange.
+template <int P, int NT, bool SOA, int MAXM>
+__global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__restrict__ points,
+                                                               int64_t *__restrict__ index,
+                                                               FpsLayout L)
 {
     static_assert((P & (P - 1)) == 0, "P must be a power of two");
     constexpr int NW = NT / TK_WAVE;
+    static_assert(NW <= 8, "the cross-wave step relates 8 x 8 candidates");
     constexpr int F32_INF = 0x7f800000;
     constexpr int F32_NEG1 = (int)0xbf800000;
-    __shared__ FpsSlot slots[2][NW];
+    __shared__ FpsSlot slots[2][8];
 
     const int tid = threadIdx.x;
     const int lane = tid & (TK_WAVE - 1);
@@ -308,17 +337,37 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
     t[0] = 0;
 
     int sel_j = 0;
-    float cx = fps_coord<SOA>(pts, L.n, 0, 0), cy = fps_coord<SOA>(pts, L.n, 0, 1),
-          cz = fps_coord<SOA>(pts, L.n, 0, 2);
+    float cx[MAXM], cy[MAXM], cz[MAXM];  // centres selected by the last exchange
+#pragma unroll
+    for (int m = 0; m < MAXM; ++m) {
+        cx[m] = fps_coord<SOA>(pts, L.n, 0, 0);
+        cy[m] = fps_coord<SOA>(pts, L.n, 0, 1);
+        cz[m] = fps_coord<SOA>(pts, L.n, 0, 2);
+    }
+    int nc = 1;
     if (tid == 0)
         out[0] = 0;
+    if (tid < 16 && (tid & 7) >= NW) {  // waves that do not exist never have a candidate
+        FpsSlot s;
+        s.val = F32_NEG1;
+        s.j = 0;
+        s.x = s.y = s.z = 0.0f;
+        s.pad[0] = s.pad[1] = s.pad[2] = 0;
+        slots[tid >> 3][tid & 7] = s;
+    }
 
-    for (int it = 1; it < L.k; ++it) {
+    int round = 0;
+    for (int it = 1; it < L.k; it += nc, ++round) {
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const float d = tk_dist2<float>(x[p], y[p], z[p], cx, cy, cz);
-            const int db = __builtin_bit_cast(int, d);
-            t[P + p] = t[P + p] < db ? t[P + p] : db;
+        for (int m = 0; m < MAXM; ++m) {
+            if (m < nc) {  // uniform
+#pragma unroll
+                for (int p = 0; p < P; ++p) {
+                    const float d = tk_dist2<float>(x[p], y[p], z[p], cx[m], cy[m], cz[m]);
+                    const int db = __builtin_bit_cast(int, d);
+                    t[P + p] = t[P + p] < db ? t[P + p] : db;
+                }
+            }
         }
 #pragma unroll
         for (int i = P - 1; i >= 1; --i)
@@ -326,11 +375,12 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
         // Only points strictly above zero are candidates (the reference starts its
         // scan from max_dist = 0 with strict '>').
         const int best = t[1] > 0 ? t[1] : 0;
-        const int wmax = wave_max_i32(best);
+        int wmax, second;
+        wave_top2_i32(best, wmax, second);  // second: over the other lanes
         const int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
         FpsPick pick;
-        FpsWalk<P, 1>::go(t, x, y, z, jv, wl, wmax, pick);
-        const int buf = it & 1;
+        FpsWalk2<P, 1>::go(t, x, y, z, jv, wl, wmax, pick, second);  // and inside lane wl
+        const int buf = round & 1;
         if (lane == 0) {
             FpsSlot s;
             s.val = wmax;
@@ -338,22 +388,50 @@ __global__ __launch_bounds__(NT) void fps_register_kernel_f32(const float *__res
             s.x = pick.x;
             s.y = pick.y;
             s.z = pick.z;
-            s.pad[0] = s.pad[1] = s.pad[2] = 0;
+            s.pad[0] = second;
+            s.pad[1] = s.pad[2] = 0;
             slots[buf][wave] = s;
         }
         __syncthreads();
-        const FpsSlot mine = slots[buf][lane < NW ? lane : 0];
-        const int cv = lane < NW ? mine.val : F32_NEG1;
-        const int gmax = wave_max_i32(cv);
-        if (gmax > 0) {  // wave-uniform
-            const int gl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(cv == gmax));
-            sel_j = read_lane(mine.j, gl);
-            cx = read_lane(mine.x, gl);
-            cy = read_lane(mine.y, gl);
-            cz = read_lane(mine.z, gl);
+        // Every wave now works out, redundantly and without a serial chain, how many of
+        // the candidates are certain winners of the coming steps. Lane (a, b) = (lane / 8,
+        // lane % 8) relates candidate a to candidate b.
+        const int ca = lane >> 3, cb = lane & 7;
+        const FpsSlot A = slots[buf][ca], Bs = slots[buf][cb];
+        const int va = A.val, vb = Bs.val;
+        // b comes before a in the reference's order (larger value, then lower position)
+        const bool before = vb > va || (vb == va && cb < ca);
+        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bs.x, Bs.y, Bs.z);
+        // a survives b's selection: b's update leaves a's minimum alone, and b's wave
+        // holds nothing else at or above it
+        const bool survives = __builtin_bit_cast(int, dab) >= va && Bs.pad[0] < va;
+        const unsigned long long m_before = __builtin_amdgcn_ballot_w64(before);
+        const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(!before || survives);
+        const int rank = __builtin_popcount((unsigned)(m_before >> (8 * ca)) & 0xffu);
+        const bool all_fine = ((unsigned)(m_fine >> (8 * ca)) & 0xffu) == 0xffu && va > 0;
+        nc = 0;
+#pragma unroll
+        for (int m = 0; m < MAXM; ++m) {
+            // the candidate of rank m, if it and every candidate before it passed
+            const unsigned long long hit = __builtin_amdgcn_ballot_w64(rank == m && all_fine);
+            if (nc != m || hit == 0ull || it + m >= L.k)  // uniform
+                break;
+            const int src = __builtin_ctzll(hit);
+            cx[m] = read_lane(A.x, src);
+            cy[m] = read_lane(A.y, src);
+            cz[m] = read_lane(A.z, src);
+            sel_j = read_lane(A.j, src);
+            if (tid == 0)
+                out[it + m] = (int64_t)sel_j;
+            nc = m + 1;
         }
-        if (tid == 0)
-            out[it] = (int64_t)sel_j;
+        if (nc == 0) {
+            // no point lies away from the chosen set; the previous choice is emitted again,
+            // as the reference does
+            if (tid == 0)
+                out[it] = (int64_t)sel_j;
+            nc = 1;
+        }
     }
 }
 
@@ -471,12 +549,13 @@ template <int P, int NT>
 void fps_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
                     const FpsLayout &L, hipStream_t s)
 {
+    constexpr int MAXM = 6;  // 4 -> 6 gains 1-4 %, 8 nothing
     if (soa)
-        hipLaunchKernelGGL((fps_register_kernel_f32<P, NT, true>), dim3((unsigned)B), dim3(NT),
-                           0, s, points, index, L);
+        hipLaunchKernelGGL((fps_multistep_kernel_f32<P, NT, true, MAXM>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L);
     else
-        hipLaunchKernelGGL((fps_register_kernel_f32<P, NT, false>), dim3((unsigned)B), dim3(NT),
-                           0, s, points, index, L);
+        hipLaunchKernelGGL((fps_multistep_kernel_f32<P, NT, false, MAXM>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L);
 }
 
 // fp32: (points per lane, lanes) by cloud size, from timing every shape on an
