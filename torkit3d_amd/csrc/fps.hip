@@ -409,25 +409,42 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
         const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(!before || survives);
         const int rank = __builtin_popcount((unsigned)(m_before >> (8 * ca)) & 0xffu);
         const bool all_fine = ((unsigned)(m_fine >> (8 * ca)) & 0xffu) == 0xffu && va > 0;
-        nc = 0;
+        const unsigned long long fine = __builtin_amdgcn_ballot_w64(all_fine);
+        // How many leading ranks passed (scalar work), then the winners' data: a
+        // v_readlane costs tens of clocks, so only accepted ranks are fetched.
+        const int left = L.k - it;  // steps still wanted
+        unsigned long long row[MAXM];
+        int good = 0;               // ranks 0..good-1 passed
+        bool chain = true;
 #pragma unroll
         for (int m = 0; m < MAXM; ++m) {
-            // the candidate of rank m, if it and every candidate before it passed
-            const unsigned long long hit = __builtin_amdgcn_ballot_w64(rank == m && all_fine);
-            if (nc != m || hit == 0ull || it + m >= L.k)  // uniform
-                break;
-            const int src = __builtin_ctzll(hit);
-            cx[m] = read_lane(A.x, src);
-            cy[m] = read_lane(A.y, src);
-            cz[m] = read_lane(A.z, src);
-            sel_j = read_lane(A.j, src);
-            if (tid == 0)
-                out[it + m] = (int64_t)sel_j;
-            nc = m + 1;
+            // the ranks are a permutation of the 8 slots, so every rank has its row
+            row[m] = __builtin_amdgcn_ballot_w64(rank == m);
+            chain = chain && (row[m] & fine) != 0ull && m < left;  // uniform
+            good += chain ? 1 : 0;
         }
-        if (nc == 0) {
-            // no point lies away from the chosen set; the previous choice is emitted again,
-            // as the reference does
+        if (good > 0) {  // uniform
+            int jsel = 0;  // lane m of the first wave: the point of rank m
+#pragma unroll
+            for (int m = 0; m < MAXM; ++m) {
+                if (m < good) {  // uniform
+                    // every lane reads the winner's slot (one broadcast LDS read; fetching
+                    // the four values from a lane's registers costs far more)
+                    const FpsSlot w = slots[buf][__builtin_ctzll(row[m]) >> 3];
+                    cx[m] = w.x;
+                    cy[m] = w.y;
+                    cz[m] = w.z;
+                    sel_j = w.j;
+                    jsel = lane == m ? sel_j : jsel;
+                }
+            }
+            if (tid < good)
+                out[it + tid] = (int64_t)jsel;
+            nc = good;
+        } else {
+            // No point lies away from the chosen set: the previous choice is emitted again,
+            // as the reference does. Every minimum is zero already, so whatever centre the
+            // next update applies changes nothing.
             if (tid == 0)
                 out[it] = (int64_t)sel_j;
             nc = 1;
