@@ -61,7 +61,8 @@ def test_interpolation_config_fp32(cuda, k):
                                         (1, 50, 300, 100), (2, 33, 40, 40), (2, 10, 5, 5),
                                         (1, 1000, 1025, 33), (2, 300, 1000, 65),
                                         (2, 200, 700, 128), (1, 100, 400, 129),
-                                        (4, 1000, 4096, 32)])
+                                        (4, 1000, 4096, 32), (1, 70, 70000, 20),
+                                        (1, 40, 66000, 7), (40, 4096, 300, 6)])
 def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
     g = gen(k)
     q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)

@@ -13,6 +13,8 @@
 // k above the largest register variant falls back to a kernel that keeps the
 // structure in the output arrays in global memory, as the reference's generic
 // variant does (knn_distance_kernel.cu:102-177).
+#include <type_traits>
+
 #include "tk3d_common.h"
 
 namespace {
@@ -386,47 +388,66 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     }
 }
 
-// fp32 variant for larger k: the slots live in LDS as a per-lane tournament tree.
+// fp32 variant with the slots in LDS as a per-lane tournament tree.
 //
 // With the slots in registers every insertion pays O(k) selects and compares, because
 // registers cannot be indexed per lane. LDS can: a lane keeps, in columns of its own
 // (row r of an array at [r * 64 + lane], conflict-free whatever r each lane uses),
 //   leaf[s]  distance in slot s           kidx[s]  key index in slot s
 //   ival[n]  largest distance below node n of a binary tree over the slots (heap
-//            numbering, node 1 the root, the leaves of slot s at KMAX + s)
+//            numbering, node 1 the root, the leaf of slot s at KMAX + s)
 //   iarg[n]  the first slot that holds ival[n]
-// An insertion overwrites the leaf of the current maximum and replays the log2(KMAX)
-// matches on the way to the root. The other side of each of those matches is known up
-// front, so all of them are fetched at once and the path costs one LDS round trip plus
-// three vector instructions per level. A right child wins a match only when strictly
-// greater, so a node reports the first slot holding its maximum - MinK's rescan order
-// (mink.cuh:74-87); MinK starts that rescan from the inserted key, hence the maximum
-// stays in the inserted slot when the root is not strictly above it.
+// ival / iarg exist for nodes 1 .. KMAX/2-1 only: a parent of two leaves is worked out
+// from its leaves when needed, which saves a quarter of the LDS (the LDS footprint
+// decides how many waves a CU holds). An insertion overwrites the leaf of the current
+// maximum and replays the log2(KMAX) matches on the way to the root. The other side of
+// each of those matches is known up front, so all of them are fetched at once and the
+// path costs one LDS round trip plus three vector instructions per level. A right child
+// wins a match only when strictly greater, so a node reports the first slot holding its
+// maximum - MinK's rescan order (mink.cuh:74-87); MinK starts that rescan from the
+// inserted key, hence the maximum stays in the inserted slot when the root is not
+// strictly above it.
 //
 // The sweep takes its keys through scalar loads (the address is the same for every
 // lane) and the rounds fetch their candidates straight from global memory, one round
-// ahead; a block is one wave and never synchronises.
+// ahead; a block is one wave and never synchronises. IDX16 stores key indices in 16
+// bits (clouds up to 65536 keys).
 //
 // NaN distances can only enter during the fill (a later key must compare below the
 // maximum). MinK never selects such a slot as maximum unless it is slot 0, in which
 // case it never inserts again. Here a NaN in slot 0 freezes the lane; a NaN elsewhere
 // plays the tournament as -inf and is recomputed when the results are written.
-template <int KMAX>
+template <int KMAX, bool IDX16> struct KnnTreeLayout {
+    static constexpr int NT = 64;
+    using Idx = typename std::conditional<IDX16, unsigned short, int>::type;
+    static constexpr int LEAF_BYTES = 4 * KMAX * NT;
+    static constexpr int KIDX_BYTES = (int)sizeof(Idx) * KMAX * NT;
+    static constexpr int IVAL_BYTES = 4 * (KMAX / 2) * NT;
+    static constexpr int IARG_BYTES = (KMAX / 2) * NT;
+    static constexpr int BYTES = LEAF_BYTES + KIDX_BYTES + IVAL_BYTES + IARG_BYTES;
+};
+
+template <int KMAX, bool IDX16>
 __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
     int n2, int k)
 {
+    using Lay = KnnTreeLayout<KMAX, IDX16>;
+    using Idx = typename Lay::Idx;
     constexpr int CHUNK = 32;
     constexpr int NT = 64;
+    constexpr int HALF = KMAX / 2;  // nodes HALF .. KMAX-1 are the parents of the leaves
     constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : KMAX == 64 ? 6 : 7;
     static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 128");
     extern __shared__ __align__(16) unsigned char knn_tree_lds[];
     const int lane = threadIdx.x;
     float *const leaf = reinterpret_cast<float *>(knn_tree_lds) + lane;
-    int *const kidx = reinterpret_cast<int *>(knn_tree_lds) + KMAX * NT + lane;
-    float *const ival = reinterpret_cast<float *>(knn_tree_lds) + 2 * KMAX * NT + lane;
-    unsigned char *const iarg = knn_tree_lds + 12 * KMAX * NT + lane;
+    Idx *const kidx = reinterpret_cast<Idx *>(knn_tree_lds + Lay::LEAF_BYTES) + lane;
+    float *const ival =
+        reinterpret_cast<float *>(knn_tree_lds + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
+    unsigned char *const iarg =
+        knn_tree_lds + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
 
     const int b = blockIdx.x / blocks_per_batch;
     const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
@@ -440,6 +461,15 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         qz = q[2];
     }
 
+    // Value and first slot of a node whose children are leaves.
+    auto leaf_parent = [&](int n, float &v, int &a) {
+        const int s = 2 * n - KMAX;
+        const float lv = leaf[s * NT], rv = leaf[(s + 1) * NT];
+        const bool right = rv > lv;
+        v = right ? rv : lv;
+        a = right ? s + 1 : s;
+    };
+
     // Fill phase: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots hold -inf.
     bool frozen = false;
     for (int s = 0; s < KMAX; ++s) {
@@ -452,22 +482,19 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
             }
         }
         leaf[s * NT] = d;
-        kidx[s * NT] = s;
+        kidx[s * NT] = (Idx)s;
     }
-    for (int n = KMAX - 1; n >= 1; --n) {
-        const int l = 2 * n, r = 2 * n + 1;
+    for (int n = HALF - 1; n >= 1; --n) {
         float lv, rv;
         int la, ra;
-        if (l >= KMAX) {
-            lv = leaf[(l - KMAX) * NT];
-            rv = leaf[(r - KMAX) * NT];
-            la = l - KMAX;
-            ra = r - KMAX;
+        if (2 * n >= HALF) {
+            leaf_parent(2 * n, lv, la);
+            leaf_parent(2 * n + 1, rv, ra);
         } else {
-            lv = ival[l * NT];
-            rv = ival[r * NT];
-            la = iarg[l * NT];
-            ra = iarg[r * NT];
+            lv = ival[2 * n * NT];
+            rv = ival[(2 * n + 1) * NT];
+            la = iarg[2 * n * NT];
+            ra = iarg[(2 * n + 1) * NT];
         }
         const bool right = rv > lv;
         ival[n * NT] = right ? rv : lv;
@@ -476,16 +503,9 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     float max_key = frozen ? -__builtin_huge_valf() : ival[NT];
     int max_idx = iarg[NT];
 
-#ifdef TK3D_KNN_STATS
-    const unsigned long long st_t0 = KNN_CLOCK();
-    unsigned long long st_sweep = 0, st_rounds = 0;
-#endif
     for (int first = 0; first < n2; first += CHUNK) {  // `first` = key index of bit 31
         // ---- sweep: bit (31 - i) of `mask` <=> key first+i is below the maximum ----
         const int maxbits = __builtin_bit_cast(int, max_key);
-#ifdef TK3D_KNN_STATS
-        const unsigned long long st_a = KNN_CLOCK();
-#endif
         unsigned mask = 0u;
         if (first + CHUNK <= n2) {
             const float *__restrict__ g = K + (int64_t)first * 3;
@@ -513,9 +533,6 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
         valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
         mask &= valid;
-#ifdef TK3D_KNN_STATS
-        st_sweep += KNN_CLOCK() - st_a;
-#endif
 
         // ---- insertion rounds, the next candidate's key in flight during the current ----
         const float *__restrict__ ck = K + (int64_t)first * 3;
@@ -523,9 +540,6 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         int i = has ? __builtin_clz(mask) : 0;
         float ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-#ifdef TK3D_KNN_STATS
-            ++st_rounds;
-#endif
             mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
             const bool has_next = mask != 0u;
             const int i_next = has_next ? __builtin_clz(mask) : 0;
@@ -535,13 +549,15 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
             if (has && d < max_key) {
                 const int p = max_idx;
                 leaf[p * NT] = d;
-                kidx[p * NT] = first + i;
+                kidx[p * NT] = (Idx)(first + i);
+                // the other side of every match on the path, fetched together
                 float sv[LEVELS];
                 int sa[LEVELS];
                 sv[0] = leaf[(p ^ 1) * NT];
                 sa[0] = p ^ 1;
+                leaf_parent(((KMAX + p) >> 1) ^ 1, sv[1], sa[1]);
 #pragma unroll
-                for (int l = 1; l < LEVELS; ++l) {
+                for (int l = 2; l < LEVELS; ++l) {
                     const int sib = ((KMAX + p) >> l) ^ 1;
                     sv[l] = ival[sib * NT];
                     sa[l] = iarg[sib * NT];
@@ -555,7 +571,8 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
                     const bool take = (node & 1) ? !(v > sv[l]) : (sv[l] > v);
                     v = take ? sv[l] : v;
                     a = take ? sa[l] : a;
-                    if (l + 1 < LEVELS) {  // the root lives in max_key / max_idx
+                    // parents of leaves are not stored; the root lives in max_key / max_idx
+                    if (l >= 1 && l + 1 < LEVELS) {
                         ival[(node >> 1) * NT] = v;
                         iarg[(node >> 1) * NT] = (unsigned char)a;
                     }
@@ -571,15 +588,6 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         }
     }
 
-#ifdef TK3D_KNN_STATS
-    if (lane == 0) {
-        const unsigned wv = blockIdx.x & 0x3fff;
-        knn_stats[wv * 4 + 0] = st_t0;
-        knn_stats[wv * 4 + 1] = KNN_CLOCK();
-        knn_stats[wv * 4 + 2] = st_sweep;
-        knn_stats[wv * 4 + 3] = st_rounds << 32;
-    }
-#endif
     if (active) {
         float *od = distance + ((int64_t)b * n1 + qi) * k;
         int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
@@ -593,22 +601,32 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     }
 }
 
-template <int KMAX>
-int knn_tree_launch(const float *query, const float *key, float *distance, int64_t *index,
-                    int64_t B, int n1, int n2, int k, hipStream_t s)
+template <int KMAX, bool IDX16>
+int knn_tree_launch_as(const float *query, const float *key, float *distance, int64_t *index,
+                       int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    constexpr int LDS_BYTES = 13 * KMAX * 64;
+    constexpr int LDS_BYTES = KnnTreeLayout<KMAX, IDX16>::BYTES;
     if (LDS_BYTES > 48 * 1024) {
-        const int allowed = tk_allow_dynamic_lds<knn_tree_kernel_f32<KMAX>>(LDS_BYTES);
+        const int allowed =
+            tk_allow_dynamic_lds<knn_tree_kernel_f32<KMAX, IDX16>>(LDS_BYTES);
         if (allowed != TK3D_OK)
             return allowed;
     }
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     if (B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_tree_kernel_f32<KMAX>), dim3((unsigned)(B * bpb)), dim3(64),
+    hipLaunchKernelGGL((knn_tree_kernel_f32<KMAX, IDX16>), dim3((unsigned)(B * bpb)), dim3(64),
                        LDS_BYTES, s, query, key, distance, index, (int)bpb, n1, n2, k);
     return tk_launch_status();
+}
+
+template <int KMAX>
+int knn_tree_launch(const float *query, const float *key, float *distance, int64_t *index,
+                    int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    if (n2 <= 65536)
+        return knn_tree_launch_as<KMAX, true>(query, key, distance, index, B, n1, n2, k, s);
+    return knn_tree_launch_as<KMAX, false>(query, key, distance, index, B, n1, n2, k, s);
 }
 
 // Any k: the structure lives in the output rows in global memory.
@@ -722,24 +740,34 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         return TK3D_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
-    if (k <= 4)
+    if (k <= 4) {
         knn_launch<T, 4>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else if (k <= 8)
-        knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else if (k <= 16)
-        knn_launch<T, 16>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
-    else if constexpr (sizeof(T) == 4) {
-        // fp32: slots in LDS as a tournament tree up to k = 128
-        if (k <= 32)
+    } else if constexpr (sizeof(T) == 4) {
+        // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
+        // 0.30 ms against 0.41 ms with the slots in registers). Small launches with k <= 8
+        // are a little faster in registers.
+        if (k <= 8 && B * N1 < 131072)
+            knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+        else if (k <= 8)
+            return knn_tree_launch<8>(query, key, distance, index, B, n1, n2, kk, s);
+        else if (k <= 16)
+            return knn_tree_launch<16>(query, key, distance, index, B, n1, n2, kk, s);
+        else if (k <= 32)
             return knn_tree_launch<32>(query, key, distance, index, B, n1, n2, kk, s);
-        if (k <= 64)
+        else if (k <= 64)
             return knn_tree_launch<64>(query, key, distance, index, B, n1, n2, kk, s);
-        if (k <= 128)
+        else if (k <= 128)
             return knn_tree_launch<128>(query, key, distance, index, B, n1, n2, kk, s);
-        hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)), dim3(KNN_BLOCK),
-                           0, s, query, key, distance, index, (int)bpb, n1, n2, kk);
+        else
+            hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)),
+                               dim3(KNN_BLOCK), 0, s, query, key, distance, index, (int)bpb,
+                               n1, n2, kk);
     } else {
-        if (k <= 32)
+        if (k <= 8)
+            knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+        else if (k <= 16)
+            knn_launch<T, 16>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+        else if (k <= 32)
             knn_launch<T, 32>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
         else if (k <= 64)
             knn_launch<T, 64>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
