@@ -23,7 +23,11 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
                                                          int n2, T r2, int k)
 {
     const int lane = threadIdx.x & (TK_WAVE - 1);
-    const int64_t gw = (int64_t)blockIdx.x * (256 / TK_WAVE) + threadIdx.x / TK_WAVE;
+    // readfirstlane tells the compiler that the wave index is uniform: the queries'
+    // coordinates, hit counters and output rows then live in scalar registers and the
+    // "query is full" tests are scalar branches.
+    const int wave_in_block = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / TK_WAVE));
+    const int64_t gw = (int64_t)blockIdx.x * (256 / TK_WAVE) + wave_in_block;
     if (gw >= total_waves)
         return;
     const int b = (int)(gw / waves_per_batch);
@@ -50,13 +54,26 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
 
     for (int j0 = 0; j0 < n2; j0 += TK_WAVE * UNROLL) {
         T kx[UNROLL], ky[UNROLL], kz[UNROLL];
+        if (j0 + TK_WAVE * UNROLL <= n2) {
+            // full chunk: unconditional loads at constant offsets from one lane address
+            const T *__restrict__ kl = K + (int64_t)(j0 + lane) * kps;
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int j = j0 + u * TK_WAVE + lane;
-            const bool ok = j < n2;
-            kx[u] = ok ? K[(int64_t)j * kps] : (T)0;
-            ky[u] = ok ? K[(int64_t)j * kps + kcs] : (T)0;
-            kz[u] = ok ? K[(int64_t)j * kps + 2 * kcs] : (T)0;
+            for (int u = 0; u < UNROLL; ++u) {
+                kx[u] = kl[u * TK_WAVE * kps];
+                ky[u] = kl[u * TK_WAVE * kps + kcs];
+                kz[u] = kl[u * TK_WAVE * kps + 2 * kcs];
+            }
+        } else {
+            // last chunk: keys that do not exist become NaN, which is never within reach
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int j = j0 + u * TK_WAVE + lane;
+                const int jc = j < n2 ? j : n2 - 1;
+                const T nan = (T)__builtin_nanf("");
+                kx[u] = j < n2 ? K[(int64_t)jc * kps] : nan;
+                ky[u] = K[(int64_t)jc * kps + kcs];
+                kz[u] = K[(int64_t)jc * kps + 2 * kcs];
+            }
         }
         bool all_done = true;
 #pragma unroll
@@ -67,7 +84,7 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
                     continue;
                 const int j = j0 + u * TK_WAVE + lane;
                 const T d = tk_dist2<T>(kx[u], ky[u], kz[u], qx[q], qy[q], qz[q]);
-                const bool hit = (j < n2) && (d < r2);
+                const bool hit = d < r2;  // false for the NaN of a key that does not exist
                 const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit);
                 if (mask == 0)
                     continue;
@@ -95,6 +112,27 @@ __global__ __launch_bounds__(256) void ball_query_kernel(const T *__restrict__ q
     }
 }
 
+template <typename T, int QW>
+int ball_query_launch(const T *query, const T *key, bool channels_first, int64_t B, int64_t N1,
+                      int64_t N2, T r2, int64_t k, int64_t *index, void *stream)
+{
+    constexpr int UNROLL = 8;  // 512 keys per trip
+    const int64_t wpb = (N1 + QW - 1) / QW;
+    const int64_t waves = B * wpb;
+    const int64_t blocks = (waves + 3) / 4;
+    if (blocks > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    if (channels_first)
+        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, true>), dim3((unsigned)blocks),
+                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
+                           (int)N1, (int)N2, r2, (int)k);
+    else
+        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, false>), dim3((unsigned)blocks),
+                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
+                           (int)N1, (int)N2, r2, (int)k);
+    return tk_launch_status();
+}
+
 template <typename T>
 int ball_query(const T *query, const T *key, bool channels_first, int64_t B, int64_t N1,
                int64_t N2, float radius, int64_t k, int64_t *index, void *stream)
@@ -110,25 +148,20 @@ int ball_query(const T *query, const T *key, bool channels_first, int64_t B, int
         return TK3D_OK;
     if (!query || !index || (N2 > 0 && !key))
         return TK3D_ERR_NULL_POINTER;
-    constexpr int QW = 4, UNROLL = 4;
-    const int64_t wpb = (N1 + QW - 1) / QW;
-    const int64_t waves = B * wpb;
-    const int64_t blocks = (waves + 3) / 4;
-    if (blocks > TK_MAX_I32)
-        return TK3D_ERR_UNSUPPORTED;
     // r2 = r*r in the data type, r being the float the caller passed
     // (ball_query.h:9, ball_query_kernel.cu:19,26).
     const T r = (T)radius;
     const T r2 = r * r;
-    if (channels_first)
-        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, true>), dim3((unsigned)blocks),
-                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
-                           (int)N1, (int)N2, r2, (int)k);
-    else
-        hipLaunchKernelGGL((ball_query_kernel<T, QW, UNROLL, false>), dim3((unsigned)blocks),
-                           dim3(256), 0, (hipStream_t)stream, query, key, index, waves, (int)wpb,
-                           (int)N1, (int)N2, r2, (int)k);
-    return tk_launch_status();
+    // Queries per wave: 4 share every key load when there are enough queries to fill the
+    // GPU with waves anyway; fewer per wave otherwise.
+    const int64_t total = B * N1;
+    if (total >= 16384)
+        return ball_query_launch<T, 4>(query, key, channels_first, B, N1, N2, r2, k, index,
+                                       stream);
+    if (total >= 4096)
+        return ball_query_launch<T, 2>(query, key, channels_first, B, N1, N2, r2, k, index,
+                                       stream);
+    return ball_query_launch<T, 1>(query, key, channels_first, B, N1, N2, r2, k, index, stream);
 }
 
 }  // namespace
