@@ -292,7 +292,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     // More queries than this with three or more candidate tiles: the cloud is full of
     // ties (quantised coordinates) and the exact sweep is the cheaper way out.
     constexpr int MAX_SCANS = 96;
-    __shared__ __align__(16) float skey[2 * STAGE * 4];
+    __shared__ __align__(16) float skey[2 * STAGE * 4 + 8];  // + 2 keys for the read-ahead
     __shared__ float sred[NW][8];
     __shared__ int sidx[NW];
     __shared__ int s_list[MAX_SCANS];
@@ -442,9 +442,14 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
             for (int i = 0; i < QPL; ++i)
                 tmin[i] = INF;
             const float4 *tk = sbuf + t * TILE;
+            // The pair after the current one is read from LDS before the current pair's
+            // 28 vector instructions, so its latency hides behind them (the last read of
+            // a tile runs into the next tile or the pad behind the buffers). Reading two
+            // pairs ahead was slower (more registers).
+            float4 ka = tk[0], kb = tk[1];
 #pragma unroll
             for (int j = 0; j < TILE; j += 2) {
-                const float4 ka = tk[j], kb = tk[j + 1];
+                const float4 na = tk[j + 2], nb = tk[j + 3];
 #pragma unroll
                 for (int i = 0; i < QPL; ++i) {
                     const float sa = __builtin_fmaf(
@@ -453,6 +458,8 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
                         kb.x, ax[i], __builtin_fmaf(kb.y, ay[i], __builtin_fmaf(kb.z, az[i], kb.w)));
                     tmin[i] = __builtin_fminf(__builtin_fminf(tmin[i], sa), sb);
                 }
+                ka = na;
+                kb = nb;
             }
             // Three smallest tile minima (ties keep the earlier tile in front).
             const int tile_id = stage0 / TILE + t;
