@@ -122,16 +122,21 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
             for (int i = 0; i < QPL; ++i)
                 tmin[i] = tk_inf<T>();
             const T *tk = skey + t * TILE * 4;
+            // the next pair of keys is read while the current pair is evaluated (the last
+            // read of a stage runs into the two pad keys behind the buffer)
+            T ax = tk[0], ay = tk[1], az = tk[2], bx = tk[4], by = tk[5], bz = tk[6];
 #pragma unroll
             for (int j = 0; j < TILE; j += 2) {
-                const T ax = tk[j * 4 + 0], ay = tk[j * 4 + 1], az = tk[j * 4 + 2];
-                const T bx = tk[j * 4 + 4], by = tk[j * 4 + 5], bz = tk[j * 4 + 6];
+                const T nax = tk[j * 4 + 8], nay = tk[j * 4 + 9], naz = tk[j * 4 + 10];
+                const T nbx = tk[j * 4 + 12], nby = tk[j * 4 + 13], nbz = tk[j * 4 + 14];
 #pragma unroll
                 for (int i = 0; i < QPL; ++i) {
                     const T da = tk_dist2<T>(ax, ay, az, qx[i], qy[i], qz[i]);
                     const T db = tk_dist2<T>(bx, by, bz, qx[i], qy[i], qz[i]);
                     tmin[i] = tk_min<T>(tk_min<T>(tmin[i], da), db);
                 }
+                ax = nax, ay = nay, az = naz;
+                bx = nbx, by = nby, bz = nbz;
             }
             const int tile_id = stage0 / TILE + t;
 #pragma unroll
@@ -170,7 +175,7 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
 template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
 __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T> args)
 {
-    __shared__ T skey[STAGE * 4];
+    __shared__ T skey[STAGE * 4 + 8];  // + 2 keys for the read-ahead
     int b, qblock;
     const ChamferDir<T> &d = chamfer_decode_block<T>(args, b, qblock);
     chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
