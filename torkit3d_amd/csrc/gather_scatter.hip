@@ -105,14 +105,6 @@ __global__ __launch_bounds__(GS_BLOCK) void gather_kernel(
     }
 }
 
-#ifdef TK3D_GATHER_STATS
-__device__ unsigned long long gather_stats[1 << 16];
-#define GA_STAMP(i)                                                                      \
-    if (threadIdx.x == 0)                                                                \
-    gather_stats[((blockIdx.z * gridDim.y + blockIdx.y) & 0x1fff) * 8 + (i)] = __builtin_readcyclecounter()
-#else
-#define GA_STAMP(i)
-#endif
 
 // Same gather with the source rows staged in LDS. Row gathers through the vector
 // cache cost one cache line per lane (64 lanes -> 64 lines per load instruction),
@@ -162,8 +154,6 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
     };
     const int64_t pfirst = ps + (int64_t)wave * (64 * V) + lane;
     fetch(pfirst);
-
-    GA_STAMP(0);
     {
         // the staged rows are contiguous in global memory: 16-byte copies when aligned
         constexpr int E = 16 / (int)sizeof(T);
@@ -178,9 +168,7 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
         for (int i = nwide * E + threadIdx.x; i < total; i += NT)
             rows[i] = src_rows[i];
     }
-    GA_STAMP(1);
     __syncthreads();
-    GA_STAMP(2);
 
     for (int64_t p0 = pfirst; p0 < pe; p0 += (int64_t)NT * V) {
         int src[V][KK];
@@ -220,7 +208,6 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
             }
         }
     }
-    GA_STAMP(3);
 }
 
 // ---- scatter ---------------------------------------------------------------------
@@ -357,14 +344,6 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v)
     return v;
 }
 
-#ifdef TK3D_SCATTER_STATS
-__device__ unsigned long long scatter_stats[1 << 16];
-#define SC_STAMP(i)                                                                      \
-    if (threadIdx.x == 0)                                                                \
-    scatter_stats[((blockIdx.z * gridDim.y + blockIdx.y) & 0x1fff) * 8 + (i)] = __builtin_readcyclecounter()
-#else
-#define SC_STAMP(i)
-#endif
 
 template <int KK, bool HAS_W, int V, int NT, int CGMAX>
 __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
@@ -386,8 +365,6 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     const int64_t ps = (int64_t)blockIdx.x * seg_len;
     const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
-
-    SC_STAMP(0);
     for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
         __syncthreads();
         for (int i = threadIdx.x; i < nc * n1; i += NT)
@@ -400,7 +377,6 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             s_maxw = HAS_W ? 0u : 0x3f800000u;
         }
         __syncthreads();
-        SC_STAMP(1);
 
         // ---- magnitudes: every 8th group first, everything on the second attempt ----
         if (HAS_W) {
@@ -466,7 +442,6 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             }
         }
         __syncthreads();
-        SC_STAMP(2);
 
         // ---- bounds and scales: lane c < CGMAX works out row c ----
         if (threadIdx.x < CGMAX) {
@@ -486,8 +461,6 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         __syncthreads();
         if (!s_finite)
             break;
-
-        SC_STAMP(3);
         struct RowScale {
             double scale;
             float bound;
@@ -511,9 +484,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             });
         if (exceeded)
             s_exceeded = 1;
-        SC_STAMP(4);
         __syncthreads();
-        SC_STAMP(5);
         if (!s_exceeded) {
             float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
             for (int i = threadIdx.x; i < nc * n1; i += NT) {
@@ -526,7 +497,6 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                     dstrows[i] = v;
                 }
             }
-            SC_STAMP(6);
             return;
         }
     }
@@ -624,10 +594,6 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         int cg = 8;
         while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
             cg /= 2;
-#ifdef TK3D_GATHER_STATS
-        if (getenv("TK3D_CG"))
-            cg = atoi(getenv("TK3D_CG"));
-#endif
         const int64_t gy = (C + cg - 1) / cg;
         // Split the points until the chip is full; every chunk re-stages its rows, so
         // keep a chunk well above the staged size.
@@ -636,10 +602,6 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         while (B * gy * chunks < 1024 && NP / (chunks * 2) >= min_chunk &&
                (NP / (chunks * 2)) * KK >= (cg * N1) / 2)
             chunks *= 2;
-#ifdef TK3D_GATHER_STATS
-        if (getenv("TK3D_CHUNKS"))
-            chunks = atoi(getenv("TK3D_CHUNKS"));
-#endif
         int64_t chunk_len = (NP + chunks - 1) / chunks;
         chunk_len = (chunk_len + 15) / 16 * 16;  // keeps 16-byte alignment of chunk starts
         chunks = (NP + chunk_len - 1) / chunk_len;

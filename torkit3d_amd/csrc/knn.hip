@@ -159,10 +159,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
 // largest number of candidates any lane has, instead of the number of distinct
 // candidate keys across all lanes. The sequence of insertions seen by one lane is
 // exactly MinK's, so the slot order is unchanged.
-#ifdef TK3D_KNN_STATS
-__device__ unsigned long long knn_stats[1 << 16];  // per wave: t0, t1, sweep cycles, rounds
-#define KNN_CLOCK() __builtin_readcyclecounter()
-#endif
 
 template <int KMAX, bool SOA, bool WEIGHTS>
 __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
@@ -214,10 +210,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
     // the fill (later keys must compare below the maximum); a wave that has one rescans
     // with float compares instead.
     const bool float_rescan = __builtin_amdgcn_ballot_w64(fill_nan) != 0;
-#ifdef TK3D_KNN_STATS
-    const unsigned long long st_t0 = KNN_CLOCK();
-    unsigned long long st_sweep = 0, st_rounds = 0;
-#endif
 
     for (int stage0 = 0; stage0 < n2; stage0 += KNN_STAGE) {
         __syncthreads();
@@ -239,9 +231,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             const int maxbits = __builtin_bit_cast(int, max_key);
             const float4 *ck = reinterpret_cast<const float4 *>(skey) + c0;
             const int first = stage0 + c0;  // global index of bit 31
-#ifdef TK3D_KNN_STATS
-            const unsigned long long st_a = KNN_CLOCK();
-#endif
             unsigned mask = 0u;
             if (c0 + CHUNK <= cnt) {
                 // A full chunk comes straight from global memory: the addresses are the
@@ -273,9 +262,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
             valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
             mask &= valid;
-#ifdef TK3D_KNN_STATS
-            st_sweep += KNN_CLOCK() - st_a;
-#endif
 
             // ---- insertion rounds; the next candidate's key is fetched from LDS while the
             // current one is inserted ----
@@ -283,9 +269,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
             int i = has ? __builtin_clz(mask) : 0;
             float4 e = ck[i];
             while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-#ifdef TK3D_KNN_STATS
-                ++st_rounds;
-#endif
                 mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
                 const bool has_next = mask != 0u;
                 const int i_next = has_next ? __builtin_clz(mask) : 0;
@@ -360,17 +343,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
         }
     }
 
-#ifdef TK3D_KNN_STATS
-    if ((tid & 63) == 0) {
-        const unsigned wv = (blockIdx.x * (KNN_BLOCK / 64) + (tid >> 6)) & 0x3fff;
-        unsigned hw;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-        knn_stats[wv * 4 + 0] = st_t0;
-        knn_stats[wv * 4 + 1] = KNN_CLOCK();
-        knn_stats[wv * 4 + 2] = st_sweep;
-        knn_stats[wv * 4 + 3] = (st_rounds << 32) | hw;
-    }
-#endif
     if (active) {
         float *od = distance + ((int64_t)b * n1 + qi) * k;
         int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
