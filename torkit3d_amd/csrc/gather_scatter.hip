@@ -599,7 +599,7 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
         // keep a chunk well above the staged size.
         int64_t chunks = 1;
         const int64_t min_chunk = (int64_t)NT * V * 4;
-        while (B * gy * chunks < 1024 && NP / (chunks * 2) >= min_chunk &&
+        while (B * gy * chunks < 512 && NP / (chunks * 2) >= min_chunk &&
                (NP / (chunks * 2)) * KK >= (cg * N1) / 2)
             chunks *= 2;
         int64_t chunk_len = (NP + chunks - 1) / chunks;
