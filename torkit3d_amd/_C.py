@@ -70,7 +70,7 @@ def sample_farthest_points_cuda(points, num_samples):
     _check(points.size(1) >= num_samples,
            "Check failed: points.size(1) >= num_samples (%d vs. %d)" % (points.size(1), num_samples))
     b, n = points.size(0), points.size(1)
-    with torch.cuda.device(points.device):
+    with _lib.on_device_of(points):
         index = torch.empty((b, num_samples), dtype=torch.int64, device=points.device)
         ws_fn = _lib.lib().tk3d_sample_farthest_points_workspace_bytes
         ws_fn.restype = ctypes.c_size_t
@@ -96,7 +96,7 @@ def ball_query_cuda(query, key, radius, max_neighbors):
     max_neighbors = int(max_neighbors)
     _check(max_neighbors >= 0, "max_neighbors must be non-negative.")
     b, n1, n2 = query.size(0), query.size(1), key.size(1)
-    with torch.cuda.device(query.device):
+    with _lib.on_device_of(query):
         index = torch.empty((b, n1, max_neighbors), dtype=torch.int64, device=query.device)
         _lib.call("tk3d_ball_query", query, ptr(query), ptr(key), i64(b), i64(n1), i64(n2),
                   ctypes.c_float(float(radius)), i64(max_neighbors), ptr(index),
@@ -118,7 +118,7 @@ def group_points_forward_cuda(input, index):
     index = index.contiguous()
     b, c, n1 = input.shape
     n2, k = index.size(1), index.size(2)
-    with torch.cuda.device(input.device):
+    with _lib.on_device_of(input):
         output = torch.empty((b, c, n2, k), dtype=input.dtype, device=input.device)
         _lib.call("tk3d_group_points_forward", input, ptr(input), ptr(index), i64(b), i64(c),
                   i64(n1), i64(n2), i64(k), ptr(output), stream_of(input))
@@ -138,7 +138,7 @@ def group_points_backward_cuda(grad_output, index, n1):
     _check_index("index", index)
     n1 = int(n1)
     b, c, n2, k = grad_output.shape
-    with torch.cuda.device(grad_output.device):
+    with _lib.on_device_of(grad_output):
         grad_input = torch.empty((b, c, n1), dtype=grad_output.dtype, device=grad_output.device)
         _lib.call("tk3d_group_points_backward", grad_output, ptr(grad_output), ptr(index),
                   i64(b), i64(c), i64(n1), i64(n2), i64(k), ptr(grad_input),
@@ -168,7 +168,7 @@ def interpolate_forward_cuda(input, index, weight):
     _check_eq(index.size(2), 3, "index.size(2) == 3")
     b, c, n1 = input.shape
     n2, k = index.size(1), index.size(2)
-    with torch.cuda.device(input.device):
+    with _lib.on_device_of(input):
         output = torch.empty((b, c, n2), dtype=input.dtype, device=input.device)
         _lib.call("tk3d_interpolate_forward", input, ptr(input), ptr(index), ptr(weight),
                   i64(b), i64(c), i64(n1), i64(n2), i64(k), ptr(output), stream_of(input))
@@ -184,7 +184,7 @@ def interpolate_backward_cuda(grad_output, index, weight, n1):
     n1 = int(n1)
     b, c, n2 = grad_output.shape
     k = index.size(2)
-    with torch.cuda.device(grad_output.device):
+    with _lib.on_device_of(grad_output):
         grad_input = torch.empty((b, c, n1), dtype=grad_output.dtype, device=grad_output.device)
         _lib.call("tk3d_interpolate_backward", grad_output, ptr(grad_output), ptr(index),
                   ptr(weight), i64(b), i64(c), i64(n1), i64(n2), i64(k), ptr(grad_input),
@@ -208,7 +208,7 @@ def knn_distance_cuda(query, key, k, version):
     _check(int(version) in (0, 1), "Invalid version")
     _check(k >= 0, "k must be non-negative.")
     b, n1, n2 = query.size(0), query.size(1), key.size(1)
-    with torch.cuda.device(query.device):
+    with _lib.on_device_of(query):
         distance = torch.empty((b, n1, k), dtype=query.dtype, device=query.device)
         index = torch.empty((b, n1, k), dtype=torch.int64, device=query.device)
         if k > 0:

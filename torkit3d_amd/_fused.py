@@ -38,7 +38,7 @@ def sample_farthest_points_gather(points, num_samples, channels_first, want_xyz=
     _check(num_samples > 0, "Check failed: num_samples > 0 (%d vs. 0)" % num_samples)
     _check(n >= num_samples,
            "Check failed: points.size(1) >= num_samples (%d vs. %d)" % (n, num_samples))
-    with torch.cuda.device(points.device):
+    with _lib.on_device_of(points):
         index = torch.empty((b, num_samples), dtype=torch.int64, device=points.device)
         sampled = None
         if want_xyz:
@@ -65,7 +65,7 @@ def ball_query_bcn(query, key, radius, max_neighbors):
     _check_same("query", query, "key", key)
     max_neighbors = int(max_neighbors)
     _check(max_neighbors >= 0, "max_neighbors must be non-negative.")
-    with torch.cuda.device(query.device):
+    with _lib.on_device_of(query):
         index = torch.empty((b, n1, max_neighbors), dtype=torch.int64, device=query.device)
         _lib.call("tk3d_ball_query_bcn", query, ptr(query), ptr(key), i64(b), i64(n1), i64(n2),
                   ctypes.c_float(float(radius)), i64(max_neighbors), ptr(index),
@@ -94,7 +94,7 @@ def group_points_concat_forward(feature, xyz, centre, index):
         _check_same("feature", feature, "xyz", xyz)
         c = feature.size(1)
     k = index.size(2)
-    with torch.cuda.device(xyz.device):
+    with _lib.on_device_of(xyz):
         out = torch.empty((b, c + 3, n2, k), dtype=xyz.dtype, device=xyz.device)
         _lib.call("tk3d_group_points_concat_forward", xyz,
                   ptr(feature) if c > 0 else ctypes.c_void_p(0), ptr(xyz), ptr(centre),
@@ -117,7 +117,7 @@ def group_points_concat_backward(grad_output, index, n1, want_feature, want_xyz)
     c = ct - 3
     _check(c >= 0, "grad_output must have at least 3 channels.")
     n1 = int(n1)
-    with torch.cuda.device(grad_output.device):
+    with _lib.on_device_of(grad_output):
         gfeat = gxyz = None
         if want_feature and c > 0:
             gfeat = torch.empty((b, c, n1), dtype=grad_output.dtype, device=grad_output.device)
@@ -141,7 +141,7 @@ def three_nn(query, key, channels_first, eps=1e-10):
     _check_eq(b, b2, "query.size(0) == key.size(0)")
     _check_same("query", query, "key", key)
     _check(n2 >= 3, "Check failed: key.size(1) >= k (%d vs. 3)" % n2)
-    with torch.cuda.device(query.device):
+    with _lib.on_device_of(query):
         distance = torch.empty((b, n1, 3), dtype=query.dtype, device=query.device)
         index = torch.empty((b, n1, 3), dtype=torch.int64, device=query.device)
         weight = torch.empty((b, n1, 3), dtype=query.dtype, device=query.device)

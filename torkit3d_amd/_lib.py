@@ -61,7 +61,34 @@ def suffix(t):
     raise RuntimeError("torkit3d_amd supports float32 and float64 tensors, got %s" % t.dtype)
 
 
+_functions = {}
+
+
 def call(name, tensor_for_dtype, *args):
-    fn = getattr(lib(), name + suffix(tensor_for_dtype))
-    fn.restype = ctypes.c_int
+    key = (name, tensor_for_dtype.dtype)
+    fn = _functions.get(key)
+    if fn is None:
+        fn = getattr(lib(), name + suffix(tensor_for_dtype))
+        fn.restype = ctypes.c_int
+        _functions[key] = fn
     check(fn(*args), name)
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device_of(t):
+    """Context in which the tensor's GPU is current (kernels, allocations and streams
+    follow the current device). Switching costs a few microseconds per call, so nothing
+    is done when that GPU is current already."""
+    if t.device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(t.device)
