@@ -239,12 +239,47 @@ def secondary_metrics(dev, steps, warmup, cpu):
         lambda: _fused.three_nn(q, key, False), steps, 3)
 
     res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()},
-           "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()}}
+           "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()},
+           "model_ms": model_metrics(dev, max(3, steps // 10))}
     if cpu:
         res["cpu_oracle_ms"] = cpu_out
         res["cpu_oracle_note"] = ("OpenMP oracle on %d threads, timed on the first 2-4 clouds of each "
                                   "configuration and scaled to the full batch" % oracle.num_threads())
     return res
+
+
+def model_metrics(dev, steps):
+    """The reference's model zoo on these ops, default constructors, training mode, fp32:
+    one forward pass and one forward + backward pass (loss = mean of the feature)."""
+    import torch
+
+    from torkit3d_amd.models.classification.dgcnn import DGCNN
+    from torkit3d_amd.models.classification.pointnet2 import PN2SSG as PN2Cls
+    from torkit3d_amd.models.segmentation.pointnet2 import PN2SSG as PN2Seg
+
+    g = torch.Generator().manual_seed(6)
+    out = {}
+    for name, make, b, n in (("pn2ssg_seg_B8_N16384", lambda: PN2Seg(3), 8, 16384),
+                             ("pn2ssg_cls_B16_N4096", lambda: PN2Cls(3), 16, 4096),
+                             ("dgcnn_cls_B8_N2048", lambda: DGCNN(3), 8, 2048)):
+        torch.manual_seed(0)
+        model = make().to(dev)
+        points = torch.rand(b, 3, n, generator=g).to(dev)
+        feature = None if name.startswith("dgcnn") else torch.randn(b, 3, n, generator=g).to(dev)
+        args = (points,) if feature is None else (points, feature)
+
+        def forward():
+            with torch.no_grad():
+                model(*args)
+
+        def train_step():
+            model.zero_grad(set_to_none=True)
+            model(*args)["feature"].mean().backward()
+
+        out[name + "_fwd_ms"] = round(gpu_time_ms(forward, steps, 2), 4)
+        out[name + "_fwd_bwd_ms"] = round(gpu_time_ms(train_step, steps, 2), 4)
+        del model
+    return out
 
 
 def main():
@@ -256,6 +291,8 @@ def main():
                     help="skip the CPU oracle timing (for profiler runs)")
     ap.add_argument("--no-secondary", action="store_true",
                     help="time only the chamfer step (for profiler runs)")
+    ap.add_argument("--models-only", action="store_true",
+                    help="time only the model zoo's passes and print those (for profiler runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy, whose known traffic "
                          "scales the profiler's FETCH_SIZE / WRITE_SIZE counters")
@@ -272,6 +309,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = "cuda:0"
+    if args.models_only:
+        print(json.dumps({"model_ms": model_metrics(dev, max(3, args.steps // 10))}))
+        return
     B, N, M = 32, 16384, 16384
     gen = torch.Generator().manual_seed(5)
     a_cpu, c_cpu = sphere_cloud(gen, B, N), sphere_cloud(gen, B, M)
