@@ -238,6 +238,24 @@ def secondary_metrics(dev, steps, warmup, cpu):
     fused["three_nn_weights_fused_ms"] = gpu_time_ms(
         lambda: _fused.three_nn(q, key, False), steps, 3)
 
+    # The same four small launches (ball query, fused grouping, 3-NN with weights,
+    # interpolation) issued from Python and replayed from a captured HIP graph.
+    def small_ops():
+        nb = _fused.ball_query_bcn(ctr_bcn, xyz_bcn, 0.2, 32)
+        _fused.group_points_concat_forward(feat, xyz_bcn, ctr_bcn, nb)
+        _, i3, w3 = _fused.three_nn(xyz_bcn, ctr_bcn, True)
+        return _C.interpolate_forward_cuda(feat_coarse, i3, w3)
+
+    feat_coarse = torch.randn(16, 64, 1024, generator=torch.Generator().manual_seed(7)).to(dev)
+    small_ops()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        small_ops()
+    fused["four_small_ops_eager_ms"] = gpu_time_ms(small_ops, steps, 3)
+    fused["four_small_ops_graph_replay_ms"] = gpu_time_ms(graph.replay, steps, 3)
+    del graph
+
     res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()},
            "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()},
            "model_ms": model_metrics(dev, max(3, steps // 10))}
