@@ -72,13 +72,13 @@ def sample_farthest_points_cuda(points, num_samples):
     b, n = points.size(0), points.size(1)
     with _lib.on_device_of(points):
         index = torch.empty((b, num_samples), dtype=torch.int64, device=points.device)
-        ws_fn = _lib.lib().tk3d_sample_farthest_points_workspace_bytes
-        ws_fn.restype = ctypes.c_size_t
-        ws_bytes = int(ws_fn(i64(b), i64(n), ctypes.c_size_t(points.element_size())))
-        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=points.device)
+        ws_bytes = _lib.fps_workspace_bytes(b, n, points.element_size())
+        ws = None
+        if ws_bytes:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=points.device)
         _lib.call("tk3d_sample_farthest_points", points, ptr(points), i64(b), i64(n),
                   i64(num_samples), ptr(index),
-                  ctypes.c_void_p(ws.data_ptr() if ws_bytes else 0),
+                  ctypes.c_void_p(ws.data_ptr() if ws is not None else 0),
                   ctypes.c_size_t(ws_bytes), stream_of(points))
     return index
 

@@ -44,14 +44,14 @@ def sample_farthest_points_gather(points, num_samples, channels_first, want_xyz=
         if want_xyz:
             shape = (b, 3, num_samples) if channels_first else (b, num_samples, 3)
             sampled = torch.empty(shape, dtype=points.dtype, device=points.device)
-        ws_fn = _lib.lib().tk3d_sample_farthest_points_workspace_bytes
-        ws_fn.restype = ctypes.c_size_t
-        ws_bytes = int(ws_fn(i64(b), i64(n), ctypes.c_size_t(points.element_size())))
-        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=points.device)
+        ws_bytes = _lib.fps_workspace_bytes(b, n, points.element_size())
+        ws = None
+        if ws_bytes:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=points.device)
         _lib.call("tk3d_sample_farthest_points_gather", points, ptr(points),
                   ctypes.c_int(1 if channels_first else 0), i64(b), i64(n), i64(num_samples),
                   ptr(index), ptr(sampled) if sampled is not None else ctypes.c_void_p(0),
-                  ctypes.c_void_p(ws.data_ptr() if ws_bytes else 0),
+                  ctypes.c_void_p(ws.data_ptr() if ws is not None else 0),
                   ctypes.c_size_t(ws_bytes), stream_of(points))
     return index, sampled
 

@@ -62,6 +62,17 @@ def suffix(t):
 
 
 _functions = {}
+_fps_workspace_fn = None
+
+
+def fps_workspace_bytes(b, n, element_size):
+    """Scratch bytes ``tk3d_sample_farthest_points*`` needs for B clouds of N points."""
+    global _fps_workspace_fn
+    if _fps_workspace_fn is None:
+        fn = lib().tk3d_sample_farthest_points_workspace_bytes
+        fn.restype = ctypes.c_size_t
+        _fps_workspace_fn = fn
+    return int(_fps_workspace_fn(i64(b), i64(n), ctypes.c_size_t(element_size)))
 
 
 def call(name, tensor_for_dtype, *args):
