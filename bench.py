@@ -94,6 +94,94 @@ def cpu_ms(fn, scale):
     return round((time.perf_counter() - t0) * 1e3 * scale, 3)
 
 
+def cpu_torch_metrics(tensors):
+    """The reference's CPU path, pure PyTorch on the host cores: the brute-force forms its
+    tests check the kernels against (tests/ops/test_*.py) and ``native.knn``
+    (torkit3d/ops/native.py:28-29), timed on the first clouds of each configuration and
+    scaled to the full batch. ``tensors`` holds CPU copies of the benchmark inputs."""
+    import torch
+
+    t = tensors
+    out = {}
+
+    def timed(fn, scale):
+        t0 = time.perf_counter()
+        fn()
+        return round((time.perf_counter() - t0) * 1e3 * scale, 3)
+
+    def chamfer(a, c, rows=1024):
+        col = torch.full((c.shape[0],), float("inf"))
+        for r in range(0, a.shape[0], rows):
+            d = ((a[r:r + rows, None, :] - c[None, :, :]) ** 2).sum(-1)
+            d.min(dim=1)
+            col = torch.minimum(col, d.min(dim=0).values)
+
+    out["chamfer_fwd_B32_N16384_ms"] = timed(lambda: chamfer(t["a"][0], t["c"][0]), 32)
+
+    def knn(k):
+        for b in range(2):
+            torch.topk(torch.cdist(t["q"][b], t["key"][b]), k, dim=1, largest=False, sorted=False)
+
+    out["knn_B32_N8192_M2048_k16_ms"] = timed(lambda: knn(16), 32 / 2)
+    out["knn_B32_N8192_M2048_k3_ms"] = timed(lambda: knn(3), 32 / 2)
+
+    def fps(p, k):
+        b, n, _ = p.shape
+        cur = torch.zeros(b, dtype=torch.int64)
+        dist = torch.full((b, n), float("inf"))
+        picks = [cur]
+        for _ in range(k - 1):
+            centre = p[torch.arange(b), cur]
+            dist = torch.minimum(dist, ((p - centre[:, None, :]) ** 2).sum(-1))
+            cur = dist.argmax(dim=1)
+            picks.append(cur)
+        return torch.stack(picks, dim=1)
+
+    out["fps_B16_N4096_K1024_ms"] = timed(lambda: fps(t["pts"][:4], 1024), 16 / 4)
+
+    def ball_query(q, key, r, k):
+        d = ((q[:, :, None, :] - key[:, None, :, :]) ** 2).sum(-1)
+        n2 = key.shape[1]
+        cand = torch.where(d < r * r, torch.arange(n2), torch.tensor(n2))
+        first = torch.topk(cand, k, dim=2, largest=False, sorted=True).values
+        first = torch.where(first == n2, first[:, :, :1], first)
+        return torch.where(first == n2, torch.tensor(-1), first)
+
+    out["ball_query_B16_N1024x4096_r0.2_k32_ms"] = timed(
+        lambda: ball_query(t["ctr"][:2], t["xyz"][:2], 0.2, 32), 16 / 2)
+
+    def group(feat, index, grad):
+        b, c, n1 = feat.shape
+        _, n2, k = index.shape
+        flat = index.reshape(b, 1, n2 * k).expand(b, c, n2 * k)
+        feat = feat.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        y = torch.gather(feat, 2, flat)
+        t1 = time.perf_counter()
+        y.backward(grad.reshape(b, c, n2 * k))
+        return (t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3
+
+    fwd, bwd = group(t["feat"][:4], t["nbr"][:4], t["go"][:4])
+    out["group_fwd_B16_C64_N4096_to_1024x32_ms"] = round(fwd * 16 / 4, 3)
+    out["group_bwd_ms"] = round(bwd * 16 / 4, 3)
+
+    def interpolate(feat, index, weight, grad):
+        b, c, n1 = feat.shape
+        n2 = index.shape[1]
+        flat = index.reshape(b, 1, n2 * 3).expand(b, c, n2 * 3)
+        feat = feat.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        y = (torch.gather(feat, 2, flat).view(b, c, n2, 3) * weight[:, None]).sum(-1)
+        t1 = time.perf_counter()
+        y.backward(grad)
+        return (t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3
+
+    fwd, bwd = interpolate(t["f4"][:4], t["kidx"][:4], t["w"][:4], t["g4"][:4])
+    out["interpolate_fwd_B32_C128_ms"] = round(fwd * 32 / 4, 3)
+    out["interpolate_bwd_ms"] = round(bwd * 32 / 4, 3)
+    return out
+
+
 def secondary_metrics(dev, steps, warmup, cpu):
     """ms per call for the other ops at their benchmark shapes (events, same stream).
 
@@ -260,6 +348,15 @@ def secondary_metrics(dev, steps, warmup, cpu):
            "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()},
            "model_ms": model_metrics(dev, max(3, steps // 10))}
     if cpu:
+        res["cpu_torch_ms"] = cpu_torch_metrics({
+            "a": a[:1].cpu(), "c": c[:1].cpu(), "q": q[:2].cpu(), "key": key[:2].cpu(),
+            "pts": pts[:4].cpu(), "ctr": ctr[:2].cpu(), "xyz": xyz[:2].cpu(),
+            "feat": feat[:4].cpu(), "nbr": nbr[:4].cpu(), "go": go[:4].cpu(),
+            "f4": f4[:4].cpu(), "kidx": kidx[:4].cpu(), "w": w[:4].cpu(), "g4": g4[:4].cpu()})
+        res["cpu_torch_note"] = ("pure PyTorch on %d threads: the brute-force forms of the "
+                                 "reference's tests and its native.knn, timed on the first 1-4 "
+                                 "clouds of each configuration and scaled to the full batch"
+                                 % torch.get_num_threads())
         res["cpu_oracle_ms"] = cpu_out
         res["cpu_oracle_note"] = ("OpenMP oracle on %d threads, timed on the first 2-4 clouds of each "
                                   "configuration and scaled to the full batch" % oracle.num_threads())
