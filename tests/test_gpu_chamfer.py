@@ -201,7 +201,7 @@ def _clouds(kind, g):
                                   "separated", "wide_range", "tiny", "huge", "overflowing",
                                   "clusters", "nan_and_inf", "all_nan_keys"])
 def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
-    a, c = _clouds(kind, gen(hash(kind) % 1000))
+    a, c = _clouds(kind, gen(sum(map(ord, kind))))
     check_forward(a.contiguous(), c.contiguous(), cuda)
 
 
@@ -210,3 +210,47 @@ def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
 def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
     g = gen(n1 + n2)
     check_forward(sphere_cloud(g, b, n1), sphere_cloud(g, b, n2), cuda)
+
+
+# ---- split sweeps ----------------------------------------------------------------------
+# When a launch would leave most of the chip idle, each query's sweep is cut into key
+# slices handled by different workgroups, and the partial results meet in a packed
+# 64-bit minimum. The merged result must still be the reference's: smallest distance,
+# lowest key index among equals, (inf, -1) without a finite distance.
+
+@pytest.mark.parametrize("b,n1,n2", [(1, 4096, 4096), (2, 3000, 5000), (1, 20000, 700),
+                                     (1, 777, 65536 + 5), (4, 512, 512), (1, 16384, 16384)])
+def test_split_sweep_shapes(cuda, b, n1, n2):
+    g = gen(n1 * 3 + n2)
+    check_forward(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), cuda)
+
+
+def test_split_sweep_ties_across_slices_keep_the_lowest_index(cuda):
+    from torkit3d_amd import _C
+
+    g = gen(77)
+    a, c = uniform_cloud(g, 1, 2048), uniform_cloud(g, 1, 8192) + 5.0
+    # The same three points sit in the first, a middle and the last part of the key cloud.
+    spots = (100, 101, 3000, 3001, 8000, 8191)
+    for j in spots:
+        c[0, j] = torch.tensor([0.25, -0.5, 0.125]) if j % 2 == 0 else torch.tensor([-0.5, 0.5, 0.75])
+    c[0, 4000] = c[0, 100]
+    check_forward(a, c, cuda)
+    _, i1, _, i2 = _C.chamfer_distance_forward_cuda(a.to(cuda), c.to(cuda))
+    assert set(i1.unique().tolist()) <= {100, 101}
+    # The batch replicated until the launch no longer splits must give the same rows.
+    many = _C.chamfer_distance_forward_cuda(a.expand(96, -1, -1).contiguous().to(cuda),
+                                            c.expand(96, -1, -1).contiguous().to(cuda))
+    one = _C.chamfer_distance_forward_cuda(a.to(cuda), c.to(cuda))
+    for m, o in zip(many, one):
+        assert torch.equal(m[0], o[0]) and torch.equal(m[95], o[0])
+
+
+def test_split_sweep_with_slices_that_hold_no_finite_distance(cuda):
+    g = gen(78)
+    a, c = uniform_cloud(g, 2, 1500), uniform_cloud(g, 2, 6000)
+    c[0, :2500] = float("nan")          # leading slices without a candidate
+    c[0, 5000:, 1] = float("inf")       # trailing slices at infinite distance
+    c[1] = float("nan")                 # a cloud without any candidate: (inf, -1) everywhere
+    a[0, 7] = float("nan")
+    check_forward(a, c, cuda)

@@ -29,7 +29,9 @@ template <typename T> struct ChamferDir {
     int64_t *idx;     // [B, nq]
     int nq;
     int nk;
-    int blocks_per_batch;
+    int blocks_per_batch;  // query blocks x key slices
+    int slices;            // key slices a query's sweep is split into (1: no split)
+    int slice_len;         // keys per slice, a multiple of the tile length
 };
 
 template <typename T> struct ChamferFwdArgs {
@@ -55,7 +57,7 @@ template <> __device__ __forceinline__ double chamfer_init_min<double>()
 // instead of fetching it 8 times.
 template <typename T>
 __device__ __forceinline__ const ChamferDir<T> &chamfer_decode_block(
-    const ChamferFwdArgs<T> &args, int &b, int &qblock)
+    const ChamferFwdArgs<T> &args, int &b, int &qblock, int &slice)
 {
     int lb = blockIdx.x;
     const int nb = gridDim.x, per = nb >> 3, full = per << 3;
@@ -66,21 +68,55 @@ __device__ __forceinline__ const ChamferDir<T> &chamfer_decode_block(
         lb -= args.nblocks0;
     const ChamferDir<T> &d = args.dir[which];
     b = lb / d.blocks_per_batch;
-    qblock = lb - b * d.blocks_per_batch;
+    const int rest = lb - b * d.blocks_per_batch;
+    qblock = rest / d.slices;
+    slice = rest - qblock * d.slices;
     return d;
+}
+
+// Result of one workgroup for query `qi` of batch `b`: distance `dist` to key `j` of the
+// workgroup's slice (j < 0: the slice holds no key with a finite distance).
+//
+// Unsplit sweeps store it. With key slices several workgroups hold partial results for
+// the same query; they meet in the index output, used as 64-bit words that hold
+// (distance bits << 32 | key index): distances are non-negative, so their bit patterns
+// order as unsigned integers and an unsigned minimum of the packed words keeps the
+// smallest distance and, among equal distances, the lowest key index - the reference's
+// strict '<' over ascending j. chamfer_split_init_kernel sets the words to (+inf, -1)
+// beforehand and chamfer_split_finish_kernel unpacks them.
+template <typename T>
+__device__ __forceinline__ void chamfer_emit(const ChamferDir<T> &d, int b, int qi, int k0,
+                                             T dist, int j)
+{
+    const int64_t o = (int64_t)b * d.nq + qi;
+    if constexpr (sizeof(T) == 4) {
+        if (d.slices > 1) {
+            if (j >= 0) {
+                const unsigned long long word =
+                    ((unsigned long long)__builtin_bit_cast(unsigned, dist) << 32) |
+                    (unsigned)(j + k0);
+                atomicMin(reinterpret_cast<unsigned long long *>(d.idx) + o, word);
+            }
+            return;
+        }
+    }
+    d.dist[o] = dist;
+    d.idx[o] = (int64_t)j;
 }
 
 // Exact sweep of one workgroup: QPL*BLOCK queries against the whole key cloud.
 // `skey` is STAGE*4 elements of LDS.
 template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
 __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int b, int qblock,
-                                                    T *skey)
+                                                    int slice, T *skey)
 {
     static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
     const int tid = threadIdx.x;
-    const int nq = d.nq, nk = d.nk;
+    const int nq = d.nq;
+    const int k0 = slice * d.slice_len;  // this workgroup sweeps keys [k0, k0 + nk)
+    const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
     const T *__restrict__ Q = d.query + (int64_t)b * nq * 3;
-    const T *__restrict__ K = d.key + (int64_t)b * nk * 3;
+    const T *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
 
     T qx[QPL], qy[QPL], qz[QPL], best[QPL];
     int btile[QPL];
@@ -101,9 +137,8 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
             const int kj = stage0 + j;
             T x = tk_inf<T>(), y = tk_inf<T>(), z = tk_inf<T>();
             if (kj < nk) {
-                x = K[(int64_t)kj * 3 + 0];
-                y = K[(int64_t)kj * 3 + 1];
-                z = K[(int64_t)kj * 3 + 2];
+                const TkPoint3<T> p = tk_load3<T>(K + (int64_t)kj * 3);
+                x = p.x, y = p.y, z = p.z;
             }
             // Keys past the end sit at +inf: their distance is +inf or NaN and
             // can never lower a minimum.
@@ -160,15 +195,12 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
             const int j0 = btile[i] * TILE;
             const int j1 = (j0 + TILE < nk) ? j0 + TILE : nk;
             for (int j = j1 - 1; j >= j0; --j) {
-                const T kx = K[(int64_t)j * 3 + 0];
-                const T ky = K[(int64_t)j * 3 + 1];
-                const T kz = K[(int64_t)j * 3 + 2];
-                const T dd = tk_dist2<T>(kx, ky, kz, qx[i], qy[i], qz[i]);
+                const TkPoint3<T> p = tk_load3<T>(K + (int64_t)j * 3);
+                const T dd = tk_dist2<T>(p.x, p.y, p.z, qx[i], qy[i], qz[i]);
                 found = (dd == best[i]) ? j : found;
             }
         }
-        d.dist[(int64_t)b * nq + qi] = best[i];
-        d.idx[(int64_t)b * nq + qi] = (int64_t)found;
+        chamfer_emit<T>(d, b, qi, k0, best[i], found);
     }
 }
 
@@ -176,9 +208,9 @@ template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
 __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T> args)
 {
     __shared__ T skey[STAGE * 4 + 8];  // + 2 keys for the read-ahead
-    int b, qblock;
-    const ChamferDir<T> &d = chamfer_decode_block<T>(args, b, qblock);
-    chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+    int b, qblock, slice;
+    const ChamferDir<T> &d = chamfer_decode_block<T>(args, b, qblock, slice);
+    chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE>(d, b, qblock, slice, skey);
 }
 
 // ---- fp32 forward with a bounded-error pre-filter -------------------------------
@@ -219,13 +251,6 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
 // exact sweep for the whole workgroup or the exact scan for the query.
 // Results are therefore bit-identical to the exact sweep for every input.
 
-#ifdef TK3D_CHAMFER_STATS
-// Tuning builds only: [0] queries with two candidate tiles, [1] queries sent to the
-// exact wave scan, [2] queries.
-__device__ unsigned long long tk3d_chamfer_stats[4];
-__device__ long long tk3d_chamfer_stamps[16];
-#endif
-
 __device__ __forceinline__ float wave_reduce_min(float v)
 {
 #pragma unroll
@@ -257,8 +282,8 @@ __device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict
     int bj = -1;
 #pragma unroll 8
     for (int j = tid; j < nk; j += BLOCK) {
-        const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
-                                        K[(int64_t)j * 3 + 2], qx, qy, qz);
+        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const float d = tk_dist2<float>(p.x, p.y, p.z, qx, qy, qz);
         if (d < best) {
             best = d;
             bj = j;
@@ -306,21 +331,25 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     const int tid = threadIdx.x;
     const int lane = tid & (TK_WAVE - 1);
     const int wave = tid / TK_WAVE;
-    int b, qblock;
-    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock);
-    const int nq = d.nq, nk = d.nk;
+    int b, qblock, slice;
+    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
+    const int nq = d.nq;
+    // This workgroup sweeps keys [k0, k0 + nk); to the filter that slice is the key cloud.
+    const int k0 = slice * d.slice_len;
+    const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
     const float *__restrict__ Q = d.query + (int64_t)b * nq * 3;
-    const float *__restrict__ K = d.key + (int64_t)b * nk * 3;
+    const float *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
     const float INF = __builtin_huge_valf();
 
     // ---- bounding box of the key cloud -> centre ----
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
     for (int j = tid; j < nk; j += BLOCK) {
+        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const float v[3] = {p.x, p.y, p.z};
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-            const float v = K[(int64_t)j * 3 + a];
-            lo[a] = __builtin_fminf(lo[a], v);
-            hi[a] = __builtin_fmaxf(hi[a], v);
+            lo[a] = __builtin_fminf(lo[a], v[a]);
+            hi[a] = __builtin_fmaxf(hi[a], v[a]);
         }
     }
 #pragma unroll
@@ -353,9 +382,10 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     // ---- largest centred squared norm, computed as the staging below computes it ----
     float kmax2 = 0.0f;
     for (int j = tid; j < nk; j += BLOCK) {
-        const float x = K[(int64_t)j * 3 + 0] - c0;
-        const float y = K[(int64_t)j * 3 + 1] - c1;
-        const float z = K[(int64_t)j * 3 + 2] - c2;
+        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const float x = p.x - c0;
+        const float y = p.y - c1;
+        const float z = p.z - c2;
         kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
     }
     kmax2 = wave_reduce_max(kmax2);
@@ -371,7 +401,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
                       (kmax2 < 1e30f);
     if (!safe) {  // uniform over the workgroup
-        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, slice, skey);
         return;
     }
     // sqrt and the norm carry a few u of rounding; 1e-6 covers them.
@@ -416,9 +446,10 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
             const int kj = st * STAGE + r * BLOCK + tid;
             float4 e = make_float4(0.0f, 0.0f, 0.0f, INF);  // past the end: s = +inf
             if (kj < nk) {
-                e.x = K[(int64_t)kj * 3 + 0] - c0;
-                e.y = K[(int64_t)kj * 3 + 1] - c1;
-                e.z = K[(int64_t)kj * 3 + 2] - c2;
+                const TkPoint3<float> p = tk_load3<float>(K + (int64_t)kj * 3);
+                e.x = p.x - c0;
+                e.y = p.y - c1;
+                e.z = p.z - c2;
                 e.w = __builtin_fmaf(e.z, e.z, __builtin_fmaf(e.y, e.y, e.x * e.x));
             }
             pre[r] = e;
@@ -504,7 +535,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
             if (tid == 0)
                 s_count = 0;
             if (total * 4 > QPL * BLOCK) {  // uniform over the workgroup
-                chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+                chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, slice, skey);
                 return;
             }
         }
@@ -556,12 +587,28 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
                         if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
                         if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
                     }
+                } else if (j0 + TILE <= nk) {
+                    // Rows of this cloud are not 16-byte aligned: one 12-byte load per key.
+#pragma unroll 2
+                    for (int g = 0; g < TILE / 4; ++g) {
+                        const int j = j0 + g * 4;
+                        const TkPoint3<float> p0 = tk_load3<float>(K + (int64_t)j * 3);
+                        const TkPoint3<float> p1 = tk_load3<float>(K + (int64_t)j * 3 + 3);
+                        const TkPoint3<float> p2 = tk_load3<float>(K + (int64_t)j * 3 + 6);
+                        const TkPoint3<float> p3 = tk_load3<float>(K + (int64_t)j * 3 + 9);
+                        const float dd0 = tk_dist2<float>(p0.x, p0.y, p0.z, qx, qy, qz);
+                        const float dd1 = tk_dist2<float>(p1.x, p1.y, p1.z, qx, qy, qz);
+                        const float dd2 = tk_dist2<float>(p2.x, p2.y, p2.z, qx, qy, qz);
+                        const float dd3 = tk_dist2<float>(p3.x, p3.y, p3.z, qx, qy, qz);
+                        if (dd0 < bestd) { bestd = dd0; bestj = j; }
+                        if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
+                        if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
+                        if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
+                    }
                 } else {
-                    const int j1 = (j0 + TILE < nk) ? j0 + TILE : nk;
-                    for (int j = j0; j < j1; ++j) {
-                        const float dd = tk_dist2<float>(K[(int64_t)j * 3 + 0],
-                                                         K[(int64_t)j * 3 + 1],
-                                                         K[(int64_t)j * 3 + 2], qx, qy, qz);
+                    for (int j = j0; j < nk; ++j) {
+                        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+                        const float dd = tk_dist2<float>(p.x, p.y, p.z, qx, qy, qz);
                         if (dd < bestd) {
                             bestd = dd;
                             bestj = j;
@@ -570,30 +617,20 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
                 }
             }
         }
-        if (ok && !over) {
-            d.dist[(int64_t)b * nq + qi] = bestd;
-            d.idx[(int64_t)b * nq + qi] = (int64_t)bestj;
-        }
+        if (ok && !over)
+            chamfer_emit<float>(d, b, qi, k0, bestd, bestj);
         if (over) {
             const int slot = atomicAdd(&s_count, 1);
             if (slot < MAX_SCANS)
                 s_list[slot] = i * BLOCK + tid;
         }
-#ifdef TK3D_CHAMFER_STATS
-        if (ok && !none && !over && second)
-            atomicAdd(&tk3d_chamfer_stats[0], 1ull);
-        if (over)
-            atomicAdd(&tk3d_chamfer_stats[1], 1ull);
-        if (ok)
-            atomicAdd(&tk3d_chamfer_stats[2], 1ull);
-#endif
     }
 
     // ---- queries with three or more candidate tiles ----
     __syncthreads();
     const int nscan = s_count;
     if (nscan > MAX_SCANS) {  // uniform over the workgroup
-        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, skey);
+        chamfer_exact_sweep<float, QPL, BLOCK, TILE, STAGE>(d, b, qblock, slice, skey);
         return;
     }
     for (int e = 0; e < nscan; ++e) {
@@ -603,10 +640,8 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
         int bj;
         chamfer_block_exact_scan<BLOCK>(K, nk, Q[(int64_t)qi * 3 + 0], Q[(int64_t)qi * 3 + 1],
                                         Q[(int64_t)qi * 3 + 2], &sred[0][0], sidx, bd, bj);
-        if (tid == 0) {
-            d.dist[(int64_t)b * nq + qi] = bd;
-            d.idx[(int64_t)b * nq + qi] = (int64_t)bj;
-        }
+        if (tid == 0)
+            chamfer_emit<float>(d, b, qi, k0, bd, bj);
     }
 }
 
@@ -724,12 +759,6 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     float *__restrict__ out = (second ? gx2 : gx1) + (int64_t)b * nx * 3;
     const int j1 = (j0 + R < nx) ? j0 + R : nx;
 
-#ifdef TK3D_CHAMFER_STATS
-#define TK3D_STAMP(n) do { if (blockIdx.x == 0 && threadIdx.x == 0) tk3d_chamfer_stamps[n] = wall_clock64(); } while (0)
-#else
-#define TK3D_STAMP(n) do { } while (0)
-#endif
-    TK3D_STAMP(0);
     bool use_float = false;
     for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
         __syncthreads();
@@ -789,7 +818,6 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
         if ((threadIdx.x & 63) == 0 && m != 0u)
             atomicMax(&s_max, m);
         __syncthreads();
-        TK3D_STAMP(1 + attempt * 4);
         const float bound = __builtin_bit_cast(float, s_max) * (attempt == 0 ? 8.0f : 1.000001f);
         if (!(bound < 3.0e38f)) {  // NaN or inf
             use_float = true;
@@ -849,7 +877,6 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
         if (exceeded)
             s_exceeded = 1;
         __syncthreads();
-        TK3D_STAMP(2 + attempt * 4);
         if (!s_exceeded) {
             // own terms: a lane takes whole points, F of them per round, with the
             // match indices and then the matched points fetched together
@@ -889,7 +916,6 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
                     }
                 }
             }
-            TK3D_STAMP(3 + attempt * 4);
             return;
         }
     }
@@ -921,46 +947,166 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     }
 }
 
+// Split sweeps: the index outputs start as packed (+inf, -1) words ...
+__global__ __launch_bounds__(256) void chamfer_split_init_kernel(ChamferFwdArgs<float> args,
+                                                                 int64_t total0, int64_t total1)
+{
+    const unsigned long long word = (0x7f800000ull << 32) | 0xffffffffull;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < total0) {
+        if (args.dir[0].slices > 1)
+            reinterpret_cast<unsigned long long *>(args.dir[0].idx)[i] = word;
+    } else if (i - total0 < total1) {
+        if (args.dir[1].slices > 1)
+            reinterpret_cast<unsigned long long *>(args.dir[1].idx)[i - total0] = word;
+    }
+}
+
+// ... and are unpacked into distance and index once every slice has been merged.
+__global__ __launch_bounds__(256) void chamfer_split_finish_kernel(ChamferFwdArgs<float> args,
+                                                                   int64_t total0, int64_t total1)
+{
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int which = i >= total0;
+    if (which)
+        i -= total0;
+    if (i >= (which ? total1 : total0))
+        return;
+    const ChamferDir<float> &d = args.dir[which];
+    if (d.slices <= 1)
+        return;
+    const unsigned long long word = reinterpret_cast<const unsigned long long *>(d.idx)[i];
+    d.dist[i] = __builtin_bit_cast(float, (unsigned)(word >> 32));
+    d.idx[i] = (int64_t)(int)(unsigned)word;
+}
+
+// A key cloud of `nk` points cut into about `want` slices of whole tiles: returns the
+// number of slices and their length.
+inline int64_t chamfer_slices(int64_t nk, int64_t want, int tile, int64_t &len)
+{
+    len = nk;
+    if (want <= 1 || nk <= tile)
+        return 1;
+    len = (nk + want - 1) / want;
+    len = (len + tile - 1) / tile * tile;
+    return (nk + len - 1) / len;
+}
+
+// Fills the launch description. `want_slices` > 1 asks for that many key slices per
+// query (fp32 only); each direction gets as many as its key cloud has whole tiles for.
+template <typename T, int QB, int TILE>
+int chamfer_fill_args(ChamferFwdArgs<T> &a, const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
+                      int64_t N2, T *dist1, int64_t *idx1, T *dist2, int64_t *idx2,
+                      int want_slices, int64_t &nblocks)
+{
+    const T *q[2] = {xyz1, xyz2}, *k[2] = {xyz2, xyz1};
+    T *dist[2] = {dist1, dist2};
+    int64_t *idx[2] = {idx1, idx2};
+    const int64_t nq[2] = {N1, N2}, nk[2] = {N2, N1};
+    int64_t nb[2];
+    for (int w = 0; w < 2; ++w) {
+        int64_t len;
+        const int64_t slices = chamfer_slices(nk[w], sizeof(T) == 4 ? want_slices : 1, TILE, len);
+        const int64_t qblocks = (nq[w] + QB - 1) / QB;
+        a.dir[w] = {q[w], k[w], dist[w], idx[w], (int)nq[w], (int)nk[w],
+                    (int)(qblocks * slices), (int)slices, (int)(len > 0 ? len : 1)};
+        nb[w] = B * qblocks * slices;
+    }
+    nblocks = nb[0] + nb[1];
+    if (nblocks > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    a.nblocks0 = (int)nb[0];
+    return TK3D_OK;
+}
+
+// Launches `kernel` on the filled description, bracketed by the init / finish kernels
+// when any direction is split.
+template <typename T, typename Kernel>
+int chamfer_forward_run(Kernel kernel, int block, const ChamferFwdArgs<T> &a, int64_t nblocks,
+                        int64_t B, hipStream_t stream)
+{
+    if (nblocks == 0)
+        return TK3D_OK;
+    bool split = false;
+    if constexpr (sizeof(T) == 4) {
+        split = a.dir[0].slices > 1 || a.dir[1].slices > 1;
+        if (split) {
+            const int64_t t0 = B * a.dir[0].nq, t1 = B * a.dir[1].nq;
+            const unsigned grid = (unsigned)((t0 + t1 + 255) / 256);
+            hipLaunchKernelGGL(chamfer_split_init_kernel, dim3(grid), dim3(256), 0, stream, a, t0,
+                               t1);
+            hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(block), 0, stream, a);
+            hipLaunchKernelGGL(chamfer_split_finish_kernel, dim3(grid), dim3(256), 0, stream, a,
+                               t0, t1);
+            return tk_launch_status();
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(block), 0, stream, a);
+    return tk_launch_status();
+}
+
 template <typename T, int QPL, int BLOCK = 256, int TILE = 32, int STAGE = 1024>
 int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
                            int64_t N2, T *dist1, int64_t *idx1, T *dist2,
-                           int64_t *idx2, hipStream_t stream)
+                           int64_t *idx2, hipStream_t stream, int slices = 1)
 {
-    constexpr int QB = QPL * BLOCK;
     ChamferFwdArgs<T> a;
-    a.dir[0] = {xyz1, xyz2, dist1, idx1, (int)N1, (int)N2, (int)((N1 + QB - 1) / QB)};
-    a.dir[1] = {xyz2, xyz1, dist2, idx2, (int)N2, (int)N1, (int)((N2 + QB - 1) / QB)};
-    const int64_t nb0 = B * a.dir[0].blocks_per_batch;
-    const int64_t nb1 = B * a.dir[1].blocks_per_batch;
-    if (nb0 + nb1 == 0)
-        return TK3D_OK;
-    if (nb0 + nb1 > TK_MAX_I32)
-        return TK3D_ERR_UNSUPPORTED;
-    a.nblocks0 = (int)nb0;
-    hipLaunchKernelGGL((chamfer_forward_kernel<T, QPL, BLOCK, TILE, STAGE>),
-                       dim3((unsigned)(nb0 + nb1)), dim3(BLOCK), 0, stream, a);
-    return tk_launch_status();
+    int64_t nblocks;
+    const int rc = chamfer_fill_args<T, QPL * BLOCK, TILE>(a, xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                           dist2, idx2, slices, nblocks);
+    if (rc != TK3D_OK)
+        return rc;
+    return chamfer_forward_run<T>(chamfer_forward_kernel<T, QPL, BLOCK, TILE, STAGE>, BLOCK, a,
+                                  nblocks, B, stream);
 }
 
 template <int QPL, int BLOCK = 256, int TILE = 64, int STAGE = 1024>
 int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                                   int64_t N2, float *dist1, int64_t *idx1, float *dist2,
-                                  int64_t *idx2, hipStream_t stream)
+                                  int64_t *idx2, hipStream_t stream, int slices = 1)
 {
-    constexpr int QB = QPL * BLOCK;
     ChamferFwdArgs<float> a;
-    a.dir[0] = {xyz1, xyz2, dist1, idx1, (int)N1, (int)N2, (int)((N1 + QB - 1) / QB)};
-    a.dir[1] = {xyz2, xyz1, dist2, idx2, (int)N2, (int)N1, (int)((N2 + QB - 1) / QB)};
-    const int64_t nb0 = B * a.dir[0].blocks_per_batch;
-    const int64_t nb1 = B * a.dir[1].blocks_per_batch;
-    if (nb0 + nb1 == 0)
-        return TK3D_OK;
-    if (nb0 + nb1 > TK_MAX_I32)
-        return TK3D_ERR_UNSUPPORTED;
-    a.nblocks0 = (int)nb0;
-    hipLaunchKernelGGL((chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE>),
-                       dim3((unsigned)(nb0 + nb1)), dim3(BLOCK), 0, stream, a);
-    return tk_launch_status();
+    int64_t nblocks;
+    const int rc = chamfer_fill_args<float, QPL * BLOCK, TILE>(
+        a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, slices, nblocks);
+    if (rc != TK3D_OK)
+        return rc;
+    return chamfer_forward_run<float>(chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE>,
+                                      BLOCK, a, nblocks, B, stream);
+}
+
+// Estimated duration in microseconds of the pre-filtered sweep launched as `qpl`
+// queries per lane, `block` lanes per workgroup and `want_slices` key slices; used only
+// to rank launch shapes. A wave issues qpl * ipp vector instructions per key (ipp per
+// pair: 3.76 measured with 4 queries per lane, 4.5 with 2, which reads LDS and keeps tile
+// minima twice as often), plus a prologue and epilogue worth `overhead_keys` keys per
+// slice (about 250 for 256-lane workgroups, 500 for 512-lane ones).
+// A SIMD with n resident waves finishes them in max(2.4 n, 5.5) cycles per instruction
+// of one wave: 2.4 is the issue cost of the instruction mix, 5.5 what a lone wave
+// achieves between dependent instructions. Workgroups spread over 256 CUs, so n steps
+// with ceil(workgroups / 256). 12 us cover launch and fixed latencies, 20 us with the
+// two extra launches of a split sweep. Within 8 % of the best shape (1 % on average) on
+// 54 timed shapes from B=1, N=512 to B=32, N=16384 and B=4, N=65536.
+inline double chamfer_sweep_cost(int64_t B, int64_t N1, int64_t N2, int qpl, int block,
+                                 double ipp, double overhead_keys, int want_slices)
+{
+    const int64_t nq[2] = {N1, N2}, nk[2] = {N2, N1};
+    const int64_t qb = (int64_t)qpl * block;
+    double groups = 0.0, instructions = 0.0;
+    for (int w = 0; w < 2; ++w) {
+        int64_t len;
+        const int64_t slices = chamfer_slices(nk[w], want_slices, 64, len);
+        const double g = (double)B * (double)((nq[w] + qb - 1) / qb) * (double)slices;
+        groups += g;
+        instructions += g * qpl * ((double)len + overhead_keys) * ipp;
+    }
+    if (groups == 0.0)
+        return 0.0;
+    const double per_wave = instructions / groups;
+    const double rounds = (double)(((int64_t)groups + 255) / 256);
+    const double resident = rounds * (block / 64) / 4.0;  // waves per SIMD
+    const double cycles = per_wave * (2.4 * resident > 5.5 ? 2.4 * resident : 5.5);
+    return (want_slices > 1 ? 20.0 : 12.0) + cycles / 2100.0;
 }
 
 template <typename T>
@@ -981,18 +1127,27 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
     // spreads over the chip.
     const int64_t work = B * (N1 > N2 ? N1 : N2);
     if constexpr (sizeof(T) == 4) {
-        // The pre-filter pays off once the key cloud is long enough to amortise its
-        // prologue (two passes over the keys per workgroup).
+        // The pre-filter pays off once the key clouds are a few hundred points long
+        // (its prologue passes over the keys twice per workgroup).
         const int64_t nkmin = N1 < N2 ? N1 : N2;
-        if (nkmin >= 2048) {
-            // Shapes timed on an MI355X: 4 queries per lane; 512-lane workgroups once
-            // that still gives every CU two of them.
-            if (B * (N1 + N2) >= (int64_t)2048 * 512)
+        if (nkmin >= 512) {
+            // Launch shapes: 4 queries per lane in 512-lane workgroups is the fastest
+            // sweep once it fills the chip; below that 2 queries per lane in 256-lane
+            // workgroups, with the key cloud cut into slices when even those are too few.
+            double best = chamfer_sweep_cost(B, N1, N2, 4, 512, 3.76, 500.0, 1);
+            int best_slices = 0;  // 0: the 4 x 512 shape
+            for (int slices = 1; slices <= 16; slices *= 2) {
+                const double c = chamfer_sweep_cost(B, N1, N2, 2, 256, 4.5, 250.0, slices);
+                if (c < best) {
+                    best = c;
+                    best_slices = slices;
+                }
+            }
+            if (best_slices == 0)
                 return chamfer_forward_filter_launch<4, 512, 64, 512>(
                     xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s);
-            if (B * (N1 + N2) >= (int64_t)1024 * 256)
-                return chamfer_forward_filter_launch<4, 256, 64, 512>(
-                    xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s);
+            return chamfer_forward_filter_launch<2, 256, 64, 512>(
+                xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s, best_slices);
         }
     }
     if (sizeof(T) == 8 || work < (int64_t)256 * 1024)

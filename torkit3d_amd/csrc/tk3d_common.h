@@ -63,6 +63,16 @@ __device__ __forceinline__ T tk_dist2(T kx, T ky, T kz, T qx, T qy, T qz)
     return d;
 }
 
+// The three coordinates p[0..2] of one point as a single 12-byte (fp64: 24-byte) load;
+// p needs only the alignment of T, which is all a row of an [N,3] array has.
+template <typename T> struct __attribute__((packed, aligned(sizeof(T)))) TkPoint3 {
+    T x, y, z;
+};
+template <typename T> __device__ __forceinline__ TkPoint3<T> tk_load3(const T *p)
+{
+    return *reinterpret_cast<const TkPoint3<T> *>(p);
+}
+
 // ---- host side --------------------------------------------------------------
 
 static inline int tk_launch_status()
