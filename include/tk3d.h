@@ -57,7 +57,9 @@ const char *tk3d_error_string(int code);
  * (torkit3d/csrc/include/chamfer_distance.h:6-8, cuda/chamfer_distance_kernel.cu:91-151).
  * dist1[b,i] = min_j d2(xyz1[b,i], xyz2[b,j]), idx1[b,i] = the lowest such j;
  * dist2/idx2 likewise with the clouds swapped. An empty or all-NaN opposite
- * cloud gives (+inf, -1) in fp32. B, N1, N2 may be 0. */
+ * cloud gives (+inf, -1) in fp32. B, N1, N2 may be 0. The fp32 call may enqueue up
+ * to three kernels and keeps partial results in idx1 / idx2 (8-byte aligned, as any
+ * int64 array is) while they run; all four outputs are final when the last one ends. */
 int tk3d_chamfer_distance_forward_f32(const float *xyz1, const float *xyz2,
                                       int64_t B, int64_t N1, int64_t N2,
                                       float *dist1, int64_t *idx1, float *dist2,
