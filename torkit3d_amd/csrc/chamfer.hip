@@ -1032,6 +1032,8 @@ int chamfer_forward_run(Kernel kernel, int block, const ChamferFwdArgs<T> &a, in
         split = a.dir[0].slices > 1 || a.dir[1].slices > 1;
         if (split) {
             const int64_t t0 = B * a.dir[0].nq, t1 = B * a.dir[1].nq;
+            if ((t0 + t1 + 255) / 256 > TK_MAX_I32)
+                return TK3D_ERR_UNSUPPORTED;
             const unsigned grid = (unsigned)((t0 + t1 + 255) / 256);
             hipLaunchKernelGGL(chamfer_split_init_kernel, dim3(grid), dim3(256), 0, stream, a, t0,
                                t1);
