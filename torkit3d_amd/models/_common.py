@@ -2,6 +2,7 @@
 import torch
 from torch import nn
 
+from ..layers.pointnet2 import BallQuery, SetAbstraction
 from ..nn import batch_index_select
 from ..ops.sample_farthest_points import sample_farthest_points, sample_farthest_points_gather
 
@@ -28,3 +29,27 @@ def farthest_points_xyz(points, num_samples):
         return batch_index_select(points, index, dim=2)
     _, xyz = sample_farthest_points_gather(points, num_samples, True)
     return xyz
+
+
+def set_abstraction_levels(in_channels, mlp_channels, radii, neighbors, use_xyz):
+    """One ``SetAbstraction`` per level, each fed by the previous level's features."""
+    levels = nn.ModuleList()
+    for channels, radius, count in zip(mlp_channels, radii, neighbors):
+        levels.append(SetAbstraction(in_channels=in_channels, mlp_channels=channels,
+                                     query_neighbor=BallQuery(radius=radius, max_neighbors=count),
+                                     use_xyz=use_xyz))
+        in_channels = channels[-1]
+    return levels
+
+
+def descend(levels, num_samples, points, feature):
+    """Runs the levels on prefixes of one farthest point sample (a prefix of a farthest
+    point sample is the sample of that size, which is why the reference samples once).
+
+    Returns the coordinates and features of every level, the input cloud first."""
+    sampled = farthest_points_xyz(points, num_samples[0])
+    xyz, features = [points], [feature]
+    for level, count in zip(levels, num_samples):
+        xyz.append(sampled[..., :count])
+        features.append(level(xyz[-2], xyz[-1], features[-1]))
+    return xyz, features

@@ -3,9 +3,8 @@
 import torch
 from torch import nn
 
-from ...layers.pointnet2 import BallQuery, SetAbstraction
 from ...nn import mlp1d_bn_relu
-from .._common import farthest_points_xyz, zero_biases
+from .._common import descend, set_abstraction_levels, zero_biases
 
 __all__ = ["PN2SSG"]
 
@@ -26,29 +25,16 @@ class PN2SSG(nn.Module):
         self.radius_list = radius_list
         self.num_neighbors = num_neighbors
         self.use_xyz = use_xyz
-
-        self.sa_layers = nn.ModuleList()
-        c_in = in_channels
-        for channels, radius, neighbors in zip(sa_channels, radius_list, num_neighbors):
-            self.sa_layers.append(SetAbstraction(
-                in_channels=c_in, mlp_channels=channels,
-                query_neighbor=BallQuery(radius=radius, max_neighbors=neighbors),
-                use_xyz=use_xyz))
-            c_in = channels[-1]
-        self.mlp_local = mlp1d_bn_relu(c_in, local_channels)
+        self.sa_layers = set_abstraction_levels(in_channels, sa_channels, radius_list,
+                                                num_neighbors, use_xyz)
+        self.mlp_local = mlp1d_bn_relu(sa_channels[-1][-1], local_channels)
         self.reset_parameters()
 
     def forward(self, points, points_feature=None):
         """points [B,3,N], points_feature [B,C,N] or None
         -> {"feature": [B, out_channels], "max_indices": [B, out_channels]}."""
-        xyz_fps = farthest_points_xyz(points, self.num_samples[0])
-        xyz, feature = points, points_feature
-        for sa_layer, count in zip(self.sa_layers, self.num_samples):
-            # A prefix of a farthest point sample is the sample of that size.
-            next_xyz = xyz_fps[..., :count]
-            feature = sa_layer(xyz, next_xyz, feature)
-            xyz = next_xyz
-        pooled, max_indices = torch.max(self.mlp_local(feature), 2)
+        _, features = descend(self.sa_layers, self.num_samples, points, points_feature)
+        pooled, max_indices = torch.max(self.mlp_local(features[-1]), 2)
         return {"feature": pooled, "max_indices": max_indices}
 
     def reset_parameters(self):

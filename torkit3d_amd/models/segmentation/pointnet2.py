@@ -2,8 +2,8 @@
 (torkit3d/models/segmentation/pointnet2.py)."""
 from torch import nn
 
-from ...layers.pointnet2 import BallQuery, FeaturePropagation, SetAbstraction
-from .._common import farthest_points_xyz, zero_biases
+from ...layers.pointnet2 import FeaturePropagation
+from .._common import descend, set_abstraction_levels, zero_biases
 
 __all__ = ["PN2SSG"]
 
@@ -22,16 +22,8 @@ class PN2SSG(nn.Module):
         self.out_channels = 128 + in_channels
         self.num_samples = num_samples
         self.use_xyz = use_xyz
-
-        self.sa_layers = nn.ModuleList()
-        c_in = in_channels
-        for channels, radius in zip(_SA_CHANNELS, radius_list):
-            self.sa_layers.append(SetAbstraction(
-                in_channels=c_in, mlp_channels=channels,
-                query_neighbor=BallQuery(radius=radius, max_neighbors=max_neighbors),
-                use_xyz=use_xyz))
-            c_in = channels[-1]
-
+        self.sa_layers = set_abstraction_levels(in_channels, _SA_CHANNELS, radius_list,
+                                                (max_neighbors,) * 4, use_xyz)
         # (coarse features + skip features, MLP) from the coarsest level upwards.
         self.fp_layers = nn.ModuleList([
             FeaturePropagation(in_channels=512 + 256, mlp_channels=(256, 256)),
@@ -44,24 +36,15 @@ class PN2SSG(nn.Module):
     def forward(self, points, points_feature=None):
         """points [B,3,N], points_feature [B,C,N] or None -> {"feature": [B,128,N],
         "fp_feature0".."fp_feature3": the output of every propagation level}."""
-        xyz_fps = farthest_points_xyz(points, self.num_samples[0])
-
-        xyz = [points]
-        feature = [points_feature]
-        for sa_layer, count in zip(self.sa_layers, self.num_samples):
-            # A prefix of a farthest point sample is the sample of that size.
-            xyz.append(xyz_fps[..., :count])
-            feature.append(sa_layer(xyz[-2], xyz[-1], feature[-1]))
-
-        outputs = {}
-        coarse = feature[4]
+        xyz, features = descend(self.sa_layers, self.num_samples, points, points_feature)
+        upward = {}
+        coarse = features[4]
         for step, fp_layer in enumerate(self.fp_layers):
             level = 3 - step
-            coarse = fp_layer(xyz[level + 1], coarse, xyz[level], feature[level])
-            outputs["fp_feature%d" % level] = coarse
+            coarse = fp_layer(xyz[level + 1], coarse, xyz[level], features[level])
+            upward["fp_feature%d" % level] = coarse
         pred_dict = {"feature": coarse}
-        for level in range(4):
-            pred_dict["fp_feature%d" % level] = outputs["fp_feature%d" % level]
+        pred_dict.update((key, upward[key]) for key in sorted(upward))
         return pred_dict
 
     def reset_parameters(self):

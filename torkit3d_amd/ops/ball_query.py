@@ -1,25 +1,16 @@
 """Ball query (API of torkit3d/ops/ball_query.py)."""
-import torch
-
 from .. import _C, _fused
+from ._common import NoGradient
 
 
-class BallQueryFunction(torch.autograd.Function):
+class BallQueryFunction(NoGradient):
     """Not differentiable (torkit3d/ops/ball_query.py:6-14). ``channels_first``
     (not in the reference) says the clouds are [B, 3, N]."""
 
     @staticmethod
-    def forward(ctx, query, key, radius, max_neighbors, channels_first=False):
-        if channels_first:
-            index = _fused.ball_query_bcn(query, key, radius, max_neighbors)
-        else:
-            index = _C.ball_query_cuda(query, key, radius, max_neighbors)
-        ctx.mark_non_differentiable(index)
-        return index
-
-    @staticmethod
-    def backward(ctx, *grad_outputs):
-        return (None,) * 5
+    def run(query, key, radius, max_neighbors, channels_first=False):
+        op = _fused.ball_query_bcn if channels_first else _C.ball_query_cuda
+        return op(query, key, radius, max_neighbors)
 
 
 def ball_query(query, key, radius, max_neighbors, transpose=True):

@@ -2,38 +2,31 @@
 import torch
 
 from .. import _C
+from ._common import on_gpu, rows_of_points, with_batch_dim
 
 
 def safe_sqrt(x, eps=1e-12):
     """sqrt(max(x, eps)) (torkit3d/ops/chamfer_distance.py:6-7)."""
-    return torch.sqrt(torch.clamp(x, eps))
+    return torch.clamp(x, eps).sqrt()
 
 
 class ChamferDistanceFunction(torch.autograd.Function):
     """forward(xyz1, xyz2) -> (dist1, dist2); backward(grad_dist1, grad_dist2) ->
-    (grad_xyz1, grad_xyz2) (torkit3d/ops/chamfer_distance.py:10-29)."""
+    (grad_xyz1, grad_xyz2) (torkit3d/ops/chamfer_distance.py:10-29). The matches found
+    by the forward kernel are kept for the backward kernel, which needs nothing else."""
 
     @staticmethod
     def forward(ctx, xyz1, xyz2):
-        xyz1, xyz2 = xyz1.contiguous(), xyz2.contiguous()
-        assert xyz1.is_cuda and xyz2.is_cuda, "Only support cuda currently."
-        dist1, idx1, dist2, idx2 = _C.chamfer_distance_forward_cuda(xyz1, xyz2)
-        ctx.save_for_backward(xyz1, xyz2, idx1, idx2)
+        clouds = on_gpu(xyz1, xyz2)
+        dist1, idx1, dist2, idx2 = _C.chamfer_distance_forward_cuda(*clouds)
+        ctx.save_for_backward(*clouds, idx1, idx2)
         ctx.mark_non_differentiable(idx1, idx2)
         return dist1, dist2
 
     @staticmethod
     def backward(ctx, grad_dist1, grad_dist2):
-        xyz1, xyz2, idx1, idx2 = ctx.saved_tensors
-        grad_dist1, grad_dist2 = grad_dist1.contiguous(), grad_dist2.contiguous()
-        assert grad_dist1.is_cuda and grad_dist2.is_cuda, "Only support cuda currently."
-        grad_xyz1, grad_xyz2 = _C.chamfer_distance_backward_cuda(
-            grad_dist1, grad_dist2, xyz1, xyz2, idx1, idx2)
-        return grad_xyz1, grad_xyz2
-
-
-def _batched(xyz):
-    return xyz.unsqueeze(0) if xyz.dim() == 2 else xyz
+        grads = on_gpu(grad_dist1, grad_dist2)
+        return tuple(_C.chamfer_distance_backward_cuda(*grads, *ctx.saved_tensors))
 
 
 def chamfer_distance(xyz1, xyz2, transpose=False, sqrt=False, eps=1e-12):
@@ -49,20 +42,15 @@ def chamfer_distance(xyz1, xyz2, transpose=False, sqrt=False, eps=1e-12):
     Returns:
         dist1 (b, n1), dist2 (b, n2).
     """
-    xyz1, xyz2 = _batched(xyz1), _batched(xyz2)
-    if transpose:
-        xyz1, xyz2 = xyz1.transpose(1, 2), xyz2.transpose(1, 2)
-    dist1, dist2 = ChamferDistanceFunction.apply(xyz1, xyz2)
-    if sqrt:
-        dist1, dist2 = safe_sqrt(dist1, eps), safe_sqrt(dist2, eps)
-    return dist1, dist2
+    clouds = [rows_of_points(with_batch_dim(c), transpose) for c in (xyz1, xyz2)]
+    dists = ChamferDistanceFunction.apply(*clouds)
+    return tuple(safe_sqrt(d, eps) for d in dists) if sqrt else dists
 
 
 def nn_distance(xyz1, xyz2, transpose=False):
     """Inference form: [dist1, idx1, dist2, idx2], no autograd node
     (torkit3d/ops/chamfer_distance.py:62-71)."""
-    xyz1, xyz2 = _batched(xyz1), _batched(xyz2)
+    clouds = [rows_of_points(with_batch_dim(c), transpose) for c in (xyz1, xyz2)]
     if transpose:
-        xyz1 = xyz1.transpose(1, 2).contiguous()
-        xyz2 = xyz2.transpose(1, 2).contiguous()
-    return _C.chamfer_distance_forward_cuda(xyz1, xyz2)
+        clouds = [c.contiguous() for c in clouds]
+    return _C.chamfer_distance_forward_cuda(*clouds)

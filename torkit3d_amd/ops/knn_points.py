@@ -2,46 +2,32 @@
 import torch
 
 from .. import _C
+from ._common import NoGradient, rows_of_points
 
 
-class KNNDistanceFunction(torch.autograd.Function):
-    """Not differentiable; backward returns None for every input
+class KNNDistanceFunction(NoGradient):
+    """(query_xyz, key_xyz, k, version) -> (distance, index), not differentiable
     (torkit3d/ops/knn_points.py:6-13)."""
 
     @staticmethod
-    def forward(ctx, query_xyz, key_xyz, k, version):
-        distance, index = _C.knn_distance_cuda(query_xyz, key_xyz, k, version)
-        ctx.mark_non_differentiable(distance, index)
-        return distance, index
-
-    @staticmethod
-    def backward(ctx, *grad_outputs):
-        return (None,) * 4
+    def run(query_xyz, key_xyz, k, version):
+        return _C.knn_distance_cuda(query_xyz, key_xyz, k, version)
 
 
 def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False, version=1):
-    """For each query point, its k nearest key points.
+    """The ``k`` key points nearest to every query point: (distance, index), each
+    [B, N1, k], in that order (the order of the reference's return statement,
+    torkit3d/ops/knn_points.py:45-51, not of its docstring).
 
-    Args:
-        query: [B, N1, 3] ([B, 3, N1] if ``transpose``).
-        key: [B, N2, 3] ([B, 3, N2] if ``transpose``).
-        k: neighbours per query, k <= N2.
-        sorted: sort each row by ascending distance.
-        sqrt_distance: return Euclidean rather than squared distances.
-        transpose: inputs are channel-first.
-        version: kernel selector of the reference (0 or 1); results are identical.
-
-    Returns:
-        (distance [B, N1, k], index [B, N1, k]) - distance first, as the reference's
-        code returns them (torkit3d/ops/knn_points.py:45-51).
+    Clouds are [B, N, 3], or [B, 3, N] with ``transpose``; ``k`` may not exceed the
+    number of keys. Distances are squared unless ``sqrt_distance``. Rows come in the
+    order the reference's top-k structure leaves them unless ``sorted`` (ascending
+    distance). ``version`` selects between the reference's two kernels (0 or 1); here
+    both values give the same result from the same kernel.
     """
-    if transpose:
-        query, key = query.transpose(1, 2), key.transpose(1, 2)
-    query, key = query.contiguous(), key.contiguous()
-    distance, index = KNNDistanceFunction.apply(query, key, k, version)
+    clouds = [rows_of_points(c, transpose).contiguous() for c in (query, key)]
+    distance, index = KNNDistanceFunction.apply(*clouds, k, version)
     if sorted:
-        distance, order = torch.sort(distance, dim=2)
-        index = torch.gather(index, 2, order)
-    if sqrt_distance:
-        distance = torch.sqrt(distance)
-    return distance, index
+        distance, order = distance.sort(dim=2)
+        index = index.gather(2, order)
+    return (distance.sqrt() if sqrt_distance else distance), index

@@ -2,25 +2,19 @@
 import torch
 
 from .. import _C, _fused
+from ._common import NoGradient
 
 
-class SampleFarthestPointsFunction(torch.autograd.Function):
+class SampleFarthestPointsFunction(NoGradient):
     """Not differentiable (torkit3d/ops/sample_farthest_points.py:6-14).
     ``channels_first`` (not in the reference) says the cloud is [B, 3, N]."""
 
     @staticmethod
-    def forward(ctx, points, num_samples, channels_first=False):
+    def run(points, num_samples, channels_first=False):
         if channels_first:
-            index, _ = _fused.sample_farthest_points_gather(points, num_samples, True,
-                                                            want_xyz=False)
-        else:
-            index = _C.sample_farthest_points_cuda(points, num_samples)
-        ctx.mark_non_differentiable(index)
-        return index
-
-    @staticmethod
-    def backward(ctx, *grad_outputs):
-        return (None,) * 3
+            return _fused.sample_farthest_points_gather(points, num_samples, True,
+                                                        want_xyz=False)[0]
+        return _C.sample_farthest_points_cuda(points, num_samples)
 
 
 def sample_farthest_points(points, num_samples, transpose=False):
