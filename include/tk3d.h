@@ -149,11 +149,15 @@ int tk3d_ball_query_bcn_f64(const double *query, const double *key, int64_t B,
  * index[b,0] = 0; index[b,i] = the point farthest from {index[b,0..i-1]}.
  * Exact ties for the maximum are resolved as the reference kernel resolves them
  * (its per-thread scan and shared-memory tree, block size = the power of two
- * >= N capped at 512). Requires 1 <= num_samples <= N.
+ * >= N capped at 512). Requires 1 <= num_samples <= N. A point with a NaN
+ * coordinate is never selected and an infinite one, once selected, is selected at
+ * every later step, as in the reference.
  *
- * Clouds too large for the register-resident kernel need a device workspace of
- * tk3d_sample_farthest_points_workspace_bytes(B, N, elem_size) bytes (0 when none
- * is needed; then `workspace` may be NULL). */
+ * Clouds too large for the register-resident kernel (more than 16384 points in fp32,
+ * 8192 in fp64) need a device workspace of
+ * tk3d_sample_farthest_points_workspace_bytes(B, N, elem_size) bytes, 8-byte aligned
+ * (0 when none is needed; then `workspace` may be NULL), and are sampled with one
+ * kernel launch per selection step, i.e. num_samples launches per call. */
 size_t tk3d_sample_farthest_points_workspace_bytes(int64_t B, int64_t N,
                                                    size_t elem_size);
 int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,

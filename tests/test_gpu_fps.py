@@ -149,3 +149,72 @@ def test_errors(cuda):
         _C.sample_farthest_points_cuda(pts, 9)
     with pytest.raises(RuntimeError):
         _C.sample_farthest_points_cuda(torch.zeros(2, 8, 4, device=cuda), 2)
+
+
+# ---- clouds beyond one workgroup's registers: one launch per step, many workgroups ----
+
+@pytest.mark.parametrize("b,n,k,dtype,transpose", [
+    (1, 20000, 300, torch.float32, False), (3, 65536 + 3, 120, torch.float32, True),
+    (2, 40000, 64, torch.float64, False), (5, 16385, 33, torch.float32, True),
+    (1, 8200, 500, torch.float64, True), (2, 17000, 17000 // 40, torch.float32, False)])
+def test_wide_path_shapes_layouts_and_types(cuda, b, n, k, dtype, transpose):
+    pts = torch.rand(b, n, 3, generator=gen(n + k), dtype=dtype)
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    dev = pts.transpose(1, 2).contiguous() if transpose else pts
+    np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
+
+
+@pytest.mark.parametrize("n", [17000, 70001])
+def test_wide_path_ties_follow_the_reference_tree_order(cuda, n):
+    pts = lattice_cloud(gen(n), 2, n, 3)
+    want = oracle.sample_farthest_points(pts.numpy(), 80)
+    np.testing.assert_array_equal(run(pts, 80, cuda), want)
+    assert not np.array_equal(want, oracle.sample_farthest_points(pts.numpy(), 80, "lowest"))
+
+
+def test_wide_path_duplicates_repeat_the_previous_choice(cuda):
+    # 5 distinct positions: from the sixth sample on nothing lies away from the chosen set
+    base = torch.rand(1, 5, 3, generator=gen(5))
+    pts = base[:, torch.randint(0, 5, (30000,), generator=gen(6))]
+    want = oracle.sample_farthest_points(pts.numpy(), 12)
+    np.testing.assert_array_equal(run(pts, 12, cuda), want)
+    assert len(set(want[0, 5:].tolist())) == 1
+
+
+def test_wide_path_with_coordinates(cuda):
+    from torkit3d_amd.ops.sample_farthest_points import sample_farthest_points_gather
+
+    pts = torch.rand(2, 3, 30000, generator=gen(7)).to(cuda)
+    idx, xyz = sample_farthest_points_gather(pts, 50, transpose=True)
+    want = oracle.sample_farthest_points(pts.transpose(1, 2).contiguous().cpu().numpy(), 50)
+    np.testing.assert_array_equal(idx.cpu().numpy(), want)
+    assert torch.equal(xyz, torch.gather(pts, 2, idx[:, None, :].expand(-1, 3, -1)))
+
+
+# ---- non-finite coordinates: the reference's "unset" minima take the first distance as
+# it comes, so a point with a NaN coordinate is never selected and the others are sampled
+# as if it were absent; a NaN in point 0 leaves nothing to select ----
+
+@pytest.mark.parametrize("n,dtype", [(300, torch.float32), (5000, torch.float32),
+                                      (5000, torch.float64), (30000, torch.float32)])
+def test_points_with_nan_are_never_selected(cuda, n, dtype):
+    pts = torch.rand(3, n, 3, generator=gen(n), dtype=dtype)
+    pts[0, 7, 1] = float("nan")
+    pts[0, n // 2] = float("nan")
+    pts[1, n - 1, 0] = float("nan")
+    pts[2, 0, 2] = float("nan")        # point 0 itself: every distance is NaN
+    k = 40
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    got = run(pts, k, cuda)
+    np.testing.assert_array_equal(got, want)
+    assert 7 not in got[0] and n // 2 not in got[0] and n - 1 not in got[1]
+    assert (got[2] == 0).all()
+
+
+def test_points_at_infinity(cuda):
+    pts = torch.rand(2, 2000, 3, generator=gen(9))
+    pts[0, 100, 0] = float("inf")
+    pts[1, 5] = float("-inf")
+    pts[1, 900, 2] = float("inf")
+    want = oracle.sample_farthest_points(pts.numpy(), 30)
+    np.testing.assert_array_equal(run(pts, 30, cuda), want)

@@ -1,7 +1,10 @@
 // Farthest point sampling for gfx950.
 //
-// One workgroup samples one cloud. The K-1 selection steps are strictly serial, so
-// the kernel is built for latency per step, not throughput:
+// Clouds that fit in one workgroup's registers (16384 points in fp32, 8192 in fp64) are
+// sampled by one workgroup each; larger ones by one launch of many workgroups per
+// selection step (fps_wide_step_kernel, further down). The K-1 selection steps are
+// strictly serial, so the one-workgroup kernels are built for latency per step, not
+// throughput:
 //   * every lane keeps P points and their running minimum distance in registers
 //     for the whole kernel - the loop touches no global memory except the one
 //     index it emits per step;
@@ -104,38 +107,22 @@ __device__ __forceinline__ int fps_point_of_position(int pos, const FpsLayout &L
     return t + cc * L.bs;
 }
 
-template <typename T, int P, int NT, bool SOA>
-__global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ points,
-                                                          int64_t *__restrict__ index,
-                                                          FpsLayout L)
+// One selection step per exchange between the waves, on points and minima held in
+// registers (lane `tid` holds positions tid * P .. tid * P + P - 1). fmin keeps a
+// minimum when a later distance is NaN, as the reference's '>' does. `md` arrives
+// holding the distances to point 0 (see fps_first_minimum).
+template <typename T, int P, int NT>
+__device__ __forceinline__ void fps_one_step_loop(int64_t *__restrict__ out, const FpsLayout &L,
+                                                  const T (&x)[P], const T (&y)[P],
+                                                  const T (&z)[P], T (&md)[P], T cx, T cy, T cz)
 {
     constexpr int NW = NT / TK_WAVE;
     __shared__ T s_val[2][NW], s_x[2][NW], s_y[2][NW], s_z[2][NW];
     __shared__ int s_j[2][NW];
-
     const int tid = threadIdx.x;
     const int lane = tid & (TK_WAVE - 1);
     const int wave = tid / TK_WAVE;
-    const T *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
-    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
-
-    T x[P], y[P], z[P], md[P];
-    const int npos = L.bs * L.c;
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-        const int pos = tid * P + p;
-        const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
-        const bool ok = j < L.n;
-        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : (T)0;
-        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : (T)0;
-        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : (T)0;
-        // Unused slots sit at -1: min() keeps them there and they never exceed 0.
-        md[p] = ok ? tk_inf<T>() : (T)-1;
-    }
-
     int sel_j = 0;
-    T cx = fps_coord<SOA>(pts, L.n, 0, 0), cy = fps_coord<SOA>(pts, L.n, 0, 1),
-      cz = fps_coord<SOA>(pts, L.n, 0, 2);
     if (tid == 0)
         out[0] = 0;
 
@@ -195,6 +182,62 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
         if (tid == 0)
             out[it] = (int64_t)sel_j;
     }
+}
+
+// The reference's minima start "unset" and take whatever the first step computes
+// (sample_farthest_points_kernel.cu:59-64), a NaN included, which then never compares
+// above anything. So a minimum starts at the distance to point 0, with -1 for a NaN and
+// for unused slots: min() keeps -1 and it never exceeds 0.
+template <typename T> __device__ __forceinline__ T fps_first_minimum(bool used, T d0)
+{
+    return (used && d0 == d0) ? d0 : (T)-1;
+}
+
+// The whole sampling of one cloud with the plain loop: loads the points into registers
+// and runs fps_one_step_loop. With `only_odd` it does so only for a cloud that holds a NaN
+// or an infinite coordinate, and returns at once for any other.
+//
+// The fp32 kernel below assumes finite coordinates (minima ordered as integers, a selected
+// point's minimum dropping to zero) and is followed by this one with `only_odd`, which
+// redoes the rare cloud it got wrong the way the reference treats it: a NaN point is never
+// selected, an infinite one, once selected, is selected at every later step. The check
+// lives here rather than in that kernel because anything added to it, even a test in
+// its prologue, moved its loop's code and cost 4-7 % at 32 points per lane; the extra
+// launch costs a few microseconds.
+template <typename T, int P, int NT, bool SOA>
+__global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ points,
+                                                          int64_t *__restrict__ index,
+                                                          FpsLayout L, int only_odd)
+{
+    const T *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
+    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
+    const int tid = threadIdx.x;
+    if (only_odd) {
+        // v - v is zero exactly for finite v; the 3n values are scanned in memory order
+        bool odd = false;
+#pragma unroll 8
+        for (int i = tid; i < L.n * 3; i += NT) {
+            const T v = pts[i];
+            odd |= !(v - v == (T)0);
+        }
+        if (!__syncthreads_or(odd ? 1 : 0))  // uniform over the workgroup
+            return;
+    }
+    T x[P], y[P], z[P], md[P];
+    const int npos = L.bs * L.c;
+    const T cx = fps_coord<SOA>(pts, L.n, 0, 0), cy = fps_coord<SOA>(pts, L.n, 0, 1),
+            cz = fps_coord<SOA>(pts, L.n, 0, 2);
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int pos = tid * P + p;
+        const int j = pos < npos ? fps_point_of_position(pos, L) : L.n;
+        const bool ok = j < L.n;
+        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : (T)0;
+        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : (T)0;
+        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : (T)0;
+        md[p] = fps_first_minimum<T>(ok, tk_dist2<T>(x[p], y[p], z[p], cx, cy, cz));
+    }
+    fps_one_step_loop<T, P, NT>(out, L, x, y, z, md, cx, cy, cz);
 }
 
 // ---- fp32 fast path ------------------------------------------------------------
@@ -452,75 +495,164 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
     }
 }
 
-// Clouds that do not fit in registers: minimum distances live in a global
-// workspace, coordinates are re-read every step (they stay in L2). Same selection
-// rule; positions are visited in priority order so the tie rule is unchanged.
-template <typename T, int NT, bool SOA>
-__global__ __launch_bounds__(NT) void fps_streaming_kernel(const T *__restrict__ points,
-                                                           int64_t *__restrict__ index,
-                                                           T *__restrict__ min_dist,
-                                                           FpsLayout L)
+// Clouds that do not fit in one workgroup's registers: every selection step is one
+// launch of many workgroups per cloud. Step s first works out the point chosen by step
+// s - 1 from the candidates that step's workgroups left in the workspace (every workgroup
+// redoes this small reduction itself), then updates the running minima of its own slice
+// of the cloud for that centre, streaming coordinates and minima through coalesced
+// loads, and leaves its own candidate for step s + 1. The kernel boundary is the
+// cross-workgroup barrier; nothing waits inside a kernel.
+//
+// Points are visited in index order; the reference's tie order is restored by comparing
+// positions (see the top of the file) whenever two minima are equal.
+template <typename T> struct FpsWideArgs {
+    const T *points;     // [B, n, 3] or [B, 3, n]
+    int64_t *index;      // [B, k]
+    T *min_dist;         // [B, n]
+    T *cand_val;         // [2, B, groups]: largest running minimum of a workgroup's slice
+    int *cand_pos;       // [2, B, groups]: its position
+    int *chosen;         // [2, B]: the point the previous step used as centre
+    int groups;          // workgroups per cloud
+    int slice;           // points per workgroup
+    int batch;           // B
+};
+
+// Position of point j in the reference's tie order: its thread's rank among the
+// bit-reversed thread ids times the points per thread, plus its turn within the thread.
+__device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
+{
+    const int t = j & (L.bs - 1);
+    const int r = (int)(__builtin_bitreverse32((unsigned)t) >> (32 - L.log2_bs));
+    return r * L.c + (j >> L.log2_bs);
+}
+
+// (value, position) pairs ordered by larger value, then lower position.
+template <typename T>
+__device__ __forceinline__ void fps_keep_better(T &val, int &pos, T oval, int opos)
+{
+    const bool take = oval > val || (oval == val && opos < pos);
+    val = take ? oval : val;
+    pos = take ? opos : pos;
+}
+
+template <typename T, int NT>
+__device__ __forceinline__ void fps_block_best(T &val, int &pos, T *s_val, int *s_pos)
 {
     constexpr int NW = NT / TK_WAVE;
-    __shared__ T s_val[2][NW];
-    __shared__ int s_pos[2][NW];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (TK_WAVE - 1);
-    const int wave = tid / TK_WAVE;
-    const T *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
-    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
-    T *__restrict__ md = min_dist + (int64_t)blockIdx.x * L.bs * L.c;
-
-    const int npos = L.bs * L.c;
-    // A thread owns a contiguous run of positions so that thread order == position order.
-    const int per = (npos + NT - 1) / NT;
-    const int p0 = tid * per;
-    const int p1 = (p0 + per < npos) ? p0 + per : npos;
-    for (int pos = p0; pos < p1; ++pos)
-        md[pos] = fps_point_of_position(pos, L) < L.n ? tk_inf<T>() : (T)-1;
-
-    int sel_j = 0;
-    if (tid == 0)
-        out[0] = 0;
-    for (int it = 1; it < L.k; ++it) {
-        const T cx = fps_coord<SOA>(pts, L.n, sel_j, 0), cy = fps_coord<SOA>(pts, L.n, sel_j, 1),
-                cz = fps_coord<SOA>(pts, L.n, sel_j, 2);
-        T best = (T)0;
-        int bpos = 0;
-        for (int pos = p0; pos < p1; ++pos) {
-            const T m = md[pos];
-            if (m < (T)0)
-                continue;
-            const int j = fps_point_of_position(pos, L);
-            const T d = tk_dist2<T>(fps_coord<SOA>(pts, L.n, j, 0), fps_coord<SOA>(pts, L.n, j, 1),
-                                    fps_coord<SOA>(pts, L.n, j, 2), cx, cy, cz);
-            const T nm = tk_min<T>(m, d);
-            md[pos] = nm;
-            if (nm > best) {
-                best = nm;
-                bpos = pos;
-            }
-        }
-        const T wmax = wave_max<T>(best);
-        const int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
-        const int wpos = read_lane(bpos, wl);
-        const int buf = it & 1;
-        if (lane == 0) {
-            s_val[buf][wave] = wmax;
-            s_pos[buf][wave] = wpos;
-        }
-        __syncthreads();
-        const bool has = lane < NW;
-        const T cv = has ? s_val[buf][has ? lane : 0] : (T)-1;
-        const T gmax = wave_max<T>(cv);
-        if (gmax > (T)0) {
-            const int gl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(cv == gmax));
-            sel_j = fps_point_of_position(s_pos[buf][gl], L);
-        }
-        if (tid == 0)
-            out[it] = (int64_t)sel_j;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const T oval = __shfl_xor(val, o);
+        const int opos = __shfl_xor(pos, o);
+        fps_keep_better<T>(val, pos, oval, opos);
     }
+    __syncthreads();  // the arrays may still be read from an earlier call
+    if ((threadIdx.x & (TK_WAVE - 1)) == 0) {
+        s_val[threadIdx.x / TK_WAVE] = val;
+        s_pos[threadIdx.x / TK_WAVE] = pos;
+    }
+    __syncthreads();
+    val = s_val[0];
+    pos = s_pos[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w)
+        fps_keep_better<T>(val, pos, s_val[w], s_pos[w]);
+}
+
+template <typename T, int NT, bool SOA>
+__global__ __launch_bounds__(NT) void fps_wide_step_kernel(FpsWideArgs<T> a, FpsLayout L,
+                                                           int step)
+{
+    __shared__ T s_val[NT / TK_WAVE];
+    __shared__ int s_pos[NT / TK_WAVE];
+    const int tid = threadIdx.x;
+    const int g = blockIdx.x, b = blockIdx.y;
+    const T *__restrict__ pts = a.points + (int64_t)b * L.n * 3;
+    constexpr int NO_POS = 0x7fffffff;
+
+    // ---- the centre of this step: what step - 1 selected ----
+    int centre = 0;
+    if (step > 1) {
+        const int from = (step - 1) & 1;
+        const T *cv = a.cand_val + ((int64_t)from * a.batch + b) * a.groups;
+        const int *cp = a.cand_pos + ((int64_t)from * a.batch + b) * a.groups;
+        T val = (T)0;
+        int pos = NO_POS;
+        for (int i = tid; i < a.groups; i += NT)
+            fps_keep_better<T>(val, pos, cv[i], cp[i]);
+        fps_block_best<T, NT>(val, pos, s_val, s_pos);
+        // Nothing above zero: no point lies away from the chosen set and the previous
+        // choice is emitted again, as the reference does.
+        centre = val > (T)0 ? fps_point_of_position(pos, L) : a.chosen[(int64_t)from * a.batch + b];
+    }
+    if (g == 0 && tid == 0) {
+        a.index[(int64_t)b * L.k + (step - 1)] = (int64_t)centre;
+        a.chosen[(int64_t)(step & 1) * a.batch + b] = centre;
+    }
+    if (step >= L.k)  // the last launch only records the last choice
+        return;
+
+    // ---- update this workgroup's slice, keep its best candidate ----
+    const T cx = fps_coord<SOA>(pts, L.n, centre, 0), cy = fps_coord<SOA>(pts, L.n, centre, 1),
+            cz = fps_coord<SOA>(pts, L.n, centre, 2);
+    T *__restrict__ md = a.min_dist + (int64_t)b * L.n;
+    const int j0 = g * a.slice;
+    const int j1 = (j0 + a.slice < L.n) ? j0 + a.slice : L.n;
+    T best = (T)0;
+    int bpos = NO_POS;
+    for (int j = j0 + tid; j < j1; j += NT) {
+        T x, y, z;
+        if (SOA) {
+            x = pts[j], y = pts[(int64_t)L.n + j], z = pts[2 * (int64_t)L.n + j];
+        } else {
+            const TkPoint3<T> p = tk_load3<T>(pts + (int64_t)j * 3);
+            x = p.x, y = p.y, z = p.z;
+        }
+        const T d = tk_dist2<T>(x, y, z, cx, cy, cz);
+        // The first step assigns whatever it computes (sample_farthest_points_kernel.cu:59-64
+        // starts from "unset"); a NaN there never compares above anything, which -1 mimics.
+        const T nm = step == 1 ? (d != d ? (T)-1 : d) : tk_min<T>(md[j], d);
+        md[j] = nm;
+        if (nm > (T)0 && nm >= best)
+            fps_keep_better<T>(best, bpos, nm, fps_position_of_point(j, L));
+    }
+    fps_block_best<T, NT>(best, bpos, s_val, s_pos);
+    if (tid == 0) {
+        const int64_t o = ((int64_t)(step & 1) * a.batch + b) * a.groups + g;
+        a.cand_val[o] = best;
+        a.cand_pos[o] = bpos;
+    }
+}
+
+// Workgroups per cloud and points per workgroup of the wide kernel.
+inline void fps_wide_shape(int64_t B, int64_t N, int &groups, int &slice)
+{
+    constexpr int64_t MIN_SLICE = 2048, MAX_GROUPS = 1024;
+    int64_t want = (2048 + B - 1) / B;  // about 2048 workgroups in flight
+    int64_t g = (N + MIN_SLICE - 1) / MIN_SLICE;
+    if (g > want)
+        g = want;
+    if (g > MAX_GROUPS)
+        g = MAX_GROUPS;
+    if (g < 1)
+        g = 1;
+    slice = (int)((N + g - 1) / g);
+    groups = (int)((N + slice - 1) / slice);
+}
+
+template <typename T> struct FpsWideLayout {
+    size_t min_dist, cand_val, cand_pos, chosen, total;
+};
+
+template <typename T> FpsWideLayout<T> fps_wide_layout(int64_t B, int64_t N, int groups)
+{
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    FpsWideLayout<T> w;
+    w.min_dist = 0;
+    w.cand_val = up((size_t)B * (size_t)N * sizeof(T));
+    w.cand_pos = w.cand_val + up((size_t)2 * B * groups * sizeof(T));
+    w.chosen = w.cand_pos + up((size_t)2 * B * groups * sizeof(int));
+    w.total = w.chosen + up((size_t)2 * B * sizeof(int));
+    return w;
 }
 
 FpsLayout fps_layout(int64_t n, int64_t k)
@@ -556,10 +688,10 @@ void fps_launch(const T *points, bool soa, int64_t B, int64_t *index, const FpsL
 {
     if (soa)
         hipLaunchKernelGGL((fps_register_kernel<T, P, NT, true>), dim3((unsigned)B), dim3(NT), 0,
-                           s, points, index, L);
+                           s, points, index, L, 0);
     else
         hipLaunchKernelGGL((fps_register_kernel<T, P, NT, false>), dim3((unsigned)B), dim3(NT),
-                           0, s, points, index, L);
+                           0, s, points, index, L, 0);
 }
 
 template <int P, int NT>
@@ -567,12 +699,17 @@ void fps_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
                     const FpsLayout &L, hipStream_t s)
 {
     constexpr int MAXM = 6;  // 4 -> 6 gains 1-4 %, 8 nothing
-    if (soa)
+    if (soa) {
         hipLaunchKernelGGL((fps_multistep_kernel_f32<P, NT, true, MAXM>), dim3((unsigned)B),
                            dim3(NT), 0, s, points, index, L);
-    else
+        hipLaunchKernelGGL((fps_register_kernel<float, P, NT, true>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L, 1);
+    } else {
         hipLaunchKernelGGL((fps_multistep_kernel_f32<P, NT, false, MAXM>), dim3((unsigned)B),
                            dim3(NT), 0, s, points, index, L);
+        hipLaunchKernelGGL((fps_register_kernel<float, P, NT, false>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L, 1);
+    }
 }
 
 // fp32: (points per lane, lanes) by cloud size, from timing every shape on an
@@ -681,15 +818,36 @@ int fps(const T *points, bool soa, int64_t B, int64_t N, int64_t K, int64_t *ind
             fps_launch<T, 16, 1024>(points, soa, B, index, L, s);
         return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
     }
-    const size_t need = (size_t)B * (size_t)npos * sizeof(T);
-    if (!workspace || workspace_bytes < need)
+    // Larger clouds: one launch per selection step, many workgroups per cloud.
+    int groups, slice;
+    fps_wide_shape(B, N, groups, slice);
+    const FpsWideLayout<T> w = fps_wide_layout<T>(B, N, groups);
+    if (!workspace || workspace_bytes < w.total || ((uintptr_t)workspace & 7) != 0)
         return TK3D_ERR_WORKSPACE;
-    if (soa)
-        hipLaunchKernelGGL((fps_streaming_kernel<T, 1024, true>), dim3((unsigned)B), dim3(1024),
-                           0, s, points, index, (T *)workspace, L);
-    else
-        hipLaunchKernelGGL((fps_streaming_kernel<T, 1024, false>), dim3((unsigned)B), dim3(1024),
-                           0, s, points, index, (T *)workspace, L);
+    if (B > 65535)
+        return TK3D_ERR_UNSUPPORTED;
+    char *base = (char *)workspace;
+    FpsWideArgs<T> a;
+    a.points = points;
+    a.index = index;
+    a.min_dist = (T *)(base + w.min_dist);
+    a.cand_val = (T *)(base + w.cand_val);
+    a.cand_pos = (int *)(base + w.cand_pos);
+    a.chosen = (int *)(base + w.chosen);
+    a.groups = groups;
+    a.slice = slice;
+    a.batch = (int)B;
+    const dim3 grid((unsigned)groups, (unsigned)B);
+    for (int64_t step = 1; step <= K; ++step) {
+        // The last launch has nothing to update: one workgroup per cloud records the choice.
+        const dim3 gr = step == K ? dim3(1u, (unsigned)B) : grid;
+        if (soa)
+            hipLaunchKernelGGL((fps_wide_step_kernel<T, 256, true>), gr, dim3(256), 0, s, a, L,
+                               (int)step);
+        else
+            hipLaunchKernelGGL((fps_wide_step_kernel<T, 256, false>), gr, dim3(256), 0, s, a, L,
+                               (int)step);
+    }
     return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
 }
 
@@ -705,7 +863,10 @@ size_t tk3d_sample_farthest_points_workspace_bytes(int64_t B, int64_t N, size_t 
     const int64_t npos = (int64_t)L.bs * L.c;
     if (npos <= fps_register_capacity(elem_size))
         return 0;
-    return (size_t)B * (size_t)npos * elem_size;
+    int groups, slice;
+    fps_wide_shape(B, N, groups, slice);
+    return elem_size == 4 ? fps_wide_layout<float>(B, N, groups).total
+                          : fps_wide_layout<double>(B, N, groups).total;
 }
 
 int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,
