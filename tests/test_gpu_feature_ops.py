@@ -227,3 +227,31 @@ def test_scatter_non_finite_gradients_follow_float_arithmetic(cuda):
     finite = np.isfinite(want)
     assert np.isnan(want).any() and np.isinf(want).any()
     np.testing.assert_allclose(got[finite], want[finite], rtol=RTOL, atol=2e-5)
+
+
+@pytest.mark.parametrize("n1", [16385, 40000, 262144, 300000])
+def test_backward_into_rows_longer_than_lds(cuda, n1):
+    """Destination rows beyond 16384 points are accumulated in windows (up to 16 of
+    them) or, longer still, with global atomics; integer-valued gradients and weights of
+    k/4 make every sum exact, so both must equal torch's scatter_add bit for bit."""
+    from torkit3d_amd import _C
+
+    g = torch.Generator().manual_seed(n1)
+    b, c, n2, k = 2, 5, 3000, 7
+    index = torch.randint(0, n1, (b, n2, k), generator=g).to(cuda)
+    index[0, :50] = n1 - 1                      # the last destination, many times
+    index[1, :50, 0] = 16384                    # first point of the second window
+    grad = torch.randint(-3, 4, (b, c, n2, k), generator=g).float().to(cuda)
+    got = _C.group_points_backward_cuda(grad, index, n1)
+    want = torch.zeros(b, c, n1, device=cuda).scatter_add_(
+        2, index.view(b, 1, -1).expand(b, c, -1), grad.view(b, c, -1))
+    assert torch.equal(got, want)
+
+    index3 = torch.randint(0, n1, (b, n2, 3), generator=g).to(cuda)
+    weight = (torch.randint(0, 5, (b, n2, 3), generator=g).float() / 4).to(cuda)
+    grad3 = torch.randint(-2, 3, (b, c, n2), generator=g).float().to(cuda)
+    got = _C.interpolate_backward_cuda(grad3, index3, weight, n1)
+    want = torch.zeros(b, c, n1, device=cuda)
+    for i in range(3):
+        want.scatter_add_(2, index3[:, None, :, i].expand(b, c, n2), grad3 * weight[:, None, :, i])
+    assert torch.equal(got, want)

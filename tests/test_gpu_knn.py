@@ -62,7 +62,9 @@ def test_interpolation_config_fp32(cuda, k):
                                         (1, 1000, 1025, 33), (2, 300, 1000, 65),
                                         (2, 200, 700, 128), (1, 100, 400, 129),
                                         (4, 1000, 4096, 32), (1, 70, 70000, 20),
-                                        (1, 40, 66000, 7), (40, 4096, 300, 6)])
+                                        (1, 40, 66000, 7), (40, 4096, 300, 6),
+                                        (2, 150, 1000, 200), (1, 70, 256, 256),
+                                        (1, 100, 3000, 257), (1, 64, 66000, 130)])
 def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
     g = gen(k)
     q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
@@ -73,7 +75,7 @@ def test_all_k_variants_and_versions(cuda, b, n1, n2, k):
 def test_lattice_ties_follow_mink_eviction_order(cuda):
     g = gen(9)
     q, key = lattice_cloud(g, 2, 400, 4), lattice_cloud(g, 2, 1500, 4)
-    for k in (3, 6, 16, 33, 64, 100):
+    for k in (3, 6, 16, 33, 64, 100, 180):
         check_raw(q, key, k, cuda)
 
 

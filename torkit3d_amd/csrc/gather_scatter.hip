@@ -221,15 +221,17 @@ __global__ __launch_bounds__(GS_BLOCK) void fill_zero_kernel(T *__restrict__ p, 
 }
 
 // Streams the points [ps, pe) of one batch for `nc` channels starting at c0 and hands
-// every contribution to `sink(ctx, c, dst, value, weight)`, where `ctx = prep(c)` is
-// evaluated once per channel and lane iteration. A lane takes V points 64 apart,
+// every contribution whose destination lies in [d0, d0 + nr) to
+// `sink(ctx, c, dst - d0, value, weight)`, where `ctx = prep(c)` is evaluated once per
+// channel and lane iteration. A lane takes V points 64 apart,
 // and the channel loop is unrolled to keep several loads in flight.
 template <typename T, int KK, bool HAS_W, int V, int NT, typename Prep, typename Sink>
 __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
                                                const int64_t *__restrict__ idx,
                                                const T *__restrict__ w, int b, int wc_total,
-                                               int c0, int nc, int n1, int64_t np, int64_t ps,
-                                               int64_t pe, int vec_ok, Prep prep, Sink sink)
+                                               int c0, int nc, int d0, int nr, int64_t np,
+                                               int64_t ps, int64_t pe, int vec_ok, Prep prep,
+                                               Sink sink)
 {
     (void)vec_ok;
     // A wave covers 64*V consecutive points, lane l the points l, l+64, ...: every load
@@ -252,7 +254,7 @@ __device__ __forceinline__ void scatter_stream(const T *__restrict__ gout,
                     if (HAS_W)
                         ww = w[((int64_t)b * np + p) * KK + i];
                 }
-                dst[v][i] = (j >= 0 && j < n1) ? (int)j : -1;
+                dst[v][i] = (j >= d0 && j < (int64_t)d0 + nr) ? (int)(j - d0) : -1;
                 wt[v][i] = ww;
             }
         }
@@ -294,7 +296,8 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
         rows[i] = (T)0;
     __syncthreads();
     scatter_stream<T, KK, HAS_W, V, NT>(
-        gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        gout, idx, w, b, wc_total, c0 + wc_off, nc, 0, n1, np, ps, pe, vec_ok,
+        [](int) { return 0; },
         [&](int, int c, int dst, T g, T ww) { atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g); });
     __syncthreads();
 
@@ -349,10 +352,10 @@ template <int KK, bool HAS_W, int V, int NT, int CGMAX>
 __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     const float *__restrict__ gout, const int64_t *__restrict__ idx,
     const float *__restrict__ w, float *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg,
-    int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count)
+    int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count, int groups, int window)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);  // [cg][n1]
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);  // [cg][nr]
     __shared__ unsigned s_maxg[CGMAX];  // bit patterns of non-negative floats order as integers
     __shared__ unsigned s_maxw;
     __shared__ int s_kexp[CGMAX];
@@ -360,14 +363,19 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     __shared__ float s_bound[CGMAX];
     __shared__ int s_finite, s_exceeded;
     const int b = blockIdx.z;
-    const int c0 = blockIdx.y * cg;
+    // blockIdx.y = destination window * groups + channel group; a workgroup accumulates
+    // the destinations [d0, d0 + nr) of its channels (the whole row when it fits in LDS)
+    const int win = blockIdx.y / groups;
+    const int c0 = (blockIdx.y - win * groups) * cg;
     const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
+    const int d0 = win * window;
+    const int nr = (d0 + window < n1) ? window : n1 - d0;
     const int64_t ps = (int64_t)blockIdx.x * seg_len;
     const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
     for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
         __syncthreads();
-        for (int i = threadIdx.x; i < nc * n1; i += NT)
+        for (int i = threadIdx.x; i < nc * nr; i += NT)
             acc[i] = 0ull;
         if (threadIdx.x < CGMAX)
             s_maxg[threadIdx.x] = 0u;
@@ -467,7 +475,7 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         };
         bool exceeded = false;
         scatter_stream<float, KK, HAS_W, V, NT>(
-            gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok,
+            gout, idx, w, b, wc_total, c0 + wc_off, nc, d0, nr, np, ps, pe, vec_ok,
             [&](int c) {
                 RowScale r;
                 r.scale = s_scale[c];
@@ -480,21 +488,22 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                 const double d = __builtin_fma((double)term, r.scale, MAGIC);
                 const unsigned long long q = __builtin_bit_cast(unsigned long long, d) -
                                              __builtin_bit_cast(unsigned long long, MAGIC);
-                atomicAdd(&acc[c * n1 + dst], q);
+                atomicAdd(&acc[c * nr + dst], q);
             });
         if (exceeded)
             s_exceeded = 1;
         __syncthreads();
         if (!s_exceeded) {
-            float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
-            for (int i = threadIdx.x; i < nc * n1; i += NT) {
-                const float v =
-                    (float)__builtin_ldexp((double)(long long)acc[i], -s_kexp[i / n1]);
+            float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1 + d0;
+            for (int i = threadIdx.x; i < nc * nr; i += NT) {
+                const int c = i / nr;
+                const float v = (float)__builtin_ldexp((double)(long long)acc[i], -s_kexp[c]);
+                float *out = dstrows + (int64_t)c * n1 + (i - c * nr);
                 if (merge_with_atomics) {
                     if (v != 0.0f)
-                        unsafeAtomicAdd(&dstrows[i], v);
+                        unsafeAtomicAdd(out, v);
                 } else {
-                    dstrows[i] = v;
+                    *out = v;
                 }
             }
             return;
@@ -504,23 +513,26 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     // ---- non-finite input: floating-point accumulation in the same LDS ----
     float *rows = reinterpret_cast<float *>(smem_raw);
     __syncthreads();
-    for (int i = threadIdx.x; i < nc * n1; i += NT)
+    for (int i = threadIdx.x; i < nc * nr; i += NT)
         rows[i] = 0.0f;
     __syncthreads();
     scatter_stream<float, KK, HAS_W, V, NT>(
-        gout, idx, w, b, wc_total, c0 + wc_off, nc, n1, np, ps, pe, vec_ok, [](int) { return 0; },
+        gout, idx, w, b, wc_total, c0 + wc_off, nc, d0, nr, np, ps, pe, vec_ok,
+        [](int) { return 0; },
         [&](int, int c, int dst, float g, float ww) {
-            atomicAdd(&rows[c * n1 + dst], HAS_W ? g * ww : g);
+            atomicAdd(&rows[c * nr + dst], HAS_W ? g * ww : g);
         });
     __syncthreads();
-    float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1;
-    for (int i = threadIdx.x; i < nc * n1; i += NT) {
+    float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1 + d0;
+    for (int i = threadIdx.x; i < nc * nr; i += NT) {
+        const int c = i / nr;
         const float v = rows[i];
+        float *out = dstrows + (int64_t)c * n1 + (i - c * nr);
         if (merge_with_atomics) {
             if (v != 0.0f)
-                unsafeAtomicAdd(&dstrows[i], v);
+                unsafeAtomicAdd(out, v);
         } else {
-            dstrows[i] = v;
+            *out = v;
         }
     }
 }
@@ -657,18 +669,25 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
         // fp32: 64-bit fixed-point accumulators, up to 128 KiB of LDS per workgroup.
         constexpr int64_t FIXED_LDS = 128 * 1024;
         constexpr int NT = 1024, V = 4, CGMAX = 8;
-        const int64_t acc_row = N1 * 8;
-        if (acc_row <= FIXED_LDS) {
+        // Rows longer than the LDS holds are accumulated in windows of destinations, each
+        // by workgroups of its own that stream the whole input and keep what lands in
+        // their window. Up to 16 windows this beats global atomics (the input is read once
+        // per window); longer rows take the global path below.
+        constexpr int64_t MAX_WINDOW = FIXED_LDS / 8, MAX_WINDOWS = 16;
+        const int64_t windows = (N1 + MAX_WINDOW - 1) / MAX_WINDOW;
+        const int64_t window = ((N1 + windows - 1) / windows + 3) / 4 * 4;
+        const int64_t acc_row = window * 8;
+        if (windows <= MAX_WINDOWS) {
             const int vec_ok = (((uintptr_t)gout & 15) == 0) && ((NP * 4) % 16 == 0);
             int cg = CGMAX;
             while (cg > 1 && (cg * acc_row > FIXED_LDS || cg > C))
                 cg /= 2;
             // Prefer more workgroups over wider channel groups until every CU has one.
-            while (cg > 2 && B * ((C + cg - 1) / cg) < 256)
+            while (cg > 2 && B * windows * ((C + cg - 1) / cg) < 256)
                 cg /= 2;
             const int64_t gy = (C + cg - 1) / cg;
             int64_t nseg = 1;
-            const int64_t groups = B * gy;
+            const int64_t groups = B * gy * windows;
             if (groups < 128) {
                 nseg = (256 + groups - 1) / groups;
                 const int64_t max_seg = (NP + 4 * NT * V - 1) / (4 * NT * V);
@@ -680,7 +699,7 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
             int64_t seg_len = (NP + nseg - 1) / nseg;
             seg_len = (seg_len + 15) / 16 * 16;
             nseg = (NP + seg_len - 1) / seg_len;
-            if (gy > 65535 || nseg > TK_MAX_I32)
+            if (gy * windows > 65535 || nseg > TK_MAX_I32)
                 return TK3D_ERR_UNSUPPORTED;
             int log2_count = 1;
             while (((int64_t)1 << log2_count) < seg_len * KK + 1)
@@ -692,9 +711,10 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
             if (nseg > 1)
                 hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
                                    dim3(GS_BLOCK), 0, s, gin, out_elems);
-            hipLaunchKernelGGL(kernel, dim3((unsigned)nseg, (unsigned)gy, (unsigned)B), dim3(NT),
-                               (size_t)(cg * acc_row), s, gout, idx, w, gin, (int)C, (int)wc_total, (int)wc_off, (int)N1, NP,
-                               cg, seg_len, nseg > 1 ? 1 : 0, vec_ok, log2_count);
+            hipLaunchKernelGGL(kernel, dim3((unsigned)nseg, (unsigned)(gy * windows), (unsigned)B),
+                               dim3(NT), (size_t)(cg * acc_row), s, gout, idx, w, gin, (int)C,
+                               (int)wc_total, (int)wc_off, (int)N1, NP, cg, seg_len,
+                               nseg > 1 ? 1 : 0, vec_ok, log2_count, (int)gy, (int)window);
             return tk_launch_status();
         }
     }

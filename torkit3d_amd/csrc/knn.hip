@@ -410,8 +410,10 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     constexpr int CHUNK = 32;
     constexpr int NT = 64;
     constexpr int HALF = KMAX / 2;  // nodes HALF .. KMAX-1 are the parents of the leaves
-    constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : KMAX == 64 ? 6 : 7;
-    static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 128");
+    constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : KMAX == 64 ? 6
+                           : KMAX == 128 ? 7 : 8;
+    static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 256");
+    static_assert(KMAX <= 256, "slot numbers are kept in one byte");
     extern __shared__ __align__(16) unsigned char knn_tree_lds[];
     const int lane = threadIdx.x;
     float *const leaf = reinterpret_cast<float *>(knn_tree_lds) + lane;
@@ -730,6 +732,10 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
             return knn_tree_launch<64>(query, key, distance, index, B, n1, n2, kk, s);
         else if (k <= 128)
             return knn_tree_launch<128>(query, key, distance, index, B, n1, n2, kk, s);
+        else if (k <= 256 && n2 <= 65536)
+            // 136 KiB of LDS per wave with 16-bit key indices: one wave per CU, still some
+            // twenty times faster than keeping the slots in global memory
+            return knn_tree_launch_as<256, true>(query, key, distance, index, B, n1, n2, kk, s);
         else
             hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)),
                                dim3(KNN_BLOCK), 0, s, query, key, distance, index, (int)bpb,
