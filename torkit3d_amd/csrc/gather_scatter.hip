@@ -494,16 +494,18 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             s_exceeded = 1;
         __syncthreads();
         if (!s_exceeded) {
-            float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1 + d0;
-            for (int i = threadIdx.x; i < nc * nr; i += NT) {
-                const int c = i / nr;
-                const float v = (float)__builtin_ldexp((double)(long long)acc[i], -s_kexp[c]);
-                float *out = dstrows + (int64_t)c * n1 + (i - c * nr);
-                if (merge_with_atomics) {
-                    if (v != 0.0f)
-                        unsafeAtomicAdd(out, v);
-                } else {
-                    *out = v;
+            for (int c = 0; c < nc; ++c) {
+                float *__restrict__ dstrow = gin + ((int64_t)b * c_total + c0 + c) * n1 + d0;
+                const unsigned long long *__restrict__ row = acc + c * nr;
+                const int kexp = s_kexp[c];
+                for (int i = threadIdx.x; i < nr; i += NT) {
+                    const float v = (float)__builtin_ldexp((double)(long long)row[i], -kexp);
+                    if (merge_with_atomics) {
+                        if (v != 0.0f)
+                            unsafeAtomicAdd(&dstrow[i], v);
+                    } else {
+                        dstrow[i] = v;
+                    }
                 }
             }
             return;
@@ -523,16 +525,16 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             atomicAdd(&rows[c * nr + dst], HAS_W ? g * ww : g);
         });
     __syncthreads();
-    float *__restrict__ dstrows = gin + ((int64_t)b * c_total + c0) * n1 + d0;
-    for (int i = threadIdx.x; i < nc * nr; i += NT) {
-        const int c = i / nr;
-        const float v = rows[i];
-        float *out = dstrows + (int64_t)c * n1 + (i - c * nr);
-        if (merge_with_atomics) {
-            if (v != 0.0f)
-                unsafeAtomicAdd(out, v);
-        } else {
-            *out = v;
+    for (int c = 0; c < nc; ++c) {
+        float *__restrict__ dstrow = gin + ((int64_t)b * c_total + c0 + c) * n1 + d0;
+        for (int i = threadIdx.x; i < nr; i += NT) {
+            const float v = rows[c * nr + i];
+            if (merge_with_atomics) {
+                if (v != 0.0f)
+                    unsafeAtomicAdd(&dstrow[i], v);
+            } else {
+                dstrow[i] = v;
+            }
         }
     }
 }
