@@ -313,6 +313,11 @@ def secondary_metrics(dev, steps, warmup, cpu):
     out["sa_chain_B8_16384_4096_1024_256_ms"] = gpu_time_ms(run_chain, max(3, steps // 10), 2)
     out["fps_B8_N16384_K4096_ms"] = gpu_time_ms(
         lambda: _C.sample_farthest_points_cuda(chain[0][0], 4096), max(3, steps // 10), 1)
+    # One large cloud: sampled by many workgroups, one launch per selection step.
+    big = torch.rand(1, 262144, 3, generator=g).to(dev)
+    out["fps_B1_N262144_K512_ms"] = gpu_time_ms(
+        lambda: _C.sample_farthest_points_cuda(big, 512), 3, 1)
+    del big
     # Fused callers against the composition of ops the reference's layers run.
     from torkit3d_amd import _fused
     from torkit3d_amd.ops.interpolate_feature import three_nn_weights as weights_of
