@@ -575,6 +575,288 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     }
 }
 
+// The tree kernel for launches with few queries. One wave per 64 queries leaves most of
+// the chip idle when B * N1 is small, and the keys cannot simply be divided among waves:
+// the slot order MinK leaves behind depends on every insertion in key order. But a key
+// that the k best of a *slice* of the keys would not take is not taken by the whole
+// sequence either (the slice's k-th best so far is no better than the whole sequence's).
+// So S waves serve the same 64 queries: wave 0 runs MinK on the first slice as usual;
+// every other wave runs a MinK of its own on its slice, starting from k empty slots, and
+// logs the keys it inserts (a superset of what the whole sequence would insert from that
+// slice); then wave 0 replays the logs slice by slice, in key order, against its own
+// structure with the usual strict test. A log that overflows makes wave 0 sweep that
+// slice in full instead. The result is MinK's, slot for slot.
+template <int KMAX, bool IDX16, int S, int CAP> struct KnnSplitLayout {
+    using Tree = KnnTreeLayout<KMAX, IDX16>;
+    using Idx = typename Tree::Idx;
+    static constexpr int LOG_BYTES = (int)sizeof(Idx) * CAP * 64;
+    static constexpr int WAVE_BYTES = Tree::BYTES + LOG_BYTES;
+    static constexpr int BYTES = S * WAVE_BYTES;
+};
+
+template <int KMAX, bool IDX16, int S, int CAP>
+__global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
+    int n2, int k, int slice_len)
+{
+    using Lay = KnnTreeLayout<KMAX, IDX16>;
+    using Split = KnnSplitLayout<KMAX, IDX16, S, CAP>;
+    using Idx = typename Lay::Idx;
+    constexpr int CHUNK = 32;
+    constexpr int NT = 64;
+    constexpr int HALF = KMAX / 2;
+    constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : KMAX == 64 ? 6
+                           : KMAX == 128 ? 7 : 8;
+    static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 256");
+    extern __shared__ __align__(16) unsigned char knn_split_lds[];
+    __shared__ int s_count[S][NT];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned char *const mine = knn_split_lds + wave * Split::WAVE_BYTES;
+    float *const leaf = reinterpret_cast<float *>(mine) + lane;
+    Idx *const kidx = reinterpret_cast<Idx *>(mine + Lay::LEAF_BYTES) + lane;
+    float *const ival = reinterpret_cast<float *>(mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
+    unsigned char *const iarg =
+        mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
+    auto log_of = [&](int w) {
+        return reinterpret_cast<Idx *>(knn_split_lds + w * Split::WAVE_BYTES + Lay::BYTES) + lane;
+    };
+    Idx *const log = log_of(wave);
+
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
+    const bool active = qi < n1;
+    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
+    float qx = 0, qy = 0, qz = 0;
+    if (active) {
+        const float *q = query + ((int64_t)b * n1 + qi) * 3;
+        qx = q[0];
+        qy = q[1];
+        qz = q[2];
+    }
+
+    auto leaf_parent = [&](int n, float &v, int &a) {
+        const int s = 2 * n - KMAX;
+        const float lv = leaf[s * NT], rv = leaf[(s + 1) * NT];
+        const bool right = rv > lv;
+        v = right ? rv : lv;
+        a = right ? s + 1 : s;
+    };
+
+    // Slots: wave 0 fills them with keys 0..k-1 (mink.cuh:63-72; unused slots hold -inf);
+    // the other waves start from k empty slots (+inf), which any real distance displaces.
+    bool frozen = false;
+    for (int s = 0; s < KMAX; ++s) {
+        float d = -__builtin_huge_valf();
+        if (s < k) {
+            if (wave == 0) {
+                d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+                if (d != d) {
+                    frozen |= s == 0;
+                    d = -__builtin_huge_valf();
+                }
+            } else {
+                d = __builtin_huge_valf();
+            }
+        }
+        leaf[s * NT] = d;
+        kidx[s * NT] = (Idx)s;
+    }
+    for (int n = HALF - 1; n >= 1; --n) {
+        float lv, rv;
+        int la, ra;
+        if (2 * n >= HALF) {
+            leaf_parent(2 * n, lv, la);
+            leaf_parent(2 * n + 1, rv, ra);
+        } else {
+            lv = ival[2 * n * NT];
+            rv = ival[(2 * n + 1) * NT];
+            la = iarg[2 * n * NT];
+            ra = iarg[(2 * n + 1) * NT];
+        }
+        const bool right = rv > lv;
+        ival[n * NT] = right ? rv : lv;
+        iarg[n * NT] = (unsigned char)(right ? ra : la);
+    }
+    float max_key = frozen ? -__builtin_huge_valf() : ival[NT];
+    int max_idx = iarg[NT];
+    int logged = 0;  // entries this lane wrote to its log (may exceed CAP: overflow)
+
+    // MinK's insertion of key j at distance d < max_key (see knn_tree_kernel_f32).
+    auto insert = [&](float d, int j) {
+        const int p = max_idx;
+        leaf[p * NT] = d;
+        kidx[p * NT] = (Idx)j;
+        float sv[LEVELS];
+        int sa[LEVELS];
+        sv[0] = leaf[(p ^ 1) * NT];
+        sa[0] = p ^ 1;
+        leaf_parent(((KMAX + p) >> 1) ^ 1, sv[1], sa[1]);
+#pragma unroll
+        for (int l = 2; l < LEVELS; ++l) {
+            const int sib = ((KMAX + p) >> l) ^ 1;
+            sv[l] = ival[sib * NT];
+            sa[l] = iarg[sib * NT];
+        }
+        float v = d;
+        int a = p;
+#pragma unroll
+        for (int l = 0; l < LEVELS; ++l) {
+            const int node = (KMAX + p) >> l;
+            const bool take = (node & 1) ? !(v > sv[l]) : (sv[l] > v);
+            v = take ? sv[l] : v;
+            a = take ? sa[l] : a;
+            if (l >= 1 && l + 1 < LEVELS) {
+                ival[(node >> 1) * NT] = v;
+                iarg[(node >> 1) * NT] = (unsigned char)a;
+            }
+        }
+        max_key = v;
+        max_idx = v != d ? a : p;
+    };
+
+    // Sweep of the keys [k_begin, k_end) in chunks of 32, inserting (and, for the waves
+    // other than 0, logging) as the tree kernel does. `skip_below`: keys the fill took.
+    auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
+        for (int first = k_begin; first < k_end; first += CHUNK) {
+            const int maxbits = __builtin_bit_cast(int, max_key);
+            unsigned mask = 0u;
+            if (first + CHUNK <= k_end) {
+                const float *__restrict__ g = K + (int64_t)first * 3;
+#pragma unroll
+                for (int i = 0; i < CHUNK; ++i) {
+                    const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
+                                                    qy, qz);
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                }
+            } else {
+                for (int i = 0; i < CHUNK; ++i) {
+                    const int j = first + i < k_end ? first + i : k_end - 1;  // masked below
+                    const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
+                                                    K[(int64_t)j * 3 + 2], qx, qy, qz);
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                }
+            }
+            int lo = skip_below - first;
+            lo = lo < 0 ? 0 : (lo > CHUNK ? CHUNK : lo);
+            int hi = k_end - first;
+            hi = hi > CHUNK ? CHUNK : hi;
+            unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
+            valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
+            mask &= valid;
+            const float *__restrict__ ck = K + (int64_t)first * 3;
+            bool has = mask != 0u;
+            int i = has ? __builtin_clz(mask) : 0;
+            float ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
+            while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+                mask &= ~(0x80000000u >> i);
+                const bool has_next = mask != 0u;
+                const int i_next = has_next ? __builtin_clz(mask) : 0;
+                const float nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
+                            nz = ck[3 * i_next + 2];
+                const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+                if (has && d < max_key) {
+                    insert(d, first + i);
+                    if (write_log) {
+                        if (logged < CAP)
+                            log[logged * NT] = (Idx)(first + i);
+                        ++logged;
+                    }
+                }
+                has = has_next;
+                i = i_next;
+                ex = nx;
+                ey = ny;
+                ez = nz;
+            }
+        }
+    };
+
+    const int k_begin = wave * slice_len;
+    const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
+    if (wave == 0)
+        sweep(0, k_end, k, false);
+    else if (k_begin < n2)
+        sweep(k_begin, k_end, 0, true);
+    s_count[wave][lane] = logged;
+    __syncthreads();
+    if (wave != 0)
+        return;
+
+    // ---- wave 0 replays the other slices in key order ----
+    for (int w = 1; w < S; ++w) {
+        const int w_begin = w * slice_len;
+        if (w_begin >= n2)
+            break;
+        const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
+        const int count = s_count[w][lane];
+        if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
+            sweep(w_begin, w_end, 0, false);
+            continue;
+        }
+        const Idx *__restrict__ wl = log_of(w);
+        int r = 0;
+        bool has = r < count;
+        int j = has ? (int)wl[0] : w_begin;
+        float ex = K[(int64_t)j * 3 + 0], ey = K[(int64_t)j * 3 + 1], ez = K[(int64_t)j * 3 + 2];
+        while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+            const bool has_next = r + 1 < count;
+            const int j_next = has_next ? (int)wl[(r + 1) * NT] : w_begin;
+            const float nx = K[(int64_t)j_next * 3 + 0], ny = K[(int64_t)j_next * 3 + 1],
+                        nz = K[(int64_t)j_next * 3 + 2];
+            const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+            if (has && d < max_key)
+                insert(d, j);
+            ++r;
+            has = has_next;
+            j = j_next;
+            ex = nx;
+            ey = ny;
+            ez = nz;
+        }
+    }
+
+    if (active) {
+        float *od = distance + ((int64_t)b * n1 + qi) * k;
+        int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
+        for (int s = 0; s < k; ++s) {
+            float d = leaf[s * NT];
+            if (d == -__builtin_huge_valf())  // a NaN of the fill phase, still in its slot
+                d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            od[s] = d;
+            oi[s] = (int64_t)kidx[s * NT];
+        }
+    }
+}
+
+// Launch with S = 4 waves per 64 queries when the plain launch would leave most SIMDs
+// without a wave; returns TK3D_ERR_UNSUPPORTED when it does not apply.
+template <int KMAX, int CAP>
+int knn_tree_split_launch(const float *query, const float *key, float *distance,
+                          int64_t *index, int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    constexpr int S = 4;
+    using Split = KnnSplitLayout<KMAX, true, S, CAP>;
+    static_assert(Split::BYTES <= 160 * 1024, "LDS of one CU");
+    int slice_len = (n2 + S - 1) / S;
+    slice_len = (slice_len + 31) / 32 * 32;
+    const int64_t bpb = ((int64_t)n1 + 63) / 64;
+    // Worth it when sweeping dominates the insertions (timed on an MI355X): from 2048 keys
+    // for k <= 8, from 4096 for k <= 16, and only while every workgroup has a CU to itself.
+    if (n2 > 65536 || n2 < (KMAX <= 8 ? 2048 : 4096) || slice_len < k || B * bpb > 256)
+        return TK3D_ERR_UNSUPPORTED;
+    constexpr auto kernel = knn_tree_split_kernel_f32<KMAX, true, S, CAP>;
+    const int allowed = tk_allow_dynamic_lds<kernel>(Split::BYTES);
+    if (allowed != TK3D_OK)
+        return allowed;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(64 * S), Split::BYTES, s, query,
+                       key, distance, index, (int)bpb, n1, n2, k, slice_len);
+    return tk_launch_status();
+}
+
 template <int KMAX, bool IDX16>
 int knn_tree_launch_as(const float *query, const float *key, float *distance, int64_t *index,
                        int64_t B, int n1, int n2, int k, hipStream_t s)
@@ -720,6 +1002,16 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
         // 0.30 ms against 0.41 ms with the slots in registers). Small launches with k <= 8
         // are a little faster in registers.
+        if (k <= 16) {
+            // few queries: four waves share the keys of every 64 queries (1.2-3.3 times
+            // faster from 2048 / 4096 keys on; k = 17..32 logs too many insertions to gain)
+            const int rc = k <= 8 ? knn_tree_split_launch<8, 224>(query, key, distance, index, B,
+                                                                  n1, n2, kk, s)
+                                  : knn_tree_split_launch<16, 224>(query, key, distance, index,
+                                                                   B, n1, n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
         if (k <= 8 && B * N1 < 131072)
             knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
         else if (k <= 8)
