@@ -113,7 +113,8 @@ def test_group_points_with_xyz_skips_unwanted_gradients(cuda):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-@pytest.mark.parametrize("b,n1,n2", [(2, 1000, 300), (32, 8192, 2048), (1, 10, 3)])
+@pytest.mark.parametrize("b,n1,n2", [(2, 1000, 300), (32, 8192, 2048), (1, 10, 3),
+                                     (2, 3000, 4100), (1, 16384, 1024)])
 def test_three_nn_matches_knn_and_the_weight_recipe(cuda, dtype, b, n1, n2):
     from torkit3d_amd import _C
     from torkit3d_amd.ops.interpolate_feature import three_nn_interpolation

@@ -156,3 +156,31 @@ def test_shared_key_sweep_ties_and_nan(cuda, k):
     key[0, 3000:3100] = float("nan")
     key[1, 4499] = float("inf")
     check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("b,n1,n2,k", [(1, 1000, 3000, 3), (2, 700, 5001, 4), (1, 64, 1024, 1),
+                                        (3, 2000, 4096, 2), (1, 300, 65536, 3),
+                                        (1, 32768, 1500, 3), (2, 100, 1025, 4)])
+def test_shared_key_sweep_for_k_up_to_4(cuda, b, n1, n2, k):
+    g = gen(n1 + n2 + k)
+    check_raw(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), k, cuda)
+
+
+@pytest.mark.parametrize("k", [1, 3, 4])
+def test_shared_key_sweep_for_small_k_on_hard_inputs(cuda, k):
+    g = gen(41)
+    # far-to-near keys: every key is inserted, the logs overflow
+    q = uniform_cloud(g, 2, 300) * 0.01
+    r = torch.linspace(5.0, 0.1, 3000)
+    key = torch.stack([r, torch.zeros_like(r), torch.zeros_like(r)], dim=1)[None].repeat(2, 1, 1)
+    check_raw(q, key + 1e-4 * uniform_cloud(g, 2, 3000), k, cuda)
+    # exact ties
+    check_raw(lattice_cloud(g, 2, 500, 4), lattice_cloud(g, 2, 2500, 4), k, cuda)
+    # NaN in the fill, at the start of a slice, in a run; an infinite key
+    q, key = uniform_cloud(g, 2, 500), uniform_cloud(g, 2, 2500)
+    key[0, 0, 1] = float("nan")
+    key[1, min(k - 1, 2), 0] = float("nan")
+    key[1, 640, 2] = float("nan")        # first key of the second slice (4 slices of 640)
+    key[0, 1500:1600] = float("nan")
+    key[1, 2499] = float("inf")
+    check_raw(q, key, k, cuda)

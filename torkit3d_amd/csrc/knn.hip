@@ -959,6 +959,203 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_global_kernel(
     }
 }
 
+// k <= 4 with few queries: the shared-key sweep of knn_tree_split_kernel_f32 with the
+// slots in registers. Four waves serve the same 64 queries; wave 0 runs MinK on the first
+// slice of the keys, the others run a MinK of their own on their slices from k empty
+// slots and log the keys they insert; wave 0 then replays the logs in key order (an
+// overflowing log makes it sweep that slice in full).
+template <bool SOA, bool WEIGHTS, int CAP>
+__global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
+    float eps, int blocks_per_batch, int n1, int n2, int k, int slice_len)
+{
+    constexpr int KMAX = 4, CHUNK = 32, NT = 64, S = 4;
+    __shared__ unsigned short s_log[S][CAP][NT];
+    __shared__ int s_count[S][NT];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
+    const bool active = qi < n1;
+    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
+    float qx = 0, qy = 0, qz = 0;
+    if (active) {
+        const float *__restrict__ Q = query + (int64_t)b * n1 * 3;
+        qx = knn_coord<SOA>(Q, n1, qi, 0);
+        qy = knn_coord<SOA>(Q, n1, qi, 1);
+        qz = knn_coord<SOA>(Q, n1, qi, 2);
+    }
+    auto dist_to = [&](int j) {
+        return tk_dist2<float>(knn_coord<SOA>(K, n2, j, 0), knn_coord<SOA>(K, n2, j, 1),
+                               knn_coord<SOA>(K, n2, j, 2), qx, qy, qz);
+    };
+
+    // Slots: wave 0 fills them with keys 0..k-1 (mink.cuh:63-72); the other waves start
+    // from k empty slots (+inf). Unused slots stay at -inf and are never the maximum.
+    float kd[KMAX];
+    int ki[KMAX];
+    float max_key = 0.0f;
+    int max_idx = 0;
+#pragma unroll
+    for (int s = 0; s < KMAX; ++s) {
+        kd[s] = -__builtin_huge_valf();
+        ki[s] = 0;
+        if (s < k) {  // uniform
+            const float d = wave == 0 ? dist_to(s) : __builtin_huge_valf();
+            kd[s] = d;
+            ki[s] = s;
+            if (s == 0 || d > max_key) {
+                max_key = d;
+                max_idx = s;
+            }
+        }
+    }
+    int logged = 0;
+    // MinK's insertion (mink.cuh:74-87): overwrite the maximum's slot, then rescan from the
+    // inserted key over ascending slots with strict '>'.
+    auto insert = [&](float d, int j) {
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s) {
+            const bool here = (s == max_idx);
+            kd[s] = here ? d : kd[s];
+            ki[s] = here ? j : ki[s];
+        }
+        max_key = d;
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s) {
+            const bool up = kd[s] > max_key;
+            max_key = up ? kd[s] : max_key;
+            max_idx = up ? s : max_idx;
+        }
+    };
+    auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
+        for (int first = k_begin; first < k_end; first += CHUNK) {
+            const int maxbits = __builtin_bit_cast(int, max_key);
+            unsigned mask = 0u;
+            if (first + CHUNK <= k_end) {
+#pragma unroll
+                for (int i = 0; i < CHUNK; ++i) {  // uniform addresses: scalar loads
+                    const unsigned diff =
+                        (unsigned)(__builtin_bit_cast(int, dist_to(first + i)) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
+                }
+            } else {
+                for (int i = 0; i < CHUNK; ++i) {
+                    const int j = first + i < k_end ? first + i : k_end - 1;  // masked below
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, dist_to(j)) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                }
+            }
+            // The sign trick orders bit patterns; a NaN maximum (a NaN in slot 0 of the
+            // fill, which MinK never replaces) admits nothing, as the strict test below
+            // confirms for every candidate anyway.
+            int lo = skip_below - first;
+            lo = lo < 0 ? 0 : (lo > CHUNK ? CHUNK : lo);
+            int hi = k_end - first;
+            hi = hi > CHUNK ? CHUNK : hi;
+            unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
+            valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
+            mask &= valid;
+            bool has = mask != 0u;
+            int i = has ? __builtin_clz(mask) : 0;
+            float d = dist_to(first + i < k_end ? first + i : k_end - 1);
+            while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+                mask &= ~(0x80000000u >> i);
+                const bool has_next = mask != 0u;
+                const int i_next = has_next ? __builtin_clz(mask) : 0;
+                const float d_next = dist_to(first + i_next < k_end ? first + i_next : k_end - 1);
+                if (has && d < max_key) {
+                    insert(d, first + i);
+                    if (write_log) {
+                        if (logged < CAP)
+                            s_log[wave][logged][lane] = (unsigned short)(first + i);
+                        ++logged;
+                    }
+                }
+                has = has_next;
+                i = i_next;
+                d = d_next;
+            }
+        }
+    };
+
+    const int k_begin = wave * slice_len;
+    const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
+    if (wave == 0)
+        sweep(0, k_end, k, false);
+    else if (k_begin < n2)
+        sweep(k_begin, k_end, 0, true);
+    s_count[wave][lane] = logged;
+    __syncthreads();
+    if (wave != 0)
+        return;
+
+    for (int w = 1; w < S; ++w) {
+        const int w_begin = w * slice_len;
+        if (w_begin >= n2)
+            break;
+        const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
+        const int count = s_count[w][lane];
+        if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
+            sweep(w_begin, w_end, 0, false);
+            continue;
+        }
+        int r = 0;
+        bool has = r < count;
+        int j = has ? (int)s_log[w][0][lane] : w_begin;
+        float d = dist_to(j);
+        while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+            const bool has_next = r + 1 < count;
+            const int j_next = has_next ? (int)s_log[w][r + 1 < CAP ? r + 1 : 0][lane] : w_begin;
+            const float d_next = dist_to(j_next);
+            if (has && d < max_key)
+                insert(d, j);
+            ++r;
+            has = has_next;
+            j = j_next;
+            d = d_next;
+        }
+    }
+
+    if (active) {
+        float *od = distance + ((int64_t)b * n1 + qi) * k;
+        int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s) {
+            if (s < k) {
+                od[s] = kd[s];
+                oi[s] = (int64_t)ki[s];
+            }
+        }
+        if constexpr (WEIGHTS) {  // k == 3
+            const float d3[3] = {kd[0], kd[1], kd[2]};
+            knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + qi) * 3);
+        }
+    }
+}
+
+// Applies when the plain launch (one wave per 64 queries) would leave SIMDs idle and the
+// key cloud is long enough; TK3D_ERR_UNSUPPORTED otherwise.
+template <bool SOA, bool WEIGHTS>
+int knn_small_split_launch(const float *query, const float *key, float *distance,
+                           int64_t *index, float *weight, float eps, int64_t B, int n1, int n2,
+                           int k, hipStream_t s)
+{
+    constexpr int S = 4, CAP = 96;
+    int slice_len = (n2 + S - 1) / S;
+    slice_len = (slice_len + 31) / 32 * 32;
+    const int64_t bpb = ((int64_t)n1 + 63) / 64;
+    // 1.2-2.8 times faster than one wave per 64 queries up to 32768 queries in the launch
+    // (timed on an MI355X, 1024 to 65536 keys); slower from 65536 queries on.
+    if (n2 > 65536 || n2 < 1024 || slice_len < k || B * bpb > 512)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((knn_small_split_kernel_f32<SOA, WEIGHTS, CAP>), dim3((unsigned)(B * bpb)),
+                       dim3(64 * S), 0, s, query, key, distance, index, weight, eps, (int)bpb, n1,
+                       n2, k, slice_len);
+    return tk_launch_status();
+}
+
 template <typename T, int KMAX, bool SOA = false, bool WEIGHTS = false>
 void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64_t B,
                 int bpb, int n1, int n2, int k, hipStream_t s, T *weight = nullptr,
@@ -997,6 +1194,12 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
     hipStream_t s = (hipStream_t)stream;
     const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
     if (k <= 4) {
+        if constexpr (sizeof(T) == 4) {
+            const int rc = knn_small_split_launch<false, false>(query, key, distance, index,
+                                                                nullptr, 0.0f, B, n1, n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
         knn_launch<T, 4>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
     } else if constexpr (sizeof(T) == 4) {
         // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
@@ -1069,6 +1272,17 @@ int three_nn(const T *query, const T *key, bool channels_first, int64_t B, int64
     if (B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
+    if constexpr (sizeof(T) == 4) {
+        const int rc = channels_first
+                           ? knn_small_split_launch<true, true>(query, key, distance, index, weight,
+                                                                (float)eps, B, (int)N1, (int)N2,
+                                                                3, s)
+                           : knn_small_split_launch<false, true>(query, key, distance, index,
+                                                                 weight, (float)eps, B, (int)N1,
+                                                                 (int)N2, 3, s);
+        if (rc != TK3D_ERR_UNSUPPORTED)
+            return rc;
+    }
     if (channels_first)
         knn_launch<T, 4, true, true>(query, key, distance, index, B, (int)bpb, (int)N1, (int)N2,
                                      3, s, weight, (T)eps);
