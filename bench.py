@@ -244,6 +244,13 @@ def secondary_metrics(dev, steps, warmup, cpu):
         cq, ck = q[:2].cpu().numpy(), key[:2].cpu().numpy()
         cpu_out["knn_B32_N8192_M2048_k16_ms"] = cpu_ms(lambda: oracle.knn(cq, ck, 16), 32 / 2)
         cpu_out["knn_B32_N8192_M2048_k3_ms"] = cpu_ms(lambda: oracle.knn(cq, ck, 3), 32 / 2)
+    # One cloud: too few queries for one wave per 64 of them to fill the chip, so four
+    # waves share the keys of every 64 queries.
+    one = (torch.rand(1, 16384, 3, generator=g) * 2 - 1).to(dev)
+    out["knn_B1_N16384_M16384_k16_ms"] = gpu_time_ms(
+        lambda: _C.knn_distance_cuda(one, one, 16, 1), max(5, steps // 5), 3)
+    out["knn_B1_N16384_M4096_k3_ms"] = gpu_time_ms(
+        lambda: _C.knn_distance_cuda(one, one[:, :4096].contiguous(), 3, 1), max(5, steps // 5), 3)
     d2, kidx = _C.knn_distance_cuda(q, key, 3, 1)
     w = three_nn_weights(d2)
     f4 = torch.randn(32, 128, 2048, generator=g).to(dev)
