@@ -3,8 +3,10 @@
 //
 // Forward design
 // --------------
-// One workgroup owns QPL*BLOCK query points of one cloud and sweeps the whole
-// opposite cloud. Key points are staged through LDS as (x,y,z,pad) quads; every
+// One workgroup owns QPL*BLOCK query points of one cloud and sweeps the opposite cloud -
+// all of it, or one slice of it when the launch would otherwise leave most of the chip
+// idle (the slices' results then meet in a packed 64-bit minimum, see chamfer_emit).
+// Key points are staged through LDS as (x,y,z,pad) quads; every
 // lane reads the same quad (a broadcast ds_read_b128) and applies it to the QPL
 // queries it keeps in registers, so one LDS read feeds QPL distance evaluations.
 //
