@@ -255,3 +255,23 @@ def test_backward_into_rows_longer_than_lds(cuda, n1):
     for i in range(3):
         want.scatter_add_(2, index3[:, None, :, i].expand(b, c, n2), grad3 * weight[:, None, :, i])
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("n1", [16385, 32768, 32769])
+def test_forward_from_rows_longer_than_64_kib(cuda, n1):
+    """Rows up to 128 KiB are staged one at a time, longer ones read through the cache;
+    both must equal torch.gather (weights k/4 keep the interpolation sums exact)."""
+    from torkit3d_amd import _C
+
+    g = torch.Generator().manual_seed(n1)
+    feat = torch.randint(-8, 9, (2, 6, n1), generator=g).float().to(cuda)
+    index = torch.randint(0, n1, (2, 3000, 5), generator=g).to(cuda)
+    index[0, 0] = n1 - 1
+    want = torch.gather(feat, 2, index.view(2, 1, -1).expand(2, 6, -1)).view(2, 6, 3000, 5)
+    assert torch.equal(_C.group_points_forward_cuda(feat, index), want)
+    index3 = torch.randint(0, n1, (2, 3000, 3), generator=g).to(cuda)
+    weight = (torch.randint(0, 5, (2, 3000, 3), generator=g).float() / 4).to(cuda)
+    want = torch.zeros(2, 6, 3000, device=cuda)
+    for i in range(3):
+        want += torch.gather(feat, 2, index3[:, None, :, i].expand(2, 6, 3000)) * weight[:, None, :, i]
+    assert torch.equal(_C.interpolate_forward_cuda(feat, index3, weight), want)

@@ -601,13 +601,21 @@ int gather(const T *in, const int64_t *idx, const T *w, int64_t B, int64_t C, in
     // 16-byte stores need every output row to start on a 16-byte boundary.
     const int vec_ok = (((uintptr_t)out & 15) == 0) && ((NP * (int64_t)sizeof(T)) % 16 == 0);
 
-    constexpr int64_t LDS_BUDGET = 64 * 1024;
+    // Rows are staged in LDS: up to 64 KiB per workgroup (two workgroups per CU), or one
+    // row of up to 128 KiB when a row alone is longer than that (32768 fp32 elements).
     const int64_t row_bytes = N1 * (int64_t)sizeof(T);
+    const int64_t LDS_BUDGET = row_bytes > 64 * 1024 ? 128 * 1024 : 64 * 1024;
     if (row_bytes > 0 && row_bytes <= LDS_BUDGET && NP >= 1024) {
         constexpr int NT = 512;
         int cg = 8;
         while (cg > 1 && (cg * row_bytes > LDS_BUDGET || cg > C))
             cg /= 2;
+        if (cg * row_bytes > 48 * 1024) {
+            const int allowed =
+                tk_allow_dynamic_lds<gather_lds_kernel<T, KK, HAS_W, V, NT>>(128 * 1024);
+            if (allowed != TK3D_OK)
+                return allowed;
+        }
         const int64_t gy = (C + cg - 1) / cg;
         // Split the points until the chip is full; every chunk re-stages its rows, so
         // keep a chunk well above the staged size.
