@@ -126,35 +126,38 @@ def test_errors(cuda):
 @pytest.mark.parametrize("b,n1,n2,k", [(1, 1000, 4096, 16), (2, 700, 5001, 9), (1, 64, 2048, 5),
                                         (3, 2000, 4100, 8), (1, 16384, 16384, 16),
                                         (1, 300, 65536, 12), (2, 100, 2049, 7),
-                                        (1, 5000, 8191, 13)])
+                                        (1, 5000, 8191, 13), (1, 500, 9000, 20),
+                                        (2, 300, 8192, 32), (1, 200, 65536, 17)])
 def test_shared_key_sweep_shapes(cuda, b, n1, n2, k):
     g = gen(n1 + n2 + k)
     check_raw(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), k, cuda)
 
 
-@pytest.mark.parametrize("k", [6, 16])
+@pytest.mark.parametrize("k", [6, 16, 24])
 def test_shared_key_sweep_with_overflowing_logs(cuda, k):
     # keys ordered from far to near: every key beats the k best before it, so every key of
     # every slice is logged and the logs overflow
     g = gen(31)
     q = uniform_cloud(g, 2, 500) * 0.01
-    r = torch.linspace(5.0, 0.1, 6000)
+    r = torch.linspace(5.0, 0.1, 9000)
     key = torch.stack([r, torch.zeros_like(r), torch.zeros_like(r)], dim=1)[None].repeat(2, 1, 1)
-    key = key + 1e-4 * uniform_cloud(g, 2, 6000)
+    key = key + 1e-4 * uniform_cloud(g, 2, 9000)
     check_raw(q, key, k, cuda)
 
 
-@pytest.mark.parametrize("k", [5, 16])
-def test_shared_key_sweep_ties_and_nan(cuda, k):
+@pytest.mark.parametrize("k,n2", [(5, 4500), (16, 4500), (28, 9000)])
+def test_shared_key_sweep_ties_and_nan(cuda, k, n2):
     g = gen(32)
-    q, key = lattice_cloud(g, 2, 800, 4), lattice_cloud(g, 2, 4500, 4)
+    q, key = lattice_cloud(g, 2, 800, 4), lattice_cloud(g, 2, n2, 4)
     check_raw(q, key, k, cuda)
-    q, key = uniform_cloud(g, 2, 800), uniform_cloud(g, 2, 4500)
+    q, key = uniform_cloud(g, 2, 800), uniform_cloud(g, 2, n2)
     key[0, 0, 1] = float("nan")          # slot 0 of the fill: the lane never inserts again
     key[1, 3, 0] = float("nan")          # a later fill slot
     key[1, 1152, 2] = float("nan")       # first key of the second slice (4 slices of 1152)
+    if n2 > 4512:
+        key[1, 4512, 2] = float("nan")   # first key of the second of 2 slices of 4512
     key[0, 3000:3100] = float("nan")
-    key[1, 4499] = float("inf")
+    key[1, n2 - 1] = float("inf")
     check_raw(q, key, k, cuda)
 
 

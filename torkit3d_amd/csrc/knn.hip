@@ -590,8 +590,8 @@ template <int KMAX, bool IDX16, int S, int CAP> struct KnnSplitLayout {
     using Tree = KnnTreeLayout<KMAX, IDX16>;
     using Idx = typename Tree::Idx;
     static constexpr int LOG_BYTES = (int)sizeof(Idx) * CAP * 64;
-    static constexpr int WAVE_BYTES = Tree::BYTES + LOG_BYTES;
-    static constexpr int BYTES = S * WAVE_BYTES;
+    static constexpr int LOGS_AT = S * Tree::BYTES;          // S trees, then S - 1 logs
+    static constexpr int BYTES = LOGS_AT + (S - 1) * LOG_BYTES;  // (wave 0 keeps none)
 };
 
 template <int KMAX, bool IDX16, int S, int CAP>
@@ -613,16 +613,17 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     __shared__ int s_count[S][NT];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    unsigned char *const mine = knn_split_lds + wave * Split::WAVE_BYTES;
+    unsigned char *const mine = knn_split_lds + wave * Lay::BYTES;
     float *const leaf = reinterpret_cast<float *>(mine) + lane;
     Idx *const kidx = reinterpret_cast<Idx *>(mine + Lay::LEAF_BYTES) + lane;
     float *const ival = reinterpret_cast<float *>(mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
     unsigned char *const iarg =
         mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
-    auto log_of = [&](int w) {
-        return reinterpret_cast<Idx *>(knn_split_lds + w * Split::WAVE_BYTES + Lay::BYTES) + lane;
+    auto log_of = [&](int w) {  // w >= 1
+        return reinterpret_cast<Idx *>(knn_split_lds + Split::LOGS_AT +
+                                       (w - 1) * Split::LOG_BYTES) + lane;
     };
-    Idx *const log = log_of(wave);
+    Idx *const log = log_of(wave > 0 ? wave : 1);  // wave 0 never writes one
 
     const int b = blockIdx.x / blocks_per_batch;
     const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
@@ -832,21 +833,22 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     }
 }
 
-// Launch with S = 4 waves per 64 queries when the plain launch would leave most SIMDs
+// Launch with S waves per 64 queries when the plain launch would leave most SIMDs
 // without a wave; returns TK3D_ERR_UNSUPPORTED when it does not apply.
-template <int KMAX, int CAP>
+template <int KMAX, int S, int CAP>
 int knn_tree_split_launch(const float *query, const float *key, float *distance,
                           int64_t *index, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    constexpr int S = 4;
     using Split = KnnSplitLayout<KMAX, true, S, CAP>;
-    static_assert(Split::BYTES <= 160 * 1024, "LDS of one CU");
+    static_assert(Split::BYTES + 64 * S * 4 <= 160 * 1024, "LDS of one CU");
     int slice_len = (n2 + S - 1) / S;
     slice_len = (slice_len + 31) / 32 * 32;
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     // Worth it when sweeping dominates the insertions (timed on an MI355X): from 2048 keys
-    // for k <= 8, from 4096 for k <= 16, and only while every workgroup has a CU to itself.
-    if (n2 > 65536 || n2 < (KMAX <= 8 ? 2048 : 4096) || slice_len < k || B * bpb > 256)
+    // for k <= 8, 4096 for k <= 16, 8192 for k <= 32, and only while every workgroup has a
+    // CU to itself.
+    constexpr int MIN_KEYS = KMAX <= 8 ? 2048 : KMAX <= 16 ? 4096 : 8192;
+    if (n2 > 65536 || n2 < MIN_KEYS || slice_len < k || B * bpb > 256)
         return TK3D_ERR_UNSUPPORTED;
     constexpr auto kernel = knn_tree_split_kernel_f32<KMAX, true, S, CAP>;
     const int allowed = tk_allow_dynamic_lds<kernel>(Split::BYTES);
@@ -1207,11 +1209,19 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         // are a little faster in registers.
         if (k <= 16) {
             // few queries: four waves share the keys of every 64 queries (1.2-3.3 times
-            // faster from 2048 / 4096 keys on; k = 17..32 logs too many insertions to gain)
-            const int rc = k <= 8 ? knn_tree_split_launch<8, 224>(query, key, distance, index, B,
-                                                                  n1, n2, kk, s)
-                                  : knn_tree_split_launch<16, 224>(query, key, distance, index,
-                                                                   B, n1, n2, kk, s);
+            // faster from 2048 / 4096 keys on)
+            const int rc = k <= 8 ? knn_tree_split_launch<8, 4, 352>(query, key, distance, index,
+                                                                     B, n1, n2, kk, s)
+                                  : knn_tree_split_launch<16, 4, 320>(query, key, distance,
+                                                                      index, B, n1, n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
+        if (k > 16 && k <= 32) {
+            // k = 17..32 logs more insertions: two waves per 64 queries, the second wave's
+            // log gets all the spare LDS (1.15-1.5 times faster from 8192 keys on)
+            const int rc = knn_tree_split_launch<32, 2, 896>(query, key, distance, index, B, n1,
+                                                             n2, kk, s);
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
