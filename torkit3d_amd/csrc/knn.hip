@@ -973,7 +973,7 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
     float eps, int blocks_per_batch, int n1, int n2, int k, int slice_len)
 {
     constexpr int KMAX = 4, CHUNK = 32, NT = 64, S = 4;
-    __shared__ unsigned short s_log[S][CAP][NT];
+    __shared__ unsigned short s_log[S - 1][CAP][NT];  // wave 0 keeps none
     __shared__ int s_count[S][NT];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1071,7 +1071,7 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
                     insert(d, first + i);
                     if (write_log) {
                         if (logged < CAP)
-                            s_log[wave][logged][lane] = (unsigned short)(first + i);
+                            s_log[wave - 1][logged][lane] = (unsigned short)(first + i);
                         ++logged;
                     }
                 }
@@ -1105,11 +1105,11 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
         }
         int r = 0;
         bool has = r < count;
-        int j = has ? (int)s_log[w][0][lane] : w_begin;
+        int j = has ? (int)s_log[w - 1][0][lane] : w_begin;
         float d = dist_to(j);
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
             const bool has_next = r + 1 < count;
-            const int j_next = has_next ? (int)s_log[w][r + 1 < CAP ? r + 1 : 0][lane] : w_begin;
+            const int j_next = has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : w_begin;
             const float d_next = dist_to(j_next);
             if (has && d < max_key)
                 insert(d, j);
