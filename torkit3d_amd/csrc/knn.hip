@@ -1149,8 +1149,10 @@ int knn_small_split_launch(const float *query, const float *key, float *distance
     slice_len = (slice_len + 31) / 32 * 32;
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     // 1.2-2.8 times faster than one wave per 64 queries up to 32768 queries in the launch
-    // (timed on an MI355X, 1024 to 65536 keys); slower from 65536 queries on.
-    if (n2 > 65536 || n2 < 1024 || slice_len < k || B * bpb > 512)
+    // (timed on an MI355X, 1024 to 65536 keys); with 65536 queries only from 16384 keys on
+    // (1.2-1.3 times), slower otherwise.
+    const int64_t groups = B * bpb;
+    if (n2 > 65536 || n2 < 1024 || slice_len < k || groups > 1024 || (groups > 512 && n2 < 16384))
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((knn_small_split_kernel_f32<SOA, WEIGHTS, CAP>), dim3((unsigned)(B * bpb)),
                        dim3(64 * S), 0, s, query, key, distance, index, weight, eps, (int)bpb, n1,
