@@ -86,8 +86,10 @@ def chamfer_forward(xyz1, xyz2, fused=True):
     return d1, i1, d2, i2
 
 
-def chamfer_backward(grad_dist1, grad_dist2, xyz1, xyz2, idx1, idx2):
-    """-> grad_xyz1 [B,N1,3], grad_xyz2 [B,N2,3]."""
+def chamfer_backward(grad_dist1, grad_dist2, xyz1, xyz2, idx1, idx2, wide=False):
+    """-> grad_xyz1 [B,N1,3], grad_xyz2 [B,N2,3]. ``wide``: every term as the reference
+    forms it, summed in double and rounded once (the yardstick for fp32 kernels, whose
+    summation order differs from the sequential one of ``wide=False``)."""
     xyz1 = _c(xyz1)
     dt = xyz1.dtype
     xyz2, g1, g2 = _c(xyz2, dt), _c(grad_dist1, dt), _c(grad_dist2, dt)
@@ -96,7 +98,7 @@ def chamfer_backward(grad_dist1, grad_dist2, xyz1, xyz2, idx1, idx2):
     n2 = xyz2.shape[1]
     gx1 = np.empty((b, n1, 3), dt)
     gx2 = np.empty((b, n2, 3), dt)
-    _call("tk3d_oracle_chamfer_backward" + _sfx(xyz1), _p(g1), _p(g2), _p(xyz1),
+    _call("tk3d_oracle_chamfer_backward" + ("_wide" if wide else "") + _sfx(xyz1), _p(g1), _p(g2), _p(xyz1),
           _p(xyz2), _p(idx1), _p(idx2), _i(b), _i(n1), _i(n2), _p(gx1), _p(gx2))
     return gx1, gx2
 
@@ -150,12 +152,13 @@ def group_forward(inp, index):
     return out
 
 
-def group_backward(grad_output, index, n1):
-    """-> grad_input [B,C,n1]."""
+def group_backward(grad_output, index, n1, wide=False):
+    """-> grad_input [B,C,n1]. ``wide``: sums in double, rounded once."""
     grad_output, index = _c(grad_output), _c(index, np.int64)
     b, c, n2, k = grad_output.shape
     gin = np.empty((b, c, n1), grad_output.dtype)
-    _call("tk3d_oracle_group_backward" + _sfx(grad_output), _p(grad_output),
+    _call("tk3d_oracle_group_backward" + ("_wide" if wide else "") + _sfx(grad_output),
+          _p(grad_output),
           _p(index), _i(b), _i(c), _i(n1), _i(n2), _i(k), _p(gin),
           restype=ctypes.c_int64)
     return gin
@@ -174,14 +177,16 @@ def interpolate_forward(inp, index, weight):
     return out
 
 
-def interpolate_backward(grad_output, index, weight, n1):
-    """-> grad_input [B,C,n1]."""
+def interpolate_backward(grad_output, index, weight, n1, wide=False):
+    """-> grad_input [B,C,n1]. ``wide``: terms in the data type, sums in double, rounded
+    once."""
     grad_output, index = _c(grad_output), _c(index, np.int64)
     weight = _c(weight, grad_output.dtype)
     b, c, n2 = grad_output.shape
     k = index.shape[2]
     gin = np.empty((b, c, n1), grad_output.dtype)
-    _call("tk3d_oracle_interpolate_backward" + _sfx(grad_output), _p(grad_output),
+    _call("tk3d_oracle_interpolate_backward" + ("_wide" if wide else "") + _sfx(grad_output),
+          _p(grad_output),
           _p(index), _p(weight), _i(b), _i(c), _i(n1), _i(n2), _i(k), _p(gin),
           restype=ctypes.c_int64)
     return gin

@@ -75,8 +75,14 @@ def test_edge_cases(cuda):
         np.testing.assert_array_equal(got, oracle.ball_query(query.numpy(), key.numpy(), r, k))
     assert (got[:, 45:] == -1).all()  # no hit: the row stays -1
     # tiny radius, queries are key points: the only hits are coincident points, first one padded
-    got = _C.ball_query_cuda(key[:, :10].contiguous().to(cuda), key.to(cuda), 1e-6, 4).cpu().numpy()
-    assert (got == got[:, :, :1]).all() or True
+    # (a lattice cloud repeats positions, so a row lists up to 4 coincident key indices in
+    # ascending order and pads with the first)
+    own = key[:, :10].contiguous()
+    got = _C.ball_query_cuda(own.to(cuda), key.to(cuda), 1e-6, 4).cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.ball_query(own.numpy(), key.numpy(), 1e-6, 4))
+    hit = torch.gather(key, 1, torch.from_numpy(got).reshape(2, -1, 1).expand(-1, -1, 3))
+    assert torch.equal(hit.view(2, 10, 4, 3), own[:, :, None, :].expand(-1, -1, 4, -1))
+    assert (got[:, :, 0] <= np.arange(10)[None, :]).all()  # the first coincident key
     # empty key cloud and k = 0
     out = _C.ball_query_cuda(query.to(cuda), torch.zeros(2, 0, 3, device=cuda), 0.5, 5)
     assert (out == -1).all()

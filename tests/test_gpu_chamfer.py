@@ -1,8 +1,9 @@
 """Chamfer / nearest-neighbour distance on the GPU against the CPU oracle.
 
 Indices and distances must be bit-identical to the oracle (same canonical
-arithmetic); gradients within 1e-5 relative / 1e-6 absolute (the scattered terms
-are summed in a different order)."""
+arithmetic); fp32 gradients within 1e-5 relative / 1e-6 absolute of the oracle's sums
+taken in double and rounded once (the kernel sums in 64-bit fixed point, the reference's
+atomics in an order that changes from run to run)."""
 import numpy as np
 import pytest
 import torch
@@ -53,8 +54,29 @@ def test_forward_fp64_and_transpose(cuda):
     assert torch.equal(out[1].cpu(), D.argmin(2)) and torch.equal(out[3].cpu(), D.argmin(1))
 
 
+def check_backward(a, c, gd1, gd2, i1, i2, cuda, exact_nonfinite=False):
+    """tk3d_chamfer_distance_backward through _C against the double-summing oracle."""
+    from torkit3d_amd import _C
+
+    got = _C.chamfer_distance_backward_cuda(gd1.to(cuda), gd2.to(cuda), a.to(cuda), c.to(cuda),
+                                            torch.as_tensor(i1).to(cuda), torch.as_tensor(i2).to(cuda))
+    want = oracle.chamfer_backward(gd1.numpy(), gd2.numpy(), a.numpy(), c.numpy(),
+                                   np.asarray(i1), np.asarray(i2), wide=True)
+    for name, g, w in zip(("grad_xyz1", "grad_xyz2"), got, want):
+        g = g.cpu().numpy()
+        if exact_nonfinite:
+            assert np.array_equal(np.isnan(g), np.isnan(w)), name
+            assert np.array_equal(np.isposinf(g), np.isposinf(w)), name
+            assert np.array_equal(np.isneginf(g), np.isneginf(w)), name
+            ok = np.isfinite(w)
+            g, w = g[ok], w[ok]
+        np.testing.assert_allclose(g, w, rtol=RTOL, atol=ATOL, err_msg=name)
+    return got
+
+
 def test_stress_config_full_size(cuda):
-    # benchmark config 5: B=32, N=M=16384, points on unit spheres + N(0, 0.01) noise
+    # benchmark config 5: B=32, N=M=16384, points on unit spheres + N(0, 0.01) noise,
+    # forward and backward
     g = gen(5)
     a, c = sphere_cloud(g, 32, 16384), sphere_cloud(g, 32, 16384)
     d1, i1, d2, i2 = check_forward(a, c, cuda)
@@ -63,6 +85,13 @@ def test_stress_config_full_size(cuda):
     np.testing.assert_allclose(((a.to(cuda) - ga) ** 2).sum(-1).cpu().numpy(),
                                d1.cpu().numpy(), rtol=1e-5, atol=1e-7)
     assert float(d1.max()) < 0.05 and int(i1.min()) >= 0 and int(i1.max()) < 16384
+    gd1, gd2 = torch.randn(32, 16384, generator=g), torch.randn(32, 16384, generator=g)
+    gx1, gx2 = check_backward(a, c, gd1, gd2, i1.cpu(), i2.cpu(), cuda)
+    # the terms sent to the other cloud cancel the own terms: both gradients sum to the
+    # same total with opposite sign (each pass adds v to one cloud and -v to the other)
+    t1 = gx1.double().sum(1).cpu().numpy()
+    t2 = gx2.double().sum(1).cpu().numpy()
+    np.testing.assert_allclose(t1, -t2, rtol=1e-4, atol=1e-3)
 
 
 def test_lattice_ties_pick_lowest_index(cuda):
@@ -102,7 +131,7 @@ def test_empty_and_nan_clouds(cuda):
     assert out[0].shape == (1, 6) and out[2].shape == (1, 4)
 
 
-@pytest.mark.parametrize("b,n1,n2", [(2, 1024, 1024), (3, 300, 5000)])
+@pytest.mark.parametrize("b,n1,n2", [(2, 1024, 1024), (3, 300, 5000), (5, 4097, 9000)])
 def test_backward_matches_oracle(cuda, b, n1, n2):
     from torkit3d_amd.ops.chamfer_distance import chamfer_distance
 
@@ -113,10 +142,63 @@ def test_backward_matches_oracle(cuda, b, n1, n2):
     d1, d2 = chamfer_distance(ad, cd)
     torch.autograd.backward([d1, d2], [gd1.to(cuda), gd2.to(cuda)])
     _, i1, _, i2 = oracle.chamfer_forward(a.numpy(), c.numpy())
-    gx1, gx2 = oracle.chamfer_backward(gd1.numpy(), gd2.numpy(), a.numpy(), c.numpy(), i1, i2)
+    gx1, gx2 = oracle.chamfer_backward(gd1.numpy(), gd2.numpy(), a.numpy(), c.numpy(), i1, i2,
+                                       wide=True)
     np.testing.assert_allclose(ad.grad.cpu().numpy(), gx1, rtol=RTOL, atol=ATOL)
-    # many sources can meet in one point of the larger cloud: allow for reordering
-    np.testing.assert_allclose(cd.grad.cpu().numpy(), gx2, rtol=RTOL, atol=1e-5)
+    np.testing.assert_allclose(cd.grad.cpu().numpy(), gx2, rtol=RTOL, atol=ATOL)
+
+
+def test_backward_with_an_empty_cloud_or_unmatched_points(cuda):
+    from torkit3d_amd import _C
+    from torkit3d_amd.ops.chamfer_distance import chamfer_distance
+
+    g = gen(2)
+    # one cloud empty: no point has a match, every gradient is zero
+    a = uniform_cloud(g, 2, 700).to(cuda).requires_grad_()
+    for empty_first in (False, True):
+        e = torch.zeros(2, 0, 3, device=cuda, requires_grad=True)
+        d1, d2 = chamfer_distance(e, a) if empty_first else chamfer_distance(a, e)
+        a.grad = None
+        torch.autograd.backward([d1, d2], [torch.ones_like(d1), torch.ones_like(d2)])
+        assert a.grad.shape == (2, 700, 3) and float(a.grad.abs().max()) == 0.0
+        assert e.grad.shape == (2, 0, 3)
+    # all-NaN keys: the forward reports index -1, which the backward must skip
+    an, cn = uniform_cloud(g, 2, 300), torch.full((2, 200, 3), float("nan"))
+    _, i1, _, i2 = _C.chamfer_distance_forward_cuda(an.to(cuda), cn.to(cuda))
+    assert (i1 == -1).all()
+    gd1, gd2 = torch.randn(2, 300, generator=g), torch.zeros(2, 200)
+    gx1, gx2 = _C.chamfer_distance_backward_cuda(gd1.to(cuda), gd2.to(cuda), an.to(cuda),
+                                                 cn.to(cuda), i1, torch.full_like(i2, -1))
+    assert float(gx1.abs().max()) == 0.0 and float(gx2.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("where", [64, 300, 511, 5000 - 1])
+def test_backward_outlier_missed_by_the_magnitude_sample(cuda, where):
+    # The fixed-point scale comes from a sample of the senders (the first 64 of every 512);
+    # a term far above 8x the sampled maximum must send the workgroup through its second
+    # attempt with the exact bound.
+    g = gen(3)
+    a, c = uniform_cloud(g, 2, 3000), uniform_cloud(g, 2, 5000)
+    gd1, gd2 = torch.randn(2, 3000, generator=g), torch.randn(2, 5000, generator=g)
+    assert where % 512 >= 64
+    gd2[1, where] = 2.0e6
+    _, i1, _, i2 = oracle.chamfer_forward(a.numpy(), c.numpy())
+    check_backward(a, c, gd1, gd2, i1, i2, cuda)
+
+
+def test_backward_non_finite_input_follows_float_arithmetic(cuda):
+    # inf and NaN have no fixed-point image: a workgroup that meets one sums in floating
+    # point and must give what float addition gives
+    g = gen(4)
+    a, c = uniform_cloud(g, 2, 2000), uniform_cloud(g, 2, 2500)
+    gd1, gd2 = torch.randn(2, 2000, generator=g), torch.randn(2, 2500, generator=g)
+    _, i1, _, i2 = oracle.chamfer_forward(a.numpy(), c.numpy())
+    gd2[0, 100] = float("inf")
+    gd2[0, 900] = float("nan")
+    gd1[1, 17] = -float("inf")
+    c = c.clone()
+    c[1, 40, 1] = float("inf")          # a coordinate: its own term and what it sends
+    check_backward(a, c, gd1, gd2, i1, i2, cuda, exact_nonfinite=True)
 
 
 def test_gradcheck_fp64(cuda):

@@ -187,3 +187,29 @@ def test_shared_key_sweep_for_small_k_on_hard_inputs(cuda, k):
     key[0, 1500:1600] = float("nan")
     key[1, 2499] = float("inf")
     check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("k", [3, 4, 5, 8, 16, 17, 33, 130])
+def test_slot_order_of_the_hand_worked_mink_run(cuda, k, dtype):
+    # Expected rows are literals worked out by hand from mink.cuh:61-89 (tests/util.py):
+    # a rejected key equal to the maximum, two slots tying for the new maximum (the lower
+    # one is the next victim), and an insertion that leaves the maximum in the written slot
+    # although a lower slot ties. Every kernel family sees the run (k selects registers,
+    # the LDS tree or the global variant; 70 queries span two waves, 5000 far keys behind
+    # the run exercise the chunked sweeps and must all be rejected).
+    from torkit3d_amd import _C
+    from util import MINK_STATES, mink_worked_example
+
+    for m in sorted(MINK_STATES):
+        key, dist, idx = mink_worked_example(m, k, np.float64)
+        for tail in (0, 5000):
+            far = np.zeros((1, tail, 3))
+            far[0, :, 0] = 50.0 + np.arange(tail) % 7
+            keys = torch.from_numpy(np.concatenate([key, far], 1)).to(dtype).to(cuda)
+            query = torch.zeros(1, 70, 3, dtype=dtype, device=cuda)
+            got_d, got_i = _C.knn_distance_cuda(query, keys, k, 1)
+            want_d = torch.from_numpy(dist).to(dtype).to(cuda).expand(70, -1)
+            want_i = torch.from_numpy(idx).to(cuda).expand(70, -1)
+            assert torch.equal(got_d[0], want_d), "distances, m=%d tail=%d" % (m, tail)
+            assert torch.equal(got_i[0], want_i), "indices, m=%d tail=%d" % (m, tail)

@@ -322,3 +322,51 @@ def test_fps_reference_tie_rule_differs_from_lowest_index():
 def test_fps_all_duplicates_repeat_previous_choice():
     pts = np.ones((2, 40, 3), np.float32)
     np.testing.assert_array_equal(oracle.sample_farthest_points(pts, 10), np.zeros((2, 10)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("k", [3, 4, 5, 8, 16, 33])
+def test_knn_slot_order_of_the_hand_worked_mink_run(k, dtype):
+    # expected rows are literals derived by hand from mink.cuh:61-89 (tests/util.py)
+    from util import MINK_STATES, mink_worked_example
+
+    for m in sorted(MINK_STATES):
+        key, dist, idx = mink_worked_example(m, k, dtype)
+        query = np.zeros((1, 2, 3), dtype)
+        query[0, 1, 1] = 100.0  # a second query far away: same order, other distances
+        got_d, got_i = oracle.knn(query, key, k)
+        np.testing.assert_array_equal(got_d[0, 0], dist, err_msg="m=%d" % m)
+        np.testing.assert_array_equal(got_i[0, 0], idx, err_msg="m=%d" % m)
+        np.testing.assert_array_equal(got_i[0, 1], idx, err_msg="m=%d far" % m)
+
+
+def test_chamfer_backward_wide_sums_in_double():
+    # fp32 terms exactly as the reference's threads form them, summed in float64 by numpy
+    g = gen(31)
+    b, n1, n2 = 3, 400, 90
+    a, c = uniform_cloud(g, b, n1).numpy(), uniform_cloud(g, b, n2).numpy()
+    gd1 = torch.randn(b, n1, generator=g).numpy()
+    gd2 = torch.randn(b, n2, generator=g).numpy()
+    _, i1, _, i2 = oracle.chamfer_forward(a, c)
+    i1[0, 5] = -1          # skipped entries
+    i2[1, 7] = n1
+    acc1 = np.zeros((b, n1, 3)), np.zeros((b, n2, 3))
+
+    def one_pass(own, other, gd, idx, x, y):
+        for bi in range(b):
+            ok = (idx[bi] >= 0) & (idx[bi] < y.shape[1])
+            j = idx[bi][ok]
+            v = (gd[bi][ok] * np.float32(2))[:, None] * (x[bi][ok] - y[bi][j])
+            assert v.dtype == np.float32
+            own[bi][ok] += v.astype(np.float64)
+            np.add.at(other[bi], j, -v.astype(np.float64))
+
+    one_pass(acc1[0], acc1[1], gd1, i1, a, c)
+    one_pass(acc1[1], acc1[0], gd2, i2, c, a)
+    gx1, gx2 = oracle.chamfer_backward(gd1, gd2, a, c, i1, i2, wide=True)
+    np.testing.assert_array_equal(gx1, acc1[0].astype(np.float32))
+    np.testing.assert_array_equal(gx2, acc1[1].astype(np.float32))
+    # and it stays within rounding of the sequential fp32 sum
+    sx1, sx2 = oracle.chamfer_backward(gd1, gd2, a, c, i1, i2)
+    np.testing.assert_allclose(gx2, sx2, rtol=1e-4, atol=1e-4)
+    assert not np.array_equal(gx2, sx2)

@@ -102,3 +102,36 @@ def test_out_of_range_indices_are_counted_not_read():
     index = np.array([[[0, 6, -1, 5]]], np.int64)
     out = oracle.group_forward(feat, index)
     np.testing.assert_array_equal(out[0, :, 0], [[0, 0, 0, 5], [6, 0, 0, 11]])
+
+
+def test_wide_backward_variants_sum_in_double():
+    # fp32 terms summed in float64 by numpy and rounded once; duplicate-heavy indices
+    g = gen(9)
+    b, c, n1, n2, k = 2, 5, 37, 300, 6
+    index = torch.randint(0, n1, (b, n2, k), generator=g).numpy()
+    index[:, :, 3:] = index[:, :, :1]       # padded rows: the first hit repeated
+    index[0, 4, 2] = -1                      # skipped
+    go = torch.randn(b, c, n2, k, generator=g).numpy()
+    want = np.zeros((b, c, n1))
+    for bi in range(b):
+        flat = index[bi].reshape(-1)
+        ok = flat >= 0
+        for ch in range(c):
+            np.add.at(want[bi, ch], flat[ok], go[bi, ch].reshape(-1)[ok].astype(np.float64))
+    got = oracle.group_backward(go, index, n1, wide=True)
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+    seq = oracle.group_backward(go, index, n1)
+    np.testing.assert_allclose(got, seq, rtol=1e-4, atol=1e-4)
+    assert not np.array_equal(got, seq)
+
+    index3 = torch.randint(0, n1, (b, n2, 3), generator=g).numpy()
+    weight = torch.rand(b, n2, 3, generator=g).numpy()
+    go3 = torch.randn(b, c, n2, generator=g).numpy()
+    want = np.zeros((b, c, n1))
+    for bi in range(b):
+        for ch in range(c):
+            term = go3[bi, ch][:, None] * weight[bi]        # fp32 products
+            assert term.dtype == np.float32
+            np.add.at(want[bi, ch], index3[bi].reshape(-1), term.reshape(-1).astype(np.float64))
+    got = oracle.interpolate_backward(go3, index3, weight, n1, wide=True)
+    np.testing.assert_array_equal(got, want.astype(np.float32))

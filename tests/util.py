@@ -77,3 +77,63 @@ def sorted_pairs(dist, idx):
     """Rows of (distance, index) sorted by distance then index."""
     order = np.lexsort((idx, dist), axis=-1)
     return np.take_along_axis(dist, order, -1), np.take_along_axis(idx, order, -1)
+
+
+# ---- a MinK run worked out by hand ------------------------------------------------------
+# mink.cuh:61-89 of the reference, k = 3, one query at the origin, keys on the x axis so
+# that the squared distance of key j is MINK_X[j]**2 (all exact in binary):
+#
+#   j   x     d      what MinK::add does                              slots (d, j) afterwards
+#   0   2     4      fill slot 0; first key: max = 4 in slot 0        (4,0)
+#   1  -2     4      fill slot 1; 4 > 4 is false: max stays slot 0    (4,0) (4,1)
+#   2   3     9      fill slot 2; 9 > 4: max = 9 in slot 2            (4,0) (4,1) (9,2)
+#   3  -3     9      9 < 9 is false: rejected (a key equal to the     unchanged
+#                    maximum never enters)
+#   4   1     1      1 < 9: overwrite slot 2; rescan from max = 1:    (4,0) (4,1) (1,4)
+#                    slot 0: 4 > 1 -> max 4, slot 0; slot 1: 4 > 4
+#                    false -> of two equal maxima the LOWER slot is
+#                    the next victim
+#   5   2     4      4 < 4 is false: rejected                         unchanged
+#   6   1.5   2.25   2.25 < 4: overwrite slot 0; rescan from 2.25:    (2.25,6) (4,1) (1,4)
+#                    slot 1: 4 > 2.25 -> max 4, slot 1
+#   7  -1.5   2.25   2.25 < 4: overwrite slot 1; rescan from 2.25:    (2.25,6) (2.25,7) (1,4)
+#                    slot 0: 2.25 > 2.25 false -> the slot just
+#                    written stays the victim although the lower
+#                    slot 0 holds an equal key
+#   8   0.5   0.25   0.25 < 2.25: overwrite slot 1 (not slot 0);      (2.25,6) (0.25,8) (1,4)
+#                    rescan: slot 0: 2.25 > 0.25 -> max 2.25, slot 0
+#   9   0     0      0 < 2.25: overwrite slot 0; rescan: slot 1:      (0,9) (0.25,8) (1,4)
+#                    0.25 > 0 -> slot 1; slot 2: 1 > 0.25 -> slot 2
+#
+# MINK_STATES[m] is the (distance, index) row after the first m keys. Reading the rescan as
+# '>=' changes the row at m = 8, starting the rescan from "no maximum" instead of the
+# written slot changes it at m = 9, accepting a key equal to the maximum changes it at
+# m = 4 and m = 6.
+MINK_X = [2.0, -2.0, 3.0, -3.0, 1.0, 2.0, 1.5, -1.5, 0.5, 0.0]
+MINK_STATES = {
+    3: ([4.0, 4.0, 9.0], [0, 1, 2]),
+    4: ([4.0, 4.0, 9.0], [0, 1, 2]),
+    5: ([4.0, 4.0, 1.0], [0, 1, 4]),
+    6: ([4.0, 4.0, 1.0], [0, 1, 4]),
+    7: ([2.25, 4.0, 1.0], [6, 1, 4]),
+    8: ([2.25, 2.25, 1.0], [6, 7, 4]),
+    9: ([2.25, 0.25, 1.0], [6, 8, 4]),
+    10: ([0.0, 0.25, 1.0], [9, 8, 4]),
+}
+MINK_NEAR = 2.0 ** -6  # |x| of the keys that pad the run to k > 3; its square is 2^-12
+
+
+def mink_worked_example(m, k=3, dtype=np.float32):
+    """Keys [1,k-3+m,3] and the expected (distance [k], index [k]) row for a query at the
+    origin. For k > 3 the run above is preceded by k-3 keys at distance 2^-12: they fill
+    slots 0..k-4 and, being smaller than every later maximum (the rescan's strict '>' never
+    selects them while a larger key is stored), stay there, so the last three slots go
+    through exactly the states of the table with every index shifted by k-3."""
+    pad = k - 3
+    xs = [MINK_NEAR if i % 2 == 0 else -MINK_NEAR for i in range(pad)] + MINK_X[:m]
+    key = np.zeros((1, len(xs), 3), dtype)
+    key[0, :, 0] = xs
+    d, i = MINK_STATES[m]
+    dist = np.asarray([MINK_NEAR ** 2] * pad + d, dtype)
+    idx = np.asarray(list(range(pad)) + [j + pad for j in i], np.int64)
+    return key, dist, idx

@@ -42,20 +42,36 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose=False):
-    """Compile every kernel source for gfx950 and link ``libtk3d.so`` in-tree."""
-    cmd = [hipcc_path()] + HIPCC_FLAGS + [
-        "-I", os.path.join(REPO, "include"), "-I", CSRC,
-        "-o", LIB_PATH + ".tmp"] + sources()
-    if verbose:
-        print(" ".join(cmd))
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines()
-                    if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+def build(verbose=False, jobs=None):
+    """Compile every kernel source for gfx950 (one hipcc process per source file, run side
+    by side) and link ``libtk3d.so`` in-tree."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    include = ["-I", os.path.join(REPO, "include"), "-I", CSRC]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd))
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + out)
+        if verbose and out.strip():
+            print(out)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
+        run([hipcc_path()] + compile_flags + include + ["-c", src, "-o", obj])
+        return obj
+
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=jobs or min(len(srcs), os.cpu_count() or 1, 16)) as pool:
+        objects = list(pool.map(compile_one, srcs))
+    run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH + ".tmp"]
+        + objects)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     return LIB_PATH
 

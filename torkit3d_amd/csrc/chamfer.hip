@@ -736,24 +736,35 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     const float *__restrict__ gd1, const float *__restrict__ gd2,
     const float *__restrict__ xyz1, const float *__restrict__ xyz2,
     const int64_t *__restrict__ idx1, const int64_t *__restrict__ idx2, int n1, int n2,
-    int ranges1, int ranges2, int nblocks1, float *__restrict__ gx1, float *__restrict__ gx2)
+    int ranges1, int ranges2, float *__restrict__ gx1, float *__restrict__ gx2)
 {
     extern __shared__ __align__(16) unsigned long long acc[];  // [R * 3]
     __shared__ unsigned s_max;
     __shared__ int s_exceeded;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
 
-    // Decode: the first nblocks1 workgroups produce grad_xyz1, the rest grad_xyz2.
+    // Decode: a batch's ranges1 + ranges2 workgroups are consecutive logical workgroups
+    // (first those that produce grad_xyz1), and each XCD takes a contiguous run of logical
+    // workgroups (blockIdx goes round-robin over the 8 XCDs): every workgroup of a batch
+    // reads both clouds, both gradients and both index arrays of that batch, which then
+    // come from HBM once and from the XCD's L2 afterwards.
     int lb = blockIdx.x;
-    const bool second = lb >= nblocks1;
-    if (second)
-        lb -= nblocks1;
-    const int ranges = second ? ranges2 : ranges1;
-    const int b = lb / ranges;
-    const int j0 = (lb - b * ranges) * R;
+    {
+        const int per = (int)gridDim.x >> 3, full = per << 3;
+        if (lb < full)
+            lb = (lb & 7) * per + (lb >> 3);
+    }
+    const int b = lb / (ranges1 + ranges2);
+    const int r = lb - b * (ranges1 + ranges2);
+    const bool second = r >= ranges1;
+    const int j0 = (second ? r - ranges1 : r) * R;
     const int nx = second ? n2 : n1, ny = second ? n1 : n2;
     const float *__restrict__ X = (second ? xyz2 : xyz1) + (int64_t)b * nx * 3;
-    const float *__restrict__ Y = (second ? xyz1 : xyz2) + (int64_t)b * ny * 3;
+    // An empty opposite cloud has no storage (its base may be NULL) and sends nothing; the
+    // loads below that fetch a placeholder element before testing the match index then
+    // read this cloud's own first point instead.
+    const float *__restrict__ Y =
+        ny > 0 ? (second ? xyz1 : xyz2) + (int64_t)b * ny * 3 : X;
     const float *__restrict__ gX = (second ? gd2 : gd1) + (int64_t)b * nx;
     const float *__restrict__ gY = (second ? gd1 : gd2) + (int64_t)b * ny;
     const int64_t *__restrict__ iX = (second ? idx2 : idx1) + (int64_t)b * nx;
@@ -912,9 +923,11 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
 #pragma unroll
                     for (int a = 0; a < 3; ++a) {
                         const float own = ok ? gg[f] * (xs[f][a] - ys[f][a]) : 0.0f;
-                        const float sent =
-                            (float)__builtin_ldexp((double)(long long)acc[p * 3 + a], -kexp);
-                        out[(int64_t)(j0 + p) * 3 + a] = own + sent;
+                        // own term and the exact sum of the sent terms meet in double:
+                        // the gradient is rounded once
+                        const double sent =
+                            __builtin_ldexp((double)(long long)acc[p * 3 + a], -kexp);
+                        out[(int64_t)(j0 + p) * 3 + a] = (float)((double)own + sent);
                     }
                 }
             }
@@ -1192,7 +1205,7 @@ int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
                 return allowed;
             hipLaunchKernelGGL(kernel, dim3((unsigned)(B * (r1 + r2))), dim3(NT), lds, s, gd1,
                                gd2, xyz1, xyz2, idx1, idx2, (int)N1, (int)N2, (int)r1, (int)r2,
-                               (int)(B * r1), gx1, gx2);
+                               gx1, gx2);
             return tk_launch_status();
         }
     }
