@@ -169,6 +169,23 @@ int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
                                     void *workspace, size_t workspace_bytes,
                                     void *stream);
 
+/* tk3d_sample_farthest_points_f32 for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops with a frozen memory pool, harnesses that
+ * forbid hipMalloc): no counterpart in the reference. The workspace of the large-cloud
+ * path is a fixed array of TK3D_FPS_STATIC_WORKSPACE_BYTES in the library's device image
+ * (each GPU the library runs on holds its copy until the process ends). Same result as
+ * tk3d_sample_farthest_points_f32. Returns TK3D_ERR_WORKSPACE when
+ * tk3d_sample_farthest_points_workspace_bytes(B, N, 4) exceeds that size (8 MiB: e.g. one
+ * cloud of 2 million points, or 64 clouds of 32000); clouds of up to 16384 points need
+ * no workspace at any batch size. Calls no hipMalloc / hipFree. The first call on a GPU
+ * looks the array's address up (hipGetSymbolAddress), so make that call outside stream
+ * capture. All calls on one GPU share the array: calls that overlap in time on the same
+ * GPU (different streams or threads) race and must be serialised by the caller. */
+#define TK3D_FPS_STATIC_WORKSPACE_BYTES (8u << 20)
+int tk3d_sample_farthest_points_static_f32(const float *points, int64_t B, int64_t N,
+                                           int64_t num_samples, int64_t *index,
+                                           void *stream);
+
 /* Farthest point sampling on either point layout, optionally returning the sampled
  * coordinates as well. Fuses what the reference's models do around the op in
  * Python: sample_farthest_points(points, K, transpose=True) copies a [B,3,N] cloud

@@ -851,6 +851,36 @@ int fps(const T *points, bool soa, int64_t B, int64_t N, int64_t K, int64_t *ind
     return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
 }
 
+// Workspace of tk3d_sample_farthest_points_static_f32: lives in the library's device
+// image, one copy per GPU, for callers that cannot allocate. In host code the array's
+// name is only a handle for hipGetSymbolAddress; kernels are handed the address that
+// call returns for the current device.
+__device__ __align__(256) unsigned char fps_static_scratch[TK3D_FPS_STATIC_WORKSPACE_BYTES];
+
+// Device address of fps_static_scratch on the current device, looked up once per device.
+int fps_static_scratch_address(void **address)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<void *> known[MAX_DEVICES];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES)
+        return TK3D_ERR_UNSUPPORTED;
+    void *p = known[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(fps_static_scratch));
+        if (e != hipSuccess)
+            return (int)e;
+        if (!p)
+            return TK3D_ERR_WORKSPACE;
+        known[dev].store(p, std::memory_order_release);  // every thread finds the same value
+    }
+    *address = p;
+    return TK3D_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -875,6 +905,24 @@ int tk3d_sample_farthest_points_f32(const float *points, int64_t B, int64_t N,
 {
     return fps<float>(points, false, B, N, num_samples, index, nullptr, workspace,
                       workspace_bytes, stream);
+}
+
+int tk3d_sample_farthest_points_static_f32(const float *points, int64_t B, int64_t N,
+                                           int64_t num_samples, int64_t *index, void *stream)
+{
+    const size_t need = tk3d_sample_farthest_points_workspace_bytes(B, N, sizeof(float));
+    if (need > (size_t)TK3D_FPS_STATIC_WORKSPACE_BYTES)
+        return TK3D_ERR_WORKSPACE;
+    void *scratch = nullptr;
+    if (need > 0) {
+        const int rc = fps_static_scratch_address(&scratch);
+        if (rc != TK3D_OK)
+            return rc;
+    }
+    // Nothing in the workspace has to start at zero: the first step assigns every running
+    // minimum and each later step reads only what the step before it wrote.
+    return fps<float>(points, false, B, N, num_samples, index, nullptr, scratch,
+                      need > 0 ? (size_t)TK3D_FPS_STATIC_WORKSPACE_BYTES : 0, stream);
 }
 
 int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
