@@ -213,3 +213,113 @@ def test_slot_order_of_the_hand_worked_mink_run(cuda, k, dtype):
             want_i = torch.from_numpy(idx).to(cuda).expand(70, -1)
             assert torch.equal(got_d[0], want_d), "distances, m=%d tail=%d" % (m, tail)
             assert torch.equal(got_i[0], want_i), "indices, m=%d tail=%d" % (m, tail)
+
+
+# ---- many queries: the pre-filtered kernel. A cheaper score rules pairs out, candidates wait
+# in per-lane queues and are inserted later with the exact arithmetic. Whatever the input,
+# distances, indices and slot order must be MinK's: these cases aim at its error bound, its
+# queues, its stage boundaries and its fallbacks. (Sizes are chosen inside the range where
+# the dispatcher takes this kernel: 65536 queries or more against 2048 keys or more.) ----
+
+def _filter_case(kind, g, k):
+    b, n1, n2 = 8, 8192 + 5, 2048 + 37          # ragged: partial workgroup, partial chunk
+    q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
+    if kind == "uniform":
+        pass
+    elif kind == "lattice":                      # exact ties everywhere
+        q, key = lattice_cloud(g, b, n1, 4), lattice_cloud(g, b, n2, 4)
+    elif kind == "far_to_near":                  # every key is inserted: queues always full
+        r = torch.linspace(5.0, 0.1, n2)
+        key = torch.stack([r, torch.zeros_like(r), torch.zeros_like(r)], dim=1)[None].repeat(b, 1, 1)
+        key = key + 1e-4 * uniform_cloud(g, b, n2)
+        q = q * 0.01
+    elif kind == "near_to_far":                  # nothing after the fill is inserted
+        r = torch.linspace(0.1, 5.0, n2)
+        key = torch.stack([r, torch.zeros_like(r), torch.zeros_like(r)], dim=1)[None].repeat(b, 1, 1)
+        q = q * 0.01
+    elif kind == "far_from_origin":              # magnitude >> spacing: a loose bound
+        q, key = q + 1000.0, key + 1000.0
+    elif kind == "separated":                    # queries far from every key
+        q = q + 50.0
+    elif kind == "tiny":                         # squares underflow
+        q, key = q * 1e-20, key * 1e-20
+    elif kind == "huge":                         # squares overflow the bound's range
+        q, key = q * 1e18, key * 1e18
+    elif kind == "huge_queries":                 # only the queries are beyond the bound
+        q = q * 3e18
+    elif kind == "clusters":
+        centres = uniform_cloud(g, b, 8) * 100.0
+        def mk(n):
+            pick = torch.randint(0, 8, (b, n), generator=g)
+            return torch.gather(centres, 1, pick[:, :, None].expand(-1, -1, 3)) \
+                + 1e-3 * uniform_cloud(g, b, n)
+        q, key = mk(n1), mk(n2)
+    elif kind == "duplicates":                   # every distance of a query ties
+        key = uniform_cloud(g, b, 1).expand(b, n2, 3).contiguous()
+    elif kind == "nan_and_inf":
+        key[0, 0, 1] = float("nan")              # slot 0 of the fill: nothing is inserted later
+        key[1, min(k - 1, 2), 0] = float("nan")  # a later fill slot keeps its NaN
+        key[2, 700, 2] = float("nan")            # beyond the fill: never inserted
+        key[3, 1, 0] = float("inf")              # an infinite coordinate: exact fallback
+        key[4, 1500, 1] = -float("inf")
+        key[5, 512:700] = float("nan")           # a run across a stage boundary
+        q[6, 3, 2] = float("nan")
+        q[7, ::50] = float("inf")
+    else:
+        raise ValueError(kind)
+    return q.contiguous(), key.contiguous()
+
+
+@pytest.mark.parametrize("k", [1, 3, 4, 7, 16])
+@pytest.mark.parametrize("kind", ["uniform", "lattice", "far_to_near", "near_to_far",
+                                  "far_from_origin", "separated", "tiny", "huge", "huge_queries",
+                                  "clusters", "duplicates", "nan_and_inf"])
+def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
+    q, key = _filter_case(kind, gen(sum(map(ord, kind)) + k), k)
+    check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("b,n1,n2,k", [(4, 8192, 8192, 12),     # 32768 queries, long key cloud
+                                        (64, 4096, 1024, 2),     # 262144 queries, two stages
+                                        (128, 2048, 513, 3),     # one key into the second stage
+                                        (128, 2048, 512, 4),     # exactly one stage
+                                        (2, 70000, 2048, 5), (40, 4096, 4097, 9)])
+def test_prefiltered_kernel_shapes(cuda, b, n1, n2, k):
+    g = gen(n1 + n2 + k)
+    check_raw(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), k, cuda)
+
+
+def test_prefiltered_three_nn_on_both_layouts(cuda):
+    from torkit3d_amd.ops.interpolate_feature import three_nn_interpolation
+
+    g = gen(43)
+    q, key = uniform_cloud(g, 9, 8192 + 3), uniform_cloud(g, 9, 2048 + 1)
+    od, oi = oracle.knn(q.numpy(), key.numpy(), 3)
+    ow = oracle.three_nn_weights(od)
+    for transpose in (False, True):
+        a = q.to(cuda).transpose(1, 2).contiguous() if transpose else q.to(cuda)
+        c = key.to(cuda).transpose(1, 2).contiguous() if transpose else key.to(cuda)
+        d, i, w = three_nn_interpolation(a, c, transpose)
+        np.testing.assert_array_equal(d.cpu().numpy(), od)
+        np.testing.assert_array_equal(i.cpu().numpy(), oi)
+        np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=3e-7, atol=0)
+
+
+@pytest.mark.parametrize("k", [3, 4, 5, 8, 16])
+def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
+    # the literal rows of tests/util.py again, now with enough queries (140000 copies) and
+    # keys (5000 far ones behind the run) for the dispatcher to take the pre-filtered kernel
+    from torkit3d_amd import _C
+    from util import MINK_STATES, mink_worked_example
+
+    for m in sorted(MINK_STATES):
+        key, dist, idx = mink_worked_example(m, k, np.float32)
+        far = np.zeros((1, 5000, 3), np.float32)
+        far[0, :, 0] = 50.0 + np.arange(5000) % 7
+        keys = torch.from_numpy(np.concatenate([key, far], 1)).to(cuda)
+        query = torch.zeros(1, 140000, 3, device=cuda)
+        got_d, got_i = _C.knn_distance_cuda(query, keys, k, 1)
+        want_d = torch.from_numpy(dist).to(cuda)
+        want_i = torch.from_numpy(idx).to(cuda)
+        assert bool((got_d[0] == want_d).all()), "distances, m=%d" % m
+        assert bool((got_i[0] == want_i).all()), "indices, m=%d" % m

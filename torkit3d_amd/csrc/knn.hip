@@ -160,18 +160,17 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_register_kernel(
 // candidate keys across all lanes. The sequence of insertions seen by one lane is
 // exactly MinK's, so the slot order is unchanged.
 
+// `skey` is KNN_STAGE * 4 floats of LDS, 16-byte aligned; the whole workgroup calls this
+// with query `qi` of batch `b` per lane (qi >= n1: the lane only helps staging).
 template <int KMAX, bool SOA, bool WEIGHTS>
-__global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
+__device__ __forceinline__ void knn_batched_body(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
-    float eps, int blocks_per_batch, int n1, int n2, int k)
+    float eps, int b, int qi, int n1, int n2, int k, float *skey)
 {
     constexpr int CHUNK = 32;
     static_assert(KNN_STAGE % CHUNK == 0, "a chunk must not straddle stages");
-    __shared__ __align__(16) float skey[KNN_STAGE * 4];
     const int tid = threadIdx.x;
-    const int b = blockIdx.x / blocks_per_batch;
-    const int qi = (blockIdx.x - b * blocks_per_batch) * KNN_BLOCK + tid;
     const bool active = qi < n1;
     const float *__restrict__ K = key + (int64_t)b * n2 * 3;
     float qx = 0, qy = 0, qz = 0;
@@ -356,6 +355,519 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
         if constexpr (WEIGHTS && KMAX >= 3) {  // k == 3
             const float d3[3] = {kd[0], kd[1], kd[2]};
             knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + qi) * 3);
+        }
+    }
+}
+
+template <int KMAX, bool SOA, bool WEIGHTS>
+__global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
+    float eps, int blocks_per_batch, int n1, int n2, int k)
+{
+    __shared__ __align__(16) float skey[KNN_STAGE * 4];
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qi = (blockIdx.x - b * blocks_per_batch) * KNN_BLOCK + threadIdx.x;
+    knn_batched_body<KMAX, SOA, WEIGHTS>(query, key, distance, index, weight, eps, b, qi, n1, n2,
+                                         k, skey);
+}
+
+// fp32, k <= 16, launches with many queries: pre-filtered sweep with deferred insertions.
+//
+// Two costs dominate the batched kernel above: its sweep spends 8 vector instructions per
+// pair (six for the canonical distance), and its insertion rounds run after every chunk
+// for as long as the slowest lane of the wave has candidates, most lanes idling.
+//
+// Sweep. As in the chamfer kernel, most pairs only need to be ruled out, which the score
+//     s(q,k) = |k'|^2 - 2 q'.k'      (k' = k - c, q' = q - c, c the centre of the key
+//                                      cloud's bounding box)
+// does with three fused multiply-adds: d2(q,k) = s + |q'|^2 up to rounding. A key can
+// only be inserted if its canonical distance is below the query's current maximum M, so
+// the sweep evaluates t = s - thr, thr = (M - |q'|^2) + slack, by starting the three fmas
+// from |k'|^2 - thr, and collects the sign bits of t: 5 instructions per pair. With
+// u = 2^-24, rho = |k'| + |q'|, R = (max|k'| + |q'|)^2:
+//     canonical d2 against the exact distance of the centred points   7.02 u rho^2
+//         (three rounded differences, a product and two fmas of non-negative terms,
+//          plus the rounding of k' and q' themselves)
+//     |k'|^2 as staged                                                 3 u |k'|^2
+//     |k'|^2 - thr and the three fmas: four roundings of partial sums
+//         bounded by R + |thr|                                         4.04 u (R + |thr|)
+//     thr itself: M - |q'|^2 and the added slack                      3 u (M + R)
+// With |thr| <= M + R the total is below 21.2 u R + 7.1 u M; the kernel uses
+// slack = 32 u R + 16 u M (+1e-37 against underflow), R from max|k'| and |q'| inflated by
+// 1e-6 for their own rounding. Every key with canonical d2 < M therefore has t < 0: the
+// sign bits are a superset of MinK's insertions. Queries or key clouds that are
+// non-finite or huge (where the bound means nothing) take every key as a candidate, or
+// the workgroup runs the exact batched sweep.
+//
+// Insertions. A candidate is re-evaluated with the canonical arithmetic and inserted
+// under MinK's strict test against the maximum as it stands then, in ascending key
+// order per query, so the slots go through exactly MinK's states. But insertion does not
+// follow every chunk: a lane keeps up to CAP non-empty chunk masks per query in a small
+// register queue and the wave runs a service step (every lane with a pending candidate
+// takes its first one) only while some lane holds T candidates or a full queue; the
+// rest waits for company. Deferring only makes M - and with it thr - a little stale,
+// i.e. admits more candidates, each rejected by the strict test when it is served.
+// Per 2048 keys a wave runs 68 steps at k = 3 and 145 at k = 16 instead of 142 and 253
+// rounds. Keys are centred and staged in LDS as (x', y', z', |k'|^2); a lane serves QPL
+// queries, so one LDS read feeds QPL pairs and the steps of its queries interleave.
+template <int KMAX, int QPL, bool SOA, bool WEIGHTS>
+__global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
+    float eps, int blocks_per_batch, int n1, int n2, int k)
+{
+    constexpr int BLOCK = KNN_BLOCK;
+    constexpr int NW = BLOCK / TK_WAVE;
+    constexpr int STAGE = 512;
+    constexpr int CHUNK = 32;
+    constexpr int CAP = 4;
+    constexpr int T = 6;
+    constexpr int PER = STAGE / BLOCK;
+    static_assert(STAGE % BLOCK == 0 && STAGE % CHUNK == 0, "stage shape");
+    static_assert(2 * STAGE * 4 * (int)sizeof(float) >= KNN_STAGE * 4 * (int)sizeof(float),
+                  "the staging buffers double as the exact sweep's stage");
+    // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
+    // the sweep runs into), then two of raw keys (x, y, z, 0) for the service steps.
+    constexpr int STAGING_FLOATS = 2 * STAGE * 4 + 32 + 2 * STAGE * 4;
+    constexpr int TRANSPOSE_FLOATS = NW * 2 * TK_WAVE * (KMAX + 1);  // see the end of the kernel
+    __shared__ __align__(16) float
+        skey[STAGING_FLOATS > TRANSPOSE_FLOATS ? STAGING_FLOATS : TRANSPOSE_FLOATS];
+    float4 *const sraw = reinterpret_cast<float4 *>(skey + 2 * STAGE * 4 + 32);
+    __shared__ float sred[NW][8];
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qblock = blockIdx.x - b * blocks_per_batch;
+    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
+    const float *__restrict__ Q = query + (int64_t)b * n1 * 3;
+    const float INF = __builtin_huge_valf();
+
+    // ---- bounding box of the key cloud -> centre; largest centred norm ----
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    for (int j = tid; j < n2; j += BLOCK) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const float v = knn_coord<SOA>(K, n2, j, a);
+            lo[a] = __builtin_fminf(lo[a], v);
+            hi[a] = __builtin_fmaxf(hi[a], v);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            lo[a] = __builtin_fminf(lo[a], __shfl_xor(lo[a], o));
+            hi[a] = __builtin_fmaxf(hi[a], __shfl_xor(hi[a], o));
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            sred[wave][a] = lo[a];
+            sred[wave][3 + a] = hi[a];
+        }
+    }
+    __syncthreads();
+    float cc[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float l = INF, h = -INF;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][a]);
+            h = __builtin_fmaxf(h, sred[w][3 + a]);
+        }
+        cc[a] = 0.5f * l + 0.5f * h;
+    }
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    float kmax2 = 0.0f;
+    for (int j = tid; j < n2; j += BLOCK) {
+        const float x = knn_coord<SOA>(K, n2, j, 0) - c0;
+        const float y = knn_coord<SOA>(K, n2, j, 1) - c1;
+        const float z = knn_coord<SOA>(K, n2, j, 2) - c2;
+        kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        kmax2 = __builtin_fmaxf(kmax2, __shfl_xor(kmax2, o));
+    if (lane == 0)
+        sred[wave][6] = kmax2;
+    __syncthreads();
+    kmax2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
+    const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
+                      (kmax2 < 1e30f);
+    if (!safe) {  // uniform over the workgroup
+#pragma unroll 1
+        for (int i = 0; i < QPL; ++i)
+            knn_batched_body<KMAX, SOA, WEIGHTS>(query, key, distance, index, weight, eps, b,
+                                                 (qblock * QPL + i) * BLOCK + tid, n1, n2, k,
+                                                 skey);
+        return;
+    }
+    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+
+    // ---- queries ----
+    float qx[QPL], qy[QPL], qz[QPL], ax[QPL], ay[QPL], az[QPL], qn[QPL], slack_r[QPL];
+    bool active[QPL], usable[QPL];
+    // Slots hold the bit patterns of the distances: squared distances are non-negative, so
+    // their patterns order as signed integers. A NaN can only enter during the fill (a later
+    // key must compare below the maximum) and MinK never selects such a slot as maximum
+    // unless it is slot 0, in which case it never inserts again: here a NaN slot holds the
+    // pattern of -inf (below everything) and is recomputed when the results are written, and
+    // a NaN in slot 0 freezes the query (maximum -inf: no key compares below it).
+    int kd[QPL][KMAX];
+    int ki[QPL][KMAX];
+    float max_key[QPL];
+    int max_idx[QPL];
+    unsigned nan_slots[QPL];
+    constexpr int NEG_INF_BITS = (int)0xff800000u;
+    // Pending chunk masks per query, oldest first (bit 31 = first key of the chunk), and
+    // the key index of bit 31 of each. Named members and no loops over the queue, so it
+    // stays in registers (an array indexed through a loop ends up in scratch memory).
+    static_assert(CAP == 4, "the queue is written out for four entries");
+    struct Pending {
+        unsigned m0, m1, m2, m3;
+        int b0, b1, b2, b3;
+    } pq[QPL];
+    int qlen[QPL], pending[QPL];
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+        const int qi = (qblock * QPL + i) * BLOCK + tid;
+        active[i] = qi < n1;
+        qx[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 0) : c0;
+        qy[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 1) : c1;
+        qz[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 2) : c2;
+        const float px = qx[i] - c0, py = qy[i] - c1, pz = qz[i] - c2;
+        ax[i] = -2.0f * px;
+        ay[i] = -2.0f * py;
+        az[i] = -2.0f * pz;
+        qn[i] = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px));
+        const float r = kmax + __builtin_sqrtf(qn[i]) * 1.000001f;
+        slack_r[i] = r * r * 1.9073486e-06f + 1e-37f;  // 32 u R
+        usable[i] = slack_r[i] < 1e30f;                  // false for NaN / inf / huge
+        // fill: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots stay at -inf
+        max_key[i] = 0.0f;
+        max_idx[i] = 0;
+        nan_slots[i] = 0u;
+        bool frozen = false;
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s) {
+            kd[i][s] = NEG_INF_BITS;
+            ki[i][s] = 0;
+            if (s < k) {  // uniform
+                const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0),
+                                                knn_coord<SOA>(K, n2, s, 1),
+                                                knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
+                const bool isnan = d != d;
+                kd[i][s] = isnan ? NEG_INF_BITS : __builtin_bit_cast(int, d);
+                ki[i][s] = s;
+                nan_slots[i] |= isnan ? (1u << s) : 0u;
+                frozen |= isnan && s == 0;
+                if (s == 0 || d > max_key[i]) {
+                    max_key[i] = d;
+                    max_idx[i] = s;
+                }
+            }
+        }
+        max_key[i] = frozen ? -INF : max_key[i];
+        pq[i] = Pending{0u, 0u, 0u, 0u, 0, 0, 0, 0};
+        qlen[i] = 0;
+        pending[i] = 0;
+    }
+
+    // One service step: every query with a pending candidate takes its first one. Written
+    // without branches so that the chains of a lane's queries interleave.
+    auto service = [&]() {
+        float4 raw[QPL];
+        int kj[QPL];
+        bool has[QPL];
+#pragma unroll
+        for (int i = 0; i < QPL; ++i) {
+            Pending &p = pq[i];
+            has[i] = qlen[i] > 0;
+            // (an empty queue has m0 == 0: the bit number is then meaningless, the address
+            // below stays inside the buffer and nothing is inserted)
+            const int bit = __builtin_clz(p.m0 | 1u);
+            kj[i] = p.b0 + bit;
+            // resident: candidates are never older than the previous stage (see below)
+            raw[i] = sraw[kj[i] & (2 * STAGE - 1)];
+            const unsigned rest = p.m0 & ~(0x80000000u >> bit);
+            const bool shift = has[i] && rest == 0u;
+            p.m0 = shift ? p.m1 : rest;
+            p.b0 = shift ? p.b1 : p.b0;
+            p.m1 = shift ? p.m2 : p.m1;
+            p.b1 = shift ? p.b2 : p.b1;
+            p.m2 = shift ? p.m3 : p.m2;
+            p.b2 = shift ? p.b3 : p.b2;
+            p.m3 = shift ? 0u : p.m3;
+            qlen[i] -= shift ? 1 : 0;
+            pending[i] -= has[i] ? 1 : 0;
+        }
+#pragma unroll
+        for (int i = 0; i < QPL; ++i) {
+            const float d = tk_dist2<float>(raw[i].x, raw[i].y, raw[i].z, qx[i], qy[i], qz[i]);
+            const bool ins = has[i] && d < max_key[i];  // MinK's strict test (mink.cuh:74)
+            const int dbits = __builtin_bit_cast(int, d);
+            // the key takes the slot of the maximum ...
+#pragma unroll
+            for (int s = 0; s < KMAX; ++s) {
+                const bool here = ins && s == max_idx[i];
+                kd[i][s] = here ? dbits : kd[i][s];
+                ki[i][s] = here ? kj[i] : ki[i][s];
+            }
+            // ... and the new maximum is the largest pattern: it stays in the written slot
+            // when nothing is strictly above the new key, otherwise it is the first slot
+            // holding the largest pattern ((top - 1 - bits) is negative exactly there; the
+            // sign bits shifted together put slot 0 in the highest position).
+            int t[KMAX];
+#pragma unroll
+            for (int s = 0; s < KMAX; ++s)
+                t[s] = kd[i][s];
+#pragma unroll
+            for (int n = KMAX; n > 1; n = (n + 2) / 3) {
+#pragma unroll
+                for (int j = 0; 3 * j < n; ++j) {
+                    int v = t[3 * j];
+                    if (3 * j + 1 < n)
+                        v = t[3 * j + 1] > v ? t[3 * j + 1] : v;
+                    if (3 * j + 2 < n)
+                        v = t[3 * j + 2] > v ? t[3 * j + 2] : v;
+                    t[j] = v;
+                }
+            }
+            const int top = t[0];
+            const unsigned below = (unsigned)top - 1u;
+            constexpr int GS = 4;
+            unsigned eq = 0u;
+#pragma unroll
+            for (int g0 = 0; g0 < KMAX; g0 += GS) {
+                unsigned part = 0u;
+#pragma unroll
+                for (int s = g0; s < g0 + GS; ++s)
+                    part = __builtin_amdgcn_alignbit(part, below - (unsigned)kd[i][s], 31);
+                eq = (eq << GS) | part;
+            }
+            // (eq | 1 keeps the count defined; eq is never 0 when it matters)
+            const int first_top = __builtin_clz(eq | 1u) - (32 - KMAX);
+            const int new_idx = top != dbits ? first_top : max_idx[i];
+            max_key[i] = ins ? __builtin_bit_cast(float, top) : max_key[i];
+            max_idx[i] = ins ? new_idx : max_idx[i];
+        }
+        // Keep the loop-carried state where it is: without this the register allocator
+        // rotates some forty values through copies on every step.
+#pragma unroll
+        for (int i = 0; i < QPL; ++i) {
+            asm volatile("" : "+v"(pq[i].m0), "+v"(pq[i].m1), "+v"(pq[i].m2), "+v"(pq[i].m3));
+            asm volatile("" : "+v"(pq[i].b0), "+v"(pq[i].b1), "+v"(pq[i].b2), "+v"(pq[i].b3));
+            asm volatile("" : "+v"(qlen[i]), "+v"(pending[i]), "+v"(max_key[i]), "+v"(max_idx[i]));
+#pragma unroll
+            for (int s = 0; s < KMAX; ++s)
+                asm volatile("" : "+v"(kd[i][s]), "+v"(ki[i][s]));
+        }
+    };
+    auto must_serve = [&]() {
+        bool need = false;
+#pragma unroll
+        for (int i = 0; i < QPL; ++i)
+            need |= pending[i] >= T || qlen[i] >= CAP;
+        return __builtin_amdgcn_ballot_w64(need) != 0;
+    };
+
+    // ---- sweep: keys centred and staged in two LDS buffers, one barrier per stage ----
+    const int nstages = (n2 + STAGE - 1) / STAGE;
+    float4 pre[PER], pre_raw[PER];
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int kj = st * STAGE + r * BLOCK + tid;
+            float4 e = make_float4(0.0f, 0.0f, 0.0f, INF);  // past the end: never a candidate
+            float4 w = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (kj < n2) {
+                w.x = knn_coord<SOA>(K, n2, kj, 0);
+                w.y = knn_coord<SOA>(K, n2, kj, 1);
+                w.z = knn_coord<SOA>(K, n2, kj, 2);
+                e.x = w.x - c0;
+                e.y = w.y - c1;
+                e.z = w.z - c2;
+                e.w = __builtin_fmaf(e.z, e.z, __builtin_fmaf(e.y, e.y, e.x * e.x));
+            }
+            pre[r] = e;
+            pre_raw[r] = w;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            reinterpret_cast<float4 *>(skey)[buf * STAGE + r * BLOCK + tid] = pre[r];
+            sraw[buf * STAGE + r * BLOCK + tid] = pre_raw[r];
+        }
+    };
+    __syncthreads();
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int st = 0; st < nstages; ++st) {
+        const int stage0 = st * STAGE;
+        if (st + 1 < nstages)
+            fetch(st + 1);
+        const float4 *sbuf = reinterpret_cast<const float4 *>(skey) + (st & 1) * STAGE;
+        const int left = n2 - stage0;
+        const int cnt = left < STAGE ? left : STAGE;
+        for (int c0k = 0; c0k < cnt; c0k += CHUNK) {
+            const int first = stage0 + c0k;  // key index of bit 31
+            float thr[QPL];
+            unsigned mask[QPL];
+#pragma unroll
+            for (int i = 0; i < QPL; ++i) {
+                thr[i] = (max_key[i] - qn[i]) + __builtin_fmaf(max_key[i], 9.5367432e-07f, slack_r[i]);
+                mask[i] = 0u;
+            }
+            const float4 *ck = sbuf + c0k;
+            // Groups of G keys: the next group is read from LDS before the current one is
+            // used, and the G scores of a query are independent chains.
+            constexpr int G = 4;
+            float4 cur[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                cur[g] = ck[g];
+#pragma unroll
+            for (int j = 0; j < CHUNK; j += G) {
+                float4 nxt[G];
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    nxt[g] = ck[j + G + g];  // runs into the next chunk / the pad at the end
+#pragma unroll
+                for (int i = 0; i < QPL; ++i) {
+                    float t[G];
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        t[g] = cur[g].w - thr[i];
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        t[g] = __builtin_fmaf(cur[g].z, az[i], t[g]);
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        t[g] = __builtin_fmaf(cur[g].y, ay[i], t[g]);
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        t[g] = __builtin_fmaf(cur[g].x, ax[i], t[g]);
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        mask[i] = __builtin_amdgcn_alignbit(mask[i],
+                                                            __builtin_bit_cast(unsigned, t[g]), 31);
+                }
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    cur[g] = nxt[g];
+            }
+            // Keys that do not exist, or that the fill phase took, are no candidates.
+            int vlo = k - first;
+            vlo = vlo < 0 ? 0 : (vlo > CHUNK ? CHUNK : vlo);
+            int vhi = cnt - c0k;
+            vhi = vhi > CHUNK ? CHUNK : vhi;
+            unsigned valid = (vlo >= CHUNK) ? 0u : (0xffffffffu >> vlo);
+            valid &= (vhi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> vhi);
+#pragma unroll
+            for (int i = 0; i < QPL; ++i) {
+                unsigned m = usable[i] ? mask[i] : 0xffffffffu;
+                m = active[i] ? (m & valid) : 0u;
+                const bool nz = m != 0u;
+                Pending &p = pq[i];
+                const int at = nz ? qlen[i] : -1;
+                p.m0 = at == 0 ? m : p.m0;
+                p.b0 = at == 0 ? first : p.b0;
+                p.m1 = at == 1 ? m : p.m1;
+                p.b1 = at == 1 ? first : p.b1;
+                p.m2 = at == 2 ? m : p.m2;
+                p.b2 = at == 2 ? first : p.b2;
+                p.m3 = at == 3 ? m : p.m3;
+                p.b3 = at == 3 ? first : p.b3;
+                qlen[i] += nz ? 1 : 0;
+                pending[i] += __builtin_popcount(m);
+            }
+            // (two steps per trip: the loop-carried state is copied between registers once
+            // per trip, some forty moves)
+            while (must_serve()) {
+                service();
+                if (!must_serve())
+                    break;
+                service();
+            }
+        }
+        if (st + 1 < nstages) {
+            // The next stage replaces the previous one in LDS: whatever is still pending
+            // from it is served first (the queue is in key order, so its head tells).
+            for (;;) {
+                bool old = false;
+#pragma unroll
+                for (int i = 0; i < QPL; ++i)
+                    old |= qlen[i] > 0 && pq[i].b0 < stage0;
+                if (!__builtin_amdgcn_ballot_w64(old))
+                    break;
+                service();
+            }
+            __syncthreads();  // every wave is done with the previous stage
+            stash((st + 1) & 1);
+        }
+        __syncthreads();
+    }
+    for (;;) {
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < QPL; ++i)
+            any |= qlen[i] > 0;
+        if (!__builtin_amdgcn_ballot_w64(any))
+            break;
+        service();
+    }
+
+    // ---- results: a wave's 64 queries own 64 * k consecutive output elements; the slots
+    // are transposed through LDS (row stride KMAX + 1: no bank conflicts) so that the
+    // stores are runs of consecutive elements instead of one element per k ----
+    __syncthreads();
+    constexpr int ROW = KMAX + 1;
+    float *const tbuf = skey + wave * (2 * TK_WAVE * ROW);  // values, then indices
+    int *const ibuf = reinterpret_cast<int *>(tbuf + TK_WAVE * ROW);
+    static_assert(NW * 2 * TK_WAVE * ROW == TRANSPOSE_FLOATS, "LDS for the transpose");
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+        const int q0 = (qblock * QPL + i) * BLOCK + wave * TK_WAVE;  // first query of the wave
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s) {
+            float d = __builtin_bit_cast(float, kd[i][s]);
+            if (s < k && ((nan_slots[i] >> s) & 1u))  // a NaN of the fill, still in its slot
+                d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                                    knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
+            kd[i][s] = __builtin_bit_cast(int, d);
+            tbuf[lane * ROW + s] = d;
+            ibuf[lane * ROW + s] = ki[i][s];
+        }
+        const int nvalid = n1 - q0 < TK_WAVE ? n1 - q0 : TK_WAVE;  // may be <= 0
+        const int total = nvalid * k;
+        float *od = distance + ((int64_t)b * n1 + q0) * k;
+        int64_t *oi = index + ((int64_t)b * n1 + q0) * k;
+#pragma unroll
+        for (int r = 0; r < KMAX; ++r) {
+            const int e = r * TK_WAVE + lane;
+            if (e < total) {
+                const int row = e / k;
+                const int col = e - row * k;
+                od[e] = tbuf[row * ROW + col];
+                oi[e] = (int64_t)ibuf[row * ROW + col];
+            }
+        }
+        if constexpr (WEIGHTS && KMAX >= 3) {  // k == 3
+            if (active[i]) {
+                const float d3[3] = {__builtin_bit_cast(float, kd[i][0]),
+                                     __builtin_bit_cast(float, kd[i][1]),
+                                     __builtin_bit_cast(float, kd[i][2])};
+                knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + q0 + lane) * 3);
+            }
         }
     }
 }
@@ -1175,6 +1687,36 @@ void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64
                            index, weight, eps, bpb, n1, n2, k);
 }
 
+// The pre-filtered kernel pays when the launch fills the chip with two queries per lane
+// and the key cloud is long enough to amortise its prologue (two passes over the keys per
+// workgroup); TK3D_ERR_UNSUPPORTED otherwise. Thresholds from timing it against the
+// kernels above on an MI355X for k = 1..16, 32768 to 524288 queries, 256 to 8192 keys:
+// 1.1-1.8 times faster inside them, 0.6-1.0 outside.
+inline bool knn_filter_pays(int64_t queries, int n2, int k)
+{
+    if (n2 >= 8192)
+        return queries >= 32768;
+    if (n2 >= 2048)
+        return queries >= (k <= 5 ? 65536 : 131072);
+    if (n2 >= 1024)
+        return queries >= 262144;
+    return n2 >= 512 && k <= 4 && queries >= 262144;
+}
+
+template <int KMAX, bool SOA, bool WEIGHTS>
+int knn_filter_launch(const float *query, const float *key, float *distance, int64_t *index,
+                      float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    constexpr int QPL = 2;
+    const int64_t bpb = ((int64_t)n1 + QPL * KNN_BLOCK - 1) / (QPL * KNN_BLOCK);
+    if (!knn_filter_pays(B * n1, n2, k) || B * bpb > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, QPL, SOA, WEIGHTS>), dim3((unsigned)(B * bpb)),
+                       dim3(KNN_BLOCK), 0, s, query, key, distance, index, weight, eps, (int)bpb,
+                       n1, n2, k);
+    return tk_launch_status();
+}
+
 template <typename T>
 int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t k,
         int version, T *distance, int64_t *index, void *stream)
@@ -1204,6 +1746,12 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
+        if constexpr (sizeof(T) == 4) {
+            const int rc = knn_filter_launch<4, false, false>(query, key, distance, index, nullptr,
+                                                              0.0f, B, n1, n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
         knn_launch<T, 4>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
     } else if constexpr (sizeof(T) == 4) {
         // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
@@ -1224,6 +1772,16 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
             // log gets all the spare LDS (1.15-1.5 times faster from 8192 keys on)
             const int rc = knn_tree_split_launch<32, 2, 896>(query, key, distance, index, B, n1,
                                                              n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
+        if (k <= 16) {
+            // many queries: pre-filtered sweep, slots in registers
+            const int rc =
+                k <= 8 ? knn_filter_launch<8, false, false>(query, key, distance, index, nullptr,
+                                                            0.0f, B, n1, n2, kk, s)
+                       : knn_filter_launch<16, false, false>(query, key, distance, index, nullptr,
+                                                             0.0f, B, n1, n2, kk, s);
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
@@ -1294,6 +1852,14 @@ int three_nn(const T *query, const T *key, bool channels_first, int64_t B, int64
                                                                  (int)N2, 3, s);
         if (rc != TK3D_ERR_UNSUPPORTED)
             return rc;
+        const int rf = channels_first
+                           ? knn_filter_launch<4, true, true>(query, key, distance, index, weight,
+                                                              (float)eps, B, (int)N1, (int)N2, 3, s)
+                           : knn_filter_launch<4, false, true>(query, key, distance, index, weight,
+                                                               (float)eps, B, (int)N1, (int)N2, 3,
+                                                               s);
+        if (rf != TK3D_ERR_UNSUPPORTED)
+            return rf;
     }
     if (channels_first)
         knn_launch<T, 4, true, true>(query, key, distance, index, B, (int)bpb, (int)N1, (int)N2,
