@@ -218,3 +218,67 @@ def test_points_at_infinity(cuda):
     pts[1, 900, 2] = float("inf")
     want = oracle.sample_farthest_points(pts.numpy(), 30)
     np.testing.assert_array_equal(run(pts, 30, cuda), want)
+
+
+# ---- 8193 to 16384 points, 2048 samples or more: the kernel that lays the points out by
+# region (Morton order) and skips the blocks a new centre cannot reach. The lane order is no
+# longer the reference's priority order there, so ties are resolved explicitly. ----
+
+def _region_cloud(kind, g, b, n):
+    if kind == "uniform":
+        return torch.rand(b, n, 3, generator=g)
+    if kind == "mixture":
+        return gaussian_mixture_cloud(g, b, n)
+    if kind == "lattice":            # ties for the maximum at almost every step
+        return lattice_cloud(g, b, n, 3)
+    if kind == "coarse_lattice":     # 27 positions: after 27 picks nothing lies away
+        return lattice_cloud(g, b, n, 2)
+    if kind == "two_far_copies":     # every maximum is held by two points, in different regions
+        half = torch.rand(b, n // 2, 3, generator=g)
+        pts = torch.cat([half, half + torch.tensor([4.0, 0.0, 0.0])], dim=1)
+        return torch.cat([pts[:, ::2], pts[:, 1::2]], dim=1).contiguous()
+    if kind == "half_duplicates":    # every point twice at the same place
+        half = torch.rand(b, n // 2, 3, generator=g)
+        return torch.cat([half, half], dim=1)
+    if kind == "line":               # degenerate boxes
+        pts = torch.zeros(b, n, 3)
+        pts[:, :, 0] = torch.rand(b, n, generator=g)
+        return pts
+    if kind == "shell":
+        u = torch.randn(b, n, 3, generator=g)
+        return u / u.norm(dim=2, keepdim=True)
+    if kind == "clusters":
+        centres = torch.rand(b, 64, 3, generator=g)
+        return centres[:, torch.randint(0, 64, (n,), generator=g)] + 1e-3 * torch.randn(b, n, 3, generator=g)
+    if kind == "far_from_origin":    # coarse float grid: many exact ties, huge offsets
+        return torch.rand(b, n, 3, generator=g) + 4096.0
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "mixture", "lattice", "coarse_lattice", "two_far_copies",
+                                  "half_duplicates", "line", "shell", "clusters", "far_from_origin"])
+def test_region_kernel_on_adversarial_clouds(cuda, kind):
+    g = gen(70)
+    pts = _region_cloud(kind, g, 2, 12000 if kind in ("uniform", "lattice") else 16384)
+    k = 2100
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
+
+
+@pytest.mark.parametrize("n,k,transpose", [(8193, 2048, False), (16384, 16384, False),
+                                           (10000, 2049, True), (16383, 4096, True)])
+def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
+    pts = torch.rand(2, n, 3, generator=gen(n + k))
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    dev = pts.transpose(1, 2).contiguous() if transpose else pts
+    np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
+
+
+def test_region_kernel_with_non_finite_points(cuda):
+    pts = torch.rand(3, 9000, 3, generator=gen(71))
+    pts[0, 7, 1] = float("nan")
+    pts[0, 4500] = float("nan")
+    pts[1, 100, 0] = float("inf")
+    pts[2, 0, 2] = float("nan")        # point 0 itself: every distance is NaN
+    k = 2048
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    np.testing.assert_array_equal(run(pts, k, cuda), want)

@@ -328,6 +328,32 @@ template <int P, int NODE> struct FpsWalk2 {
     }
 };
 
+// FpsWalk2 for a caller that keeps the point indices elsewhere: reports the leaf reached.
+template <int P, int NODE> struct FpsWalk3 {
+    static __device__ __forceinline__ void go(const int (&t)[2 * P], const float (&x)[P],
+                                              const float (&y)[P], const float (&z)[P], int wl,
+                                              int wmax, FpsPick &out, int &passed)
+    {
+        if constexpr (NODE >= P) {
+            constexpr int p = NODE - P;
+            out.x = read_lane(x[p], wl);
+            out.y = read_lane(y[p], wl);
+            out.z = read_lane(z[p], wl);
+            out.j = p;  // the leaf; the caller turns it into a point index
+        } else {
+            const int left = read_lane(t[2 * NODE], wl);
+            const int right = read_lane(t[2 * NODE + 1], wl);
+            if (left == wmax) {
+                passed = right > passed ? right : passed;
+                FpsWalk3<P, 2 * NODE>::go(t, x, y, z, wl, wmax, out, passed);
+            } else {
+                passed = left > passed ? left : passed;
+                FpsWalk3<P, 2 * NODE + 1>::go(t, x, y, z, wl, wmax, out, passed);
+            }
+        }
+    }
+};
+
 // fp32 kernel that takes up to MAXM selection steps per cross-wave exchange.
 //
 // A step's fixed cost (wave reduction, slot exchange, barrier: about 1000 clocks) is
@@ -495,6 +521,388 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
     }
 }
 
+// Position of point j in the reference's tie order: its thread's rank among the
+// bit-reversed thread ids times the points per thread, plus its turn within the thread.
+__device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
+{
+    const int t = j & (L.bs - 1);
+    const int r = (int)(__builtin_bitreverse32((unsigned)t) >> (32 - L.log2_bs));
+    return r * L.c + (j >> L.log2_bs);
+}
+
+// fp32 kernel for clouds of 4097 to 16384 points: the multi-step kernel above with the
+// points laid out by region, so that an update only visits the points a new centre can
+// reach.
+//
+// At 16 or 32 points per lane a step is dominated by the update of the running minima
+// (nine instructions per point and centre), and almost all of that work changes nothing:
+// every running minimum is at most tau, the value of the last exchange's first winner (it
+// was the largest of them all, and minima only shrink), so a centre can lower a point's
+// minimum only if it lies within sqrt(tau) of it - a ball that shrinks as the sampling
+// proceeds. Hence:
+//   * the prologue sorts the points along a Morton curve (bitonic sort of (code, index)
+//     in LDS) and cuts the sorted sequence into 32 regions; region R goes to wave R % 8
+//     as block R / 8 of the lanes' registers (P / 4 points per lane and block), so
+//     neighbouring regions sit in different waves, i.e. on different SIMDs;
+//   * every wave keeps the bounding boxes of its four blocks. Before an update, lane
+//     (m, q) evaluates the canonical distance from centre m to box q - the same rounded
+//     operations as tk_dist2 on the per-axis gaps, each of which is monotone, so the
+//     result is a lower bound of the canonical distance to every point of the box - and a
+//     block is updated only if that bound is below tau. Skipping is therefore exact: a
+//     skipped update would have changed no minimum.
+// On uniform clouds a centre reaches two to five of the 32 regions once a few hundred
+// points are selected, and the waves that own them update one block each, side by side.
+//
+// Ties. With this layout the lane order is no longer the reference's priority order
+// (see the top of the file), so equal maxima are resolved explicitly: a wave that holds
+// its maximum more than once picks the point with the lowest reference position (the
+// rare slow path below), the slots carry that position, and candidates with equal values
+// are ranked by it. The acceptance rules are those of fps_multistep_kernel_f32.
+template <int P, bool SOA, int MAXM>
+__global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__restrict__ points,
+                                                             int64_t *__restrict__ index,
+                                                             FpsLayout L)
+{
+    constexpr int NT = 512, NW = 8, NB = 4, PB = P / NB, S = NT * P, RS = TK_WAVE * PB;
+    static_assert(P % NB == 0 && (P & (P - 1)) == 0 && MAXM * NB <= TK_WAVE, "shape");
+    constexpr int F32_INF = 0x7f800000;
+    constexpr int F32_NEG1 = (int)0xbf800000;
+    extern __shared__ __align__(16) unsigned char fps_region_lds[];
+    unsigned long long *const keys = reinterpret_cast<unsigned long long *>(fps_region_lds);
+    __shared__ FpsSlot slots[2][8];
+    __shared__ float s_box[NW][NB][8];  // lo.xyz, hi.xyz of a wave's block
+    __shared__ float s_red[NW][8];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const float *__restrict__ pts = points + (int64_t)blockIdx.x * L.n * 3;
+    int64_t *__restrict__ out = index + (int64_t)blockIdx.x * L.k;
+    const float INF = __builtin_huge_valf();
+
+    // ---- bounding box of the cloud ----
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    for (int j = tid; j < L.n; j += NT) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const float v = fps_coord<SOA>(pts, L.n, j, a);
+            lo[a] = __builtin_fminf(lo[a], v);
+            hi[a] = __builtin_fmaxf(hi[a], v);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            lo[a] = __builtin_fminf(lo[a], __shfl_xor(lo[a], o));
+            hi[a] = __builtin_fmaxf(hi[a], __shfl_xor(hi[a], o));
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            s_red[wave][a] = lo[a];
+            s_red[wave][3 + a] = hi[a];
+        }
+    }
+    __syncthreads();
+    float origin[3], scale[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float l = INF, h = -INF;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            l = __builtin_fminf(l, s_red[w][a]);
+            h = __builtin_fmaxf(h, s_red[w][3 + a]);
+        }
+        origin[a] = l;
+        const float extent = h - l;
+        scale[a] = extent > 0.0f ? 1023.0f / extent : 0.0f;  // also 0 for NaN / inf extents
+    }
+
+    // ---- (Morton code, point) pairs, sorted; slots beyond the cloud sort last ----
+    auto spread = [](unsigned v) {  // 10 bits -> every third bit
+        v = (v | (v << 16)) & 0x030000ffu;
+        v = (v | (v << 8)) & 0x0300f00fu;
+        v = (v | (v << 4)) & 0x030c30c3u;
+        v = (v | (v << 2)) & 0x09249249u;
+        return v;
+    };
+    for (int e = tid; e < S; e += NT) {
+        unsigned code = 0x7fffffffu;
+        if (e < L.n) {
+            unsigned c3[3];
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                const float f = (fps_coord<SOA>(pts, L.n, e, a) - origin[a]) * scale[a];
+                // (a NaN or an out-of-range value lands in cell 0 or 1023: any order of the
+                // points is a valid layout)
+                const float g = __builtin_fminf(__builtin_fmaxf(f, 0.0f), 1023.0f);
+                c3[a] = (unsigned)(int)g;
+            }
+            code = spread(c3[0]) | (spread(c3[1]) << 1) | (spread(c3[2]) << 2);
+        }
+        keys[e] = ((unsigned long long)code << 32) | (unsigned)e;
+    }
+    __syncthreads();
+    for (int kk = 2; kk <= S; kk <<= 1) {
+        for (int jj = kk >> 1; jj > 0; jj >>= 1) {
+            for (int i = tid; i < S / 2; i += NT) {
+                const int a = ((i & ~(jj - 1)) << 1) | (i & (jj - 1));
+                const int b = a + jj;
+                const unsigned long long ka = keys[a], kb = keys[b];
+                const bool ascending = (a & kk) == 0;
+                if ((ka > kb) == ascending) {
+                    keys[a] = kb;
+                    keys[b] = ka;
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- this lane's points: block q, turn u <-> sorted rank (q*8 + wave) * RS + u*64 + lane.
+    // The point indices stay in the sorted list in LDS (32 registers less). ----
+    auto rank_of = [&](int in_lane, int p) {
+        return ((p / PB) * NW + wave) * RS + (p % PB) * TK_WAVE + in_lane;
+    };
+    float x[P], y[P], z[P];
+    int t[2 * P];  // t[P + p]: running minimum of point p (bits); t[1..P-1]: maxima
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int j = (int)(unsigned)keys[rank_of(lane, p)];
+        const bool ok = j < L.n;
+        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : 0.0f;
+        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : 0.0f;
+        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : 0.0f;
+        t[P + p] = ok ? F32_INF : F32_NEG1;
+    }
+    t[0] = 0;
+    // boxes of the wave's blocks (an empty block gets an empty box: never reached)
+#pragma unroll
+    for (int q = 0; q < NB; ++q) {
+        float bl[3] = {INF, INF, INF}, bh[3] = {-INF, -INF, -INF};
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+            const int p = q * PB + u;
+            const bool ok = t[P + p] == F32_INF;
+            const float v[3] = {x[p], y[p], z[p]};
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                bl[a] = __builtin_fminf(bl[a], ok ? v[a] : INF);
+                bh[a] = __builtin_fmaxf(bh[a], ok ? v[a] : -INF);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                bl[a] = __builtin_fminf(bl[a], __shfl_xor(bl[a], o));
+                bh[a] = __builtin_fmaxf(bh[a], __shfl_xor(bh[a], o));
+            }
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                s_box[wave][q][a] = bl[a];
+                s_box[wave][q][3 + a] = bh[a];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = P - 1; i >= 1; --i)  // later only the touched blocks' maxima are redone
+        t[i] = t[2 * i] > t[2 * i + 1] ? t[2 * i] : t[2 * i + 1];
+
+    int sel_j = 0;
+    float cx[MAXM], cy[MAXM], cz[MAXM];  // centres selected by the last exchange
+#pragma unroll
+    for (int m = 0; m < MAXM; ++m) {
+        cx[m] = fps_coord<SOA>(pts, L.n, 0, 0);
+        cy[m] = fps_coord<SOA>(pts, L.n, 0, 1);
+        cz[m] = fps_coord<SOA>(pts, L.n, 0, 2);
+    }
+    int nc = 1;
+    float tau = INF;  // every running minimum is at most this
+    if (tid == 0)
+        out[0] = 0;
+    __syncthreads();  // the boxes are written
+
+    int round = 0;
+    for (int it = 1; it < L.k; it += nc, ++round) {
+        // ---- which blocks can the centres reach? lane (m, q) = (lane / 4, lane % 4) ----
+        unsigned long long reach;
+        {
+            const int m = lane >> 2, q = lane & (NB - 1);
+            float mx = cx[0], my = cy[0], mz = cz[0];
+#pragma unroll
+            for (int mm = 1; mm < MAXM; ++mm) {
+                mx = m == mm ? cx[mm] : mx;
+                my = m == mm ? cy[mm] : my;
+                mz = m == mm ? cz[mm] : mz;
+            }
+            const float *box = s_box[wave][q];
+            const float gx = __builtin_fmaxf(__builtin_fmaxf(box[0] - mx, mx - box[3]), 0.0f);
+            const float gy = __builtin_fmaxf(__builtin_fmaxf(box[1] - my, my - box[4]), 0.0f);
+            const float gz = __builtin_fmaxf(__builtin_fmaxf(box[2] - mz, mz - box[5]), 0.0f);
+            const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
+            // (a NaN bound counts as reachable)
+            reach = __builtin_amdgcn_ballot_w64(m < nc && !(bound >= tau));
+        }
+        // bit m * 4 + q of `reach`: most blocks are reached by no centre at all, so the
+        // blocks are tested first and the centres only inside a reached block
+        unsigned touched = 0u;
+        constexpr unsigned long long EVERY_CENTRE = 0x111111111111111ull;  // bit 4 m, any m
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            if ((reach >> q) & EVERY_CENTRE) {  // uniform
+#pragma unroll
+                for (int m = 0; m < MAXM; ++m) {
+                    if ((reach >> (m * NB + q)) & 1ull) {  // uniform
+#pragma unroll
+                        for (int u = 0; u < PB; ++u) {
+                            const int p = q * PB + u;
+                            const float d =
+                                tk_dist2<float>(x[p], y[p], z[p], cx[m], cy[m], cz[m]);
+                            const int db = __builtin_bit_cast(int, d);
+                            t[P + p] = t[P + p] < db ? t[P + p] : db;
+                        }
+                    }
+                }
+                touched |= 1u << q;
+            }
+        }
+        // maxima of the touched blocks (node 4 + q is the root of block q), then the top
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            if ((touched >> q) & 1u) {  // uniform
+#pragma unroll
+                for (int width = PB / 2; width >= 1; width /= 2) {
+                    const int first = (NB + q) * width;
+#pragma unroll
+                    for (int i = first + width - 1; i >= first; --i)
+                        t[i] = t[2 * i] > t[2 * i + 1] ? t[2 * i] : t[2 * i + 1];
+                }
+            }
+        }
+        t[2] = t[4] > t[5] ? t[4] : t[5];
+        t[3] = t[6] > t[7] ? t[6] : t[7];
+        t[1] = t[2] > t[3] ? t[2] : t[3];
+        // Only points strictly above zero are candidates (the reference starts its
+        // scan from max_dist = 0 with strict '>').
+        const int best = t[1] > 0 ? t[1] : 0;
+        int wmax, second;
+        wave_top2_i32(best, wmax, second);  // second: over the other lanes
+        int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
+        FpsPick pick;
+        FpsWalk3<P, 1>::go(t, x, y, z, wl, wmax, pick, second);  // and inside lane wl
+        pick.j = (int)(unsigned)keys[rank_of(wl, pick.j)];         // leaf -> point
+        if (second == wmax && wmax > 0) {  // uniform
+            // The wave holds its maximum more than once: the reference takes the point with
+            // the lowest position in its own order.
+            int lane_pos = 0x7fffffff, lane_p = 0;
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const int pos = fps_position_of_point((int)(unsigned)keys[rank_of(lane, p)], L);
+                const bool take = t[P + p] == wmax && pos < lane_pos;
+                lane_pos = take ? pos : lane_pos;
+                lane_p = take ? p : lane_p;
+            }
+            int wave_pos = lane_pos;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const int other = __shfl_xor(wave_pos, o);
+                wave_pos = other < wave_pos ? other : wave_pos;
+            }
+            wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(lane_pos == wave_pos));
+            const int wp = read_lane(lane_p, wl);
+            float sx = x[0], sy = y[0], sz = z[0];
+#pragma unroll
+            for (int p = 1; p < P; ++p) {
+                if (wp == p) {  // uniform
+                    sx = x[p];
+                    sy = y[p];
+                    sz = z[p];
+                }
+            }
+            pick.x = read_lane(sx, wl);
+            pick.y = read_lane(sy, wl);
+            pick.z = read_lane(sz, wl);
+            pick.j = (int)(unsigned)keys[rank_of(wl, wp)];
+        }
+        const int buf = round & 1;
+        if (lane == 0) {
+            FpsSlot s;
+            s.val = wmax;
+            s.j = pick.j;
+            s.x = pick.x;
+            s.y = pick.y;
+            s.z = pick.z;
+            s.pad[0] = second;
+            s.pad[1] = fps_position_of_point(pick.j, L);
+            s.pad[2] = 0;
+            slots[buf][wave] = s;
+        }
+        __syncthreads();
+        // Every wave now works out, redundantly and without a serial chain, how many of
+        // the candidates are certain winners of the coming steps. Lane (a, b) = (lane / 8,
+        // lane % 8) relates candidate a to candidate b.
+        const int ca = lane >> 3, cb = lane & 7;
+        const FpsSlot A = slots[buf][ca], Bs = slots[buf][cb];
+        const int va = A.val, vb = Bs.val;
+        // b comes before a in the reference's order (larger value, then lower position)
+        const bool before = vb > va || (vb == va && Bs.pad[1] < A.pad[1]);
+        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bs.x, Bs.y, Bs.z);
+        // a survives b's selection: b's update leaves a's minimum alone, and b's wave
+        // holds nothing else at or above it
+        const bool survives = __builtin_bit_cast(int, dab) >= va && Bs.pad[0] < va;
+        const unsigned long long m_before = __builtin_amdgcn_ballot_w64(before);
+        const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(!before || survives);
+        const int rank = __builtin_popcount((unsigned)(m_before >> (8 * ca)) & 0xffu);
+        const bool all_fine = ((unsigned)(m_fine >> (8 * ca)) & 0xffu) == 0xffu && va > 0;
+        const unsigned long long fine = __builtin_amdgcn_ballot_w64(all_fine);
+        const int left = L.k - it;  // steps still wanted
+        unsigned long long row[MAXM];
+        int good = 0;               // ranks 0..good-1 passed
+        bool chain = true;
+#pragma unroll
+        for (int m = 0; m < MAXM; ++m) {
+            // the ranks are a permutation of the 8 slots, so every rank has its row
+            row[m] = __builtin_amdgcn_ballot_w64(rank == m);
+            chain = chain && (row[m] & fine) != 0ull && m < left;  // uniform
+            good += chain ? 1 : 0;
+        }
+        if (good > 0) {  // uniform
+            // the slots of all ranks are read together (one LDS round trip), then the
+            // accepted ones are kept
+            FpsSlot w[MAXM];
+#pragma unroll
+            for (int m = 0; m < MAXM; ++m)
+                w[m] = slots[buf][__builtin_ctzll(row[m]) >> 3];
+            int jsel = 0;  // lane m of the first wave: the point of rank m
+            tau = __builtin_bit_cast(float, w[0].val);  // the largest minimum of all
+#pragma unroll
+            for (int m = 0; m < MAXM; ++m) {
+                const bool keep = m < good;  // uniform
+                cx[m] = keep ? w[m].x : cx[m];
+                cy[m] = keep ? w[m].y : cy[m];
+                cz[m] = keep ? w[m].z : cz[m];
+                sel_j = keep ? w[m].j : sel_j;
+                jsel = (keep && lane == m) ? w[m].j : jsel;
+            }
+            if (tid < good)
+                out[it + tid] = (int64_t)jsel;
+            nc = good;
+        } else {
+            // No point lies away from the chosen set: the previous choice is emitted again,
+            // as the reference does. Every minimum is zero already: nothing is reachable.
+            if (tid == 0)
+                out[it] = (int64_t)sel_j;
+            nc = 1;
+            tau = 0.0f;
+        }
+    }
+}
+
 // Clouds that do not fit in one workgroup's registers: every selection step is one
 // launch of many workgroups per cloud. Step s first works out the point chosen by step
 // s - 1 from the candidates that step's workgroups left in the workspace (every workgroup
@@ -516,15 +924,6 @@ template <typename T> struct FpsWideArgs {
     int slice;           // points per workgroup
     int batch;           // B
 };
-
-// Position of point j in the reference's tie order: its thread's rank among the
-// bit-reversed thread ids times the points per thread, plus its turn within the thread.
-__device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
-{
-    const int t = j & (L.bs - 1);
-    const int r = (int)(__builtin_bitreverse32((unsigned)t) >> (32 - L.log2_bs));
-    return r * L.c + (j >> L.log2_bs);
-}
 
 // (value, position) pairs ordered by larger value, then lower position.
 template <typename T>
@@ -712,11 +1111,39 @@ void fps_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
     }
 }
 
+// Clouds of 4097 to 16384 points: the region kernel, then the same check for non-finite
+// coordinates as above.
+template <int P>
+int fps_region_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
+                          const FpsLayout &L, hipStream_t s)
+{
+    constexpr int MAXM = 6;
+    constexpr int LDS = 512 * P * 8;  // the sort's (code, point) pairs
+    if (soa) {
+        constexpr auto kernel = fps_region_kernel_f32<P, true, MAXM>;
+        const int allowed = tk_allow_dynamic_lds<kernel>(LDS);
+        if (allowed != TK3D_OK)
+            return allowed;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(512), LDS, s, points, index, L);
+        hipLaunchKernelGGL((fps_register_kernel<float, P, 512, true>), dim3((unsigned)B),
+                           dim3(512), 0, s, points, index, L, 1);
+    } else {
+        constexpr auto kernel = fps_region_kernel_f32<P, false, MAXM>;
+        const int allowed = tk_allow_dynamic_lds<kernel>(LDS);
+        if (allowed != TK3D_OK)
+            return allowed;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(512), LDS, s, points, index, L);
+        hipLaunchKernelGGL((fps_register_kernel<float, P, 512, false>), dim3((unsigned)B),
+                           dim3(512), 0, s, points, index, L, 1);
+    }
+    return TK3D_OK;
+}
+
 // fp32: (points per lane, lanes) by cloud size, from timing every shape on an
 // MI355X: two waves per SIMD (512 lanes) hide each other's reduction latency; more
 // waves only repeat the per-wave reduction.
-void fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
-                      const FpsLayout &L, int64_t npos, hipStream_t s)
+int fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
+                     const FpsLayout &L, int64_t npos, hipStream_t s)
 {
     if (npos <= 64 * 2)
         fps_launch_f32<2, 64>(points, soa, B, index, L, s);
@@ -730,8 +1157,14 @@ void fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
         fps_launch_f32<8, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 16)
         fps_launch_f32<16, 512>(points, soa, B, index, L, s);
+    else if (L.k >= 2048)
+        // The region kernel's sort costs about 0.15 ms per call, which the skipped updates
+        // repay once a few thousand points are sampled from more than 8192 (16384 -> 4096:
+        // 3.35 -> 2.9 ms; 16384 -> 512 would go from 0.52 to 0.61 ms).
+        return fps_region_launch_f32<32>(points, soa, B, index, L, s);
     else
         fps_launch_f32<32, 512>(points, soa, B, index, L, s);
+    return TK3D_OK;
 }
 
 // Coordinates of the picks: sampled[b, i, :] = points[b, index[b, i], :] in the layout of
@@ -798,7 +1231,9 @@ int fps(const T *points, bool soa, int64_t B, int64_t N, int64_t K, int64_t *ind
     const int64_t npos = (int64_t)L.bs * L.c;
     if (npos <= fps_register_capacity(sizeof(T))) {
         if constexpr (sizeof(T) == 4) {
-            fps_dispatch_f32(points, soa, B, index, L, npos, s);
+            const int rc = fps_dispatch_f32(points, soa, B, index, L, npos, s);
+            if (rc != TK3D_OK)
+                return rc;
             return fps_finish<T>(points, soa, B, N, K, index, sampled, s);
         }
         // Fewest points per lane that still covers the cloud: short serial chains.

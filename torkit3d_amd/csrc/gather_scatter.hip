@@ -362,15 +362,31 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
     __shared__ double s_scale[CGMAX];
     __shared__ float s_bound[CGMAX];
     __shared__ int s_finite, s_exceeded;
-    const int b = blockIdx.z;
-    // blockIdx.y = destination window * groups + channel group; a workgroup accumulates
-    // the destinations [d0, d0 + nr) of its channels (the whole row when it fits in LDS)
-    const int win = blockIdx.y / groups;
-    const int c0 = (blockIdx.y - win * groups) * cg;
+    // Workgroups are handed to the 8 XCDs round-robin by linear id. Every workgroup of a
+    // batch streams that batch's index and weight arrays, so each XCD takes a contiguous
+    // range of logical workgroups (batch slowest): a batch's arrays then come from HBM
+    // once and from one XCD's L2 afterwards, instead of once per XCD.
+    int b, by, bx;
+    {
+        const unsigned long long gx = gridDim.x, gyy = gridDim.y;
+        const unsigned long long total = gx * gyy * gridDim.z;
+        unsigned long long lin = blockIdx.x + gx * (blockIdx.y + gyy * blockIdx.z);
+        const unsigned long long per = total >> 3, full = per << 3;
+        if (lin < full)
+            lin = (lin & 7ull) * per + (lin >> 3);
+        const unsigned long long rest = lin / gx;
+        bx = (int)(lin - rest * gx);
+        by = (int)(rest % gyy);
+        b = (int)(rest / gyy);
+    }
+    // by = destination window * groups + channel group; a workgroup accumulates the
+    // destinations [d0, d0 + nr) of its channels (the whole row when it fits in LDS)
+    const int win = by / groups;
+    const int c0 = (by - win * groups) * cg;
     const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
     const int d0 = win * window;
     const int nr = (d0 + window < n1) ? window : n1 - d0;
-    const int64_t ps = (int64_t)blockIdx.x * seg_len;
+    const int64_t ps = (int64_t)bx * seg_len;
     const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
     for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
