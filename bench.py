@@ -17,7 +17,9 @@ already resident in HBM. The headline value is pair-distances per second,
   secondary     milliseconds for farthest point sampling, ball query, group
                 points (B=16, N=4096), the KNN / interpolation configuration and the
                 set-abstraction chain of the stress configuration, with the CPU
-                oracle's time for the same ops beside them.
+                oracle's time for the same ops beside them; a roofline object per op
+                (algorithmic bytes or FLOP of the launch over its measured duration);
+                and the shapes the reference's author profiled.
 
 Everything runs on one GPU; --gpus above 1 is refused.
 """
@@ -77,7 +79,7 @@ def cpu_baseline_chamfer(a, c, budget_s=12.0):
     oracle.chamfer_forward(a[:nb].numpy(), c[:nb].numpy())
     dt = time.perf_counter() - t0
     pairs = 2.0 * nb * n * c.shape[1]
-    return {
+    res = {
         "value": pairs / dt,
         "unit": "pair-dists/s",
         "cores": oracle.num_threads(),
@@ -85,6 +87,26 @@ def cpu_baseline_chamfer(a, c, budget_s=12.0):
         "sample": "oracle chamfer forward on the first %d of %d clouds (N=M=%d), %.2f s" % (
             nb, a.shape[0], n, dt),
     }
+    # The reference's own CPU path for this op is the brute-force PyTorch form its test
+    # checks the kernel against (tests/ops/test_chamfer_distance.py:8-31): timed here on
+    # one cloud pair, row-chunked so that the difference tensor fits in memory.
+    import torch
+
+    def torch_chamfer(x, y, rows=1024):
+        col = torch.full((y.shape[0],), float("inf"))
+        for r in range(0, x.shape[0], rows):
+            d = ((x[r:r + rows, None, :] - y[None, :, :]) ** 2).sum(-1)
+            d.min(dim=1)
+            col = torch.minimum(col, d.min(dim=0).values)
+
+    t0 = time.perf_counter()
+    torch_chamfer(a[0], c[0])
+    dt = time.perf_counter() - t0
+    res["torch_value"] = 2.0 * n * c.shape[1] / dt
+    res["torch_cores"] = torch.get_num_threads()
+    res["torch_sample"] = ("pure PyTorch brute force (the reference's test oracle) on 1 of %d "
+                           "clouds (N=M=%d), %.2f s" % (a.shape[0], n, dt))
+    return res
 
 
 def cpu_ms(fn, scale):
@@ -180,6 +202,18 @@ def cpu_torch_metrics(tensors):
     out["interpolate_fwd_B32_C128_ms"] = round(fwd * 32 / 4, 3)
     out["interpolate_bwd_ms"] = round(bwd * 32 / 4, 3)
     return out
+
+
+def op_roofline(bound, detail, work, ms, unit_work):
+    """Roofline object of one launch: `work` algorithmic bytes (bound "hbm") or FLOP
+    (bound "mfma": the compute class, here the fp32 vector ALUs) over `ms` milliseconds."""
+    if bound == "hbm":
+        achieved, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = work / (ms * 1e-3) / 1e12, FP32_VECTOR_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": bound, "bound_detail": detail, unit_work: work, "ms": round(ms, 5),
+            "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4)}
 
 
 def secondary_metrics(dev, steps, warmup, cpu):
@@ -325,6 +359,66 @@ def secondary_metrics(dev, steps, warmup, cpu):
     out["fps_B1_N262144_K512_ms"] = gpu_time_ms(
         lambda: _C.sample_farthest_points_cuda(big, 512), 3, 1)
     del big
+    # Small chamfer configuration, backward (B=2, N=M=1024).
+    _, j1, _, j2 = _C.chamfer_distance_forward_cuda(s1, s2)
+    sg1 = torch.randn(2, 1024, generator=g).to(dev)
+    sg2 = torch.randn(2, 1024, generator=g).to(dev)
+    out["chamfer_bwd_B2_N1024_ms"] = gpu_time_ms(
+        lambda: _C.chamfer_distance_backward_cuda(sg1, sg2, s1, s2, j1, j2), steps, warmup)
+
+    # The shapes the reference's author profiled (tests/ops/test_knn_distance.py:58-61,
+    # tests/ops/test_sample_farthest_points.py:74-76; no numbers were recorded there).
+    author = {}
+    g = torch.Generator().manual_seed(8)
+    for bb, n1, n2, kk in ((32, 2048, 8192, 32), (4, 512, 10000, 64), (4, 10000, 512, 3)):
+        aq = torch.randn(bb, n1, 3, generator=g).to(dev)
+        ak = torch.randn(bb, n2, 3, generator=g).to(dev)
+        author["knn_B%d_N%d_M%d_k%d_ms" % (bb, n1, n2, kk)] = gpu_time_ms(
+            lambda: _C.knn_distance_cuda(aq, ak, kk, 1), max(5, steps // 5), 3)
+    for bb, nn, kk in ((16, 8192, 2048), (4, 10000, 512)):
+        ap = torch.rand(bb, nn, 3, generator=g).to(dev)
+        author["fps_B%d_N%d_K%d_ms" % (bb, nn, kk)] = gpu_time_ms(
+            lambda: _C.sample_farthest_points_cuda(ap, kk), max(3, steps // 10), 1)
+
+    # Roofline per op: algorithmic work of one launch over its measured duration.
+    valu = "fp32 vector ALU, 8 FLOP per pair-distance (top-k upkeep not counted)"
+    roof = {
+        "fps_B16_N4096_K1024": dict(
+            op_roofline("hbm", "serial chain of 1023 selection steps: latency bound, neither "
+                        "roofline applies; bytes = points read once + indices written",
+                        16 * 4096 * 12 + 16 * 1024 * 8, out["fps_B16_N4096_K1024_ms"], "bytes"),
+            us_per_step=round(out["fps_B16_N4096_K1024_ms"] * 1e3 / 1023, 4),
+            flop=8 * 16 * 1023 * 4096),
+        "fps_B8_N16384_K4096": dict(
+            op_roofline("hbm", "serial chain of 4095 selection steps: latency bound",
+                        8 * 16384 * 12 + 8 * 4096 * 8, out["fps_B8_N16384_K4096_ms"], "bytes"),
+            us_per_step=round(out["fps_B8_N16384_K4096_ms"] * 1e3 / 4095, 4),
+            flop=8 * 8 * 4095 * 16384),
+        "ball_query_B16_N1024x4096_r0.2_k32": op_roofline(
+            "hbm", "5.2 MB per launch: launch and latency bound",
+            16 * (1024 + 4096) * 12 + 16 * 1024 * 32 * 8,
+            out["ball_query_B16_N1024x4096_r0.2_k32_ms"], "bytes"),
+        "group_fwd_B16_C64_N4096_to_1024x32": op_roofline(
+            "hbm", "", 16 * 64 * 4096 * 4 + 16 * 1024 * 32 * 8 + 16 * 64 * 1024 * 32 * 4,
+            out["group_fwd_B16_C64_N4096_to_1024x32_ms"], "bytes"),
+        "group_bwd": op_roofline(
+            "hbm", "", 16 * 64 * 4096 * 4 + 16 * 1024 * 32 * 8 + 16 * 64 * 1024 * 32 * 4,
+            out["group_bwd_ms"], "bytes"),
+        "knn_B32_N8192_M2048_k16": op_roofline(
+            "mfma", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k16_ms"], "flop"),
+        "knn_B32_N8192_M2048_k3": op_roofline(
+            "mfma", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k3_ms"], "flop"),
+        "interpolate_fwd_B32_C128": op_roofline(
+            "hbm", "", 32 * 128 * 2048 * 4 + 32 * 8192 * 3 * 12 + 32 * 128 * 8192 * 4,
+            out["interpolate_fwd_B32_C128_ms"], "bytes"),
+        "interpolate_bwd": op_roofline(
+            "hbm", "", 32 * 128 * 2048 * 4 + 32 * 8192 * 3 * 12 + 32 * 128 * 8192 * 4,
+            out["interpolate_bwd_ms"], "bytes"),
+        "chamfer_bwd_B32_N16384": op_roofline(
+            "hbm", "60 bytes per point", 60 * 2 * 32 * 16384,
+            out["chamfer_bwd_B32_N16384_ms"], "bytes"),
+    }
+
     # Fused callers against the composition of ops the reference's layers run.
     from torkit3d_amd import _fused
     from torkit3d_amd.ops.interpolate_feature import three_nn_weights as weights_of
@@ -373,6 +467,8 @@ def secondary_metrics(dev, steps, warmup, cpu):
     del graph
 
     res = {"gpu_ms": {k: round(v, 5) for k, v in out.items()},
+           "roofline": roof,
+           "reference_profile_shapes_ms": {k: round(v, 5) for k, v in author.items()},
            "fused_vs_unfused_ms": {k: round(v, 5) for k, v in fused.items()},
            "model_ms": model_metrics(dev, max(3, steps // 10))}
     if cpu:

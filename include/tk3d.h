@@ -103,6 +103,18 @@ int tk3d_knn_distance_f64(const double *query, const double *key, int64_t B,
                           int64_t N1, int64_t N2, int64_t k, int version,
                           double *distance, int64_t *index, void *stream);
 
+/* KNN on [B,3,N] clouds (query [B,3,N1], key [B,3,N2]), the layout the reference's
+ * models hold: knn_points(..., transpose=True) copies both clouds to [B,N,3] before the
+ * call (torkit3d/ops/knn_points.py:40-45). Same result as tk3d_knn_distance_* on the
+ * transposed clouds, without the copies, for k <= 64; returns TK3D_ERR_UNSUPPORTED
+ * (nothing launched) for larger k, where the caller copies as the reference does. */
+int tk3d_knn_distance_bcn_f32(const float *query, const float *key, int64_t B,
+                              int64_t N1, int64_t N2, int64_t k, int version,
+                              float *distance, int64_t *index, void *stream);
+int tk3d_knn_distance_bcn_f64(const double *query, const double *key, int64_t B,
+                              int64_t N1, int64_t N2, int64_t k, int version,
+                              double *distance, int64_t *index, void *stream);
+
 /* 3 nearest neighbours and their interpolation weights in one launch. Fuses what
  * FeatureInterpolator.forward does in Python (torkit3d/layers/pointnet2.py:125-130):
  * knn_points(query, key, 3), then 1/clamp(d2, min=eps), a sum and a division as

@@ -282,3 +282,10 @@ def test_region_kernel_with_non_finite_points(cuda):
     k = 2048
     want = oracle.sample_farthest_points(pts.numpy(), k)
     np.testing.assert_array_equal(run(pts, k, cuda), want)
+
+
+@pytest.mark.parametrize("b,n,k", [(16, 8192, 2048), (4, 10000, 512)])
+def test_shapes_the_reference_author_profiled(cuda, b, n, k):
+    # tests/ops/test_sample_farthest_points.py:74-76 (profile runs, no recorded result)
+    pts = torch.rand(b, n, 3, generator=gen(8))
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))

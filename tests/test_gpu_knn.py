@@ -323,3 +323,37 @@ def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
         want_i = torch.from_numpy(idx).to(cuda)
         assert bool((got_d[0] == want_d).all()), "distances, m=%d" % m
         assert bool((got_i[0] == want_i).all()), "indices, m=%d" % m
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("b,n1,n2,k", [(2, 700, 900, 3), (8, 8192 + 1, 2048 + 3, 4),   # pre-filtered
+                                        (2, 300, 1000, 7), (16, 8192, 2048, 16),        # pre-filtered
+                                        (2, 300, 1000, 16), (1, 100, 500, 33), (1, 64, 300, 64),
+                                        (1, 40, 200, 65)])                               # copies
+def test_channels_first_clouds_are_read_in_place(cuda, b, n1, n2, k, dtype):
+    # knn_points(transpose=True) on [B,3,N] clouds: same rows as on the [B,N,3] clouds
+    from torkit3d_amd import _fused
+    from torkit3d_amd.ops.knn_points import knn_points
+
+    g = gen(n1 + k)
+    q, key = uniform_cloud(g, b, n1).to(dtype), uniform_cloud(g, b, n2).to(dtype)
+    od, oi = oracle.knn(q.numpy(), key.numpy(), k)
+    qt = q.to(cuda).transpose(1, 2).contiguous()
+    kt = key.to(cuda).transpose(1, 2).contiguous()
+    d, i = knn_points(qt, kt, k, transpose=True)
+    np.testing.assert_array_equal(d.cpu().numpy(), od)
+    np.testing.assert_array_equal(i.cpu().numpy(), oi)
+    raw = _fused.knn_distance_bcn(qt, kt, k, 1)
+    assert (raw is None) == (k > 64)
+    if raw is not None:
+        assert torch.equal(raw[0], d) and torch.equal(raw[1], i)
+
+
+@pytest.mark.parametrize("b,n1,n2,k", [(32, 2048, 8192, 32), (4, 512, 10000, 64),
+                                        (4, 10000, 512, 3)])
+def test_shapes_the_reference_author_profiled(cuda, b, n1, n2, k):
+    # tests/ops/test_knn_distance.py:58-61 (profile runs, randn clouds, no recorded result)
+    g = gen(8)
+    q = torch.randn(b, n1, 3, generator=g)
+    key = torch.randn(b, n2, 3, generator=g)
+    check_raw(q, key, k, cuda)

@@ -15,6 +15,7 @@ from ._lib import i64, ptr, stream_of
 __all__ = [
     "sample_farthest_points_gather",
     "ball_query_bcn",
+    "knn_distance_bcn",
     "group_points_concat_forward",
     "group_points_concat_backward",
     "three_nn",
@@ -71,6 +72,30 @@ def ball_query_bcn(query, key, radius, max_neighbors):
                   ctypes.c_float(float(radius)), i64(max_neighbors), ptr(index),
                   stream_of(query))
     return index
+
+
+def knn_distance_bcn(query, key, k, version):
+    """query [B,3,N1], key [B,3,N2] -> [distance [B,N1,k], index [B,N1,k]]; equals
+    ``_C.knn_distance_cuda`` on the transposed clouds. Returns None when the library has
+    no kernel for this k on this layout (k > 64): the caller then copies to [B,N,3]."""
+    b, n1 = _cloud_dims("query", query, True)
+    b2, n2 = _cloud_dims("key", key, True)
+    _check_eq(b, b2, "key.size(0) == query.size(0)")
+    _check_same("query", query, "key", key)
+    k = int(k)
+    _check(n2 >= k, "Check failed: key.size(1) >= k (%d vs. %d)" % (n2, k))
+    _check(int(version) in (0, 1), "Invalid version")
+    _check(k >= 0, "k must be non-negative.")
+    if k > 64:
+        return None
+    with _lib.on_device_of(query):
+        distance = torch.empty((b, n1, k), dtype=query.dtype, device=query.device)
+        index = torch.empty((b, n1, k), dtype=torch.int64, device=query.device)
+        if k > 0:
+            _lib.call("tk3d_knn_distance_bcn", query, ptr(query), ptr(key), i64(b), i64(n1),
+                      i64(n2), i64(k), ctypes.c_int(int(version)), ptr(distance), ptr(index),
+                      stream_of(query))
+    return [distance, index]
 
 
 def group_points_concat_forward(feature, xyz, centre, index):

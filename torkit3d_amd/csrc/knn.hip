@@ -1822,6 +1822,61 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
     return tk_launch_status();
 }
 
+// KNN on [B,3,N] clouds with the kernels that read either layout (slots in registers):
+// k <= 64; TK3D_ERR_UNSUPPORTED beyond, where the caller copies to [B,N,3] instead.
+template <typename T>
+int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t k,
+            int version, T *distance, int64_t *index, void *stream)
+{
+    if (B < 0 || N1 < 0 || N2 < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (version != 0 && version != 1)
+        return TK3D_ERR_BAD_VERSION;
+    if (k <= 0 || k > N2)
+        return TK3D_ERR_BAD_K;
+    if (N1 > TK_MAX_I32 / 4 || N2 > TK_MAX_I32 / 4 || !tk_fits(TK_MAX_ELEMS, B, N1, k) ||
+        !tk_fits(TK_MAX_ELEMS, B, N2, 3) || k > 64)
+        return TK3D_ERR_UNSUPPORTED;
+    if (B * N1 == 0)
+        return TK3D_OK;
+    if (!query || !key || !distance || !index)
+        return TK3D_ERR_NULL_POINTER;
+    const int64_t bpb = (N1 + KNN_BLOCK - 1) / KNN_BLOCK;
+    if (B * bpb > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
+    if constexpr (sizeof(T) == 4) {
+        int rc = TK3D_ERR_UNSUPPORTED;
+        if (k <= 4) {
+            rc = knn_small_split_launch<true, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                     n1, n2, kk, s);
+            if (rc == TK3D_ERR_UNSUPPORTED)
+                rc = knn_filter_launch<4, true, false>(query, key, distance, index, nullptr, 0.0f,
+                                                       B, n1, n2, kk, s);
+        } else if (k <= 8) {
+            rc = knn_filter_launch<8, true, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                   n1, n2, kk, s);
+        } else if (k <= 16) {
+            rc = knn_filter_launch<16, true, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                    n1, n2, kk, s);
+        }
+        if (rc != TK3D_ERR_UNSUPPORTED)
+            return rc;
+    }
+    if (k <= 4)
+        knn_launch<T, 4, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+    else if (k <= 8)
+        knn_launch<T, 8, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+    else if (k <= 16)
+        knn_launch<T, 16, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+    else if (k <= 32)
+        knn_launch<T, 32, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+    else
+        knn_launch<T, 64, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+    return tk_launch_status();
+}
+
 // 3 nearest neighbours with the interpolation weights formed in the same kernel.
 template <typename T>
 int three_nn(const T *query, const T *key, bool channels_first, int64_t B, int64_t N1,
@@ -1888,6 +1943,20 @@ int tk3d_three_nn_f64(const double *query, const double *key, int channels_first
 {
     return three_nn<double>(query, key, channels_first != 0, B, N1, N2, eps, distance, index,
                             weight, stream);
+}
+
+int tk3d_knn_distance_bcn_f32(const float *query, const float *key, int64_t B, int64_t N1,
+                              int64_t N2, int64_t k, int version, float *distance,
+                              int64_t *index, void *stream)
+{
+    return knn_bcn<float>(query, key, B, N1, N2, k, version, distance, index, stream);
+}
+
+int tk3d_knn_distance_bcn_f64(const double *query, const double *key, int64_t B, int64_t N1,
+                              int64_t N2, int64_t k, int version, double *distance,
+                              int64_t *index, void *stream)
+{
+    return knn_bcn<double>(query, key, B, N1, N2, k, version, distance, index, stream);
 }
 
 int tk3d_knn_distance_f32(const float *query, const float *key, int64_t B, int64_t N1,

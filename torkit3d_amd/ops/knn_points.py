@@ -1,7 +1,7 @@
 """K nearest neighbours with distances (API of torkit3d/ops/knn_points.py)."""
 import torch
 
-from .. import _C
+from .. import _C, _fused
 from ._common import NoGradient, rows_of_points
 
 
@@ -12,6 +12,15 @@ class KNNDistanceFunction(NoGradient):
     @staticmethod
     def run(query_xyz, key_xyz, k, version):
         return _C.knn_distance_cuda(query_xyz, key_xyz, k, version)
+
+
+class KNNDistanceChannelsFirstFunction(NoGradient):
+    """The same on [B,3,N] clouds, read in place (the reference copies them to [B,N,3]
+    first, torkit3d/ops/knn_points.py:40-45)."""
+
+    @staticmethod
+    def run(query_xyz, key_xyz, k, version):
+        return _fused.knn_distance_bcn(query_xyz, key_xyz, k, version)
 
 
 def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False, version=1):
@@ -25,8 +34,12 @@ def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False
     distance). ``version`` selects between the reference's two kernels (0 or 1); here
     both values give the same result from the same kernel.
     """
-    clouds = [rows_of_points(c, transpose).contiguous() for c in (query, key)]
-    distance, index = KNNDistanceFunction.apply(*clouds, k, version)
+    if (transpose and k <= 64 and query.dim() == 3 and key.dim() == 3
+            and query.is_contiguous() and key.is_contiguous()):
+        distance, index = KNNDistanceChannelsFirstFunction.apply(query, key, k, version)
+    else:
+        clouds = [rows_of_points(c, transpose).contiguous() for c in (query, key)]
+        distance, index = KNNDistanceFunction.apply(*clouds, k, version)
     if sorted:
         distance, order = distance.sort(dim=2)
         index = index.gather(2, order)
