@@ -253,15 +253,9 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
 //     scalar branches (left child first = lowest position), and the leaf reached
 //     reads that point's coordinates from fixed registers - log2(P) steps, no
 //     per-point compares or select chains in the loop;
-//   * a wave publishes one 32-byte slot (value, runner-up, point, xyz); after the single
-//     barrier every wave loads the slots and decides by itself how many of the
-//     candidates are winners (see fps_multistep_kernel_f32).
-struct __align__(16) FpsSlot {
-    int val;  // bit pattern of the wave's maximum
-    int j;    // point index of the wave's candidate
-    float x, y, z;
-    int pad[3];  // pad[0]: the wave's second-largest minimum
-};
+//   * a wave publishes its candidate (xyz, value) and (runner-up, point) in LDS; after the
+//     single barrier every wave loads all candidates and decides by itself how many of
+//     them are winners (see fps_multistep_kernel_f32).
 
 struct FpsPick {
     float x, y, z;
@@ -370,6 +364,11 @@ template <int P, int NODE> struct FpsWalk3 {
 // every other point is at or below V_m by the sort, minima only shrink, and the
 // accepted winners drop to zero. The chain stops at the first candidate that fails;
 // on uniform clouds about 2.7 steps are taken per exchange.
+//
+// The check is a chain of dependent instructions issued by one wave, so its length in
+// instructions is its cost: conditions are single compares whose lane masks are combined
+// in scalar registers, and the accepted candidates never go back to LDS - the coming
+// update reads their coordinates with v_readlane from the lanes that already hold them.
 template <int P, int NT, bool SOA, int MAXM>
 __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__restrict__ points,
                                                                int64_t *__restrict__ index,
@@ -380,7 +379,8 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
     static_assert(NW <= 8, "the cross-wave step relates 8 x 8 candidates");
     constexpr int F32_INF = 0x7f800000;
     constexpr int F32_NEG1 = (int)0xbf800000;
-    __shared__ FpsSlot slots[2][8];
+    __shared__ float4 s_cand[2][8];  // a wave's candidate: x, y, z, running minimum (bits)
+    __shared__ int2 s_aux[2][8];     // the wave's second-largest minimum, the candidate's index
 
     const int tid = threadIdx.x;
     const int lane = tid & (TK_WAVE - 1);
@@ -405,37 +405,38 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
     }
     t[0] = 0;
 
-    int sel_j = 0;
-    float cx[MAXM], cy[MAXM], cz[MAXM];  // centres selected by the last exchange
-#pragma unroll
-    for (int m = 0; m < MAXM; ++m) {
-        cx[m] = fps_coord<SOA>(pts, L.n, 0, 0);
-        cy[m] = fps_coord<SOA>(pts, L.n, 0, 1);
-        cz[m] = fps_coord<SOA>(pts, L.n, 0, 2);
-    }
+    // Lane (a, b) = (lane / 8, lane % 8) relates candidate a to candidate b after an
+    // exchange. The centres of the coming update are the candidates of the lanes in
+    // `centres` (lane 8 a stands for candidate a); the first update is point 0.
+    const int ca = lane >> 3, cb = lane & 7;
+    float ax = fps_coord<SOA>(pts, L.n, 0, 0);
+    float ay = fps_coord<SOA>(pts, L.n, 0, 1);
+    float az = fps_coord<SOA>(pts, L.n, 0, 2);
+    unsigned long long centres = 1ull;
+    // the last point emitted is the candidate of lane ctz(last_mask) / 8, whose index that
+    // lane keeps in last_j; no mask: point 0
+    unsigned long long last_mask = 0ull;
+    int last_j = 0;
+    constexpr unsigned long long FIRST_OF_EIGHT = 0x0101010101010101ull;  // lanes b == 0
+    constexpr unsigned long long EARLIER = 0x7f3f1f0f07030100ull;         // lanes b < a
     int nc = 1;
     if (tid == 0)
         out[0] = 0;
     if (tid < 16 && (tid & 7) >= NW) {  // waves that do not exist never have a candidate
-        FpsSlot s;
-        s.val = F32_NEG1;
-        s.j = 0;
-        s.x = s.y = s.z = 0.0f;
-        s.pad[0] = s.pad[1] = s.pad[2] = 0;
-        slots[tid >> 3][tid & 7] = s;
+        s_cand[tid >> 3][tid & 7] = make_float4(0.0f, 0.0f, 0.0f, -1.0f);
+        s_aux[tid >> 3][tid & 7] = make_int2(0, 0);
     }
 
     int round = 0;
     for (int it = 1; it < L.k; it += nc, ++round) {
+        for (unsigned long long todo = centres; todo != 0ull; todo &= todo - 1) {  // uniform
+            const int l = __builtin_ctzll(todo);
+            const float sx = read_lane(ax, l), sy = read_lane(ay, l), sz = read_lane(az, l);
 #pragma unroll
-        for (int m = 0; m < MAXM; ++m) {
-            if (m < nc) {  // uniform
-#pragma unroll
-                for (int p = 0; p < P; ++p) {
-                    const float d = tk_dist2<float>(x[p], y[p], z[p], cx[m], cy[m], cz[m]);
-                    const int db = __builtin_bit_cast(int, d);
-                    t[P + p] = t[P + p] < db ? t[P + p] : db;
-                }
+            for (int p = 0; p < P; ++p) {
+                const float d = tk_dist2<float>(x[p], y[p], z[p], sx, sy, sz);
+                const int db = __builtin_bit_cast(int, d);
+                t[P + p] = t[P + p] < db ? t[P + p] : db;
             }
         }
 #pragma unroll
@@ -451,71 +452,66 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
         FpsWalk2<P, 1>::go(t, x, y, z, jv, wl, wmax, pick, second);  // and inside lane wl
         const int buf = round & 1;
         if (lane == 0) {
-            FpsSlot s;
-            s.val = wmax;
-            s.j = pick.j;
-            s.x = pick.x;
-            s.y = pick.y;
-            s.z = pick.z;
-            s.pad[0] = second;
-            s.pad[1] = s.pad[2] = 0;
-            slots[buf][wave] = s;
+            s_cand[buf][wave] = make_float4(pick.x, pick.y, pick.z, __builtin_bit_cast(float, wmax));
+            s_aux[buf][wave] = make_int2(second, pick.j);
         }
         __syncthreads();
         // Every wave now works out, redundantly and without a serial chain, how many of
-        // the candidates are certain winners of the coming steps. Lane (a, b) = (lane / 8,
-        // lane % 8) relates candidate a to candidate b.
-        const int ca = lane >> 3, cb = lane & 7;
-        const FpsSlot A = slots[buf][ca], Bs = slots[buf][cb];
-        const int va = A.val, vb = Bs.val;
-        // b comes before a in the reference's order (larger value, then lower position)
-        const bool before = vb > va || (vb == va && cb < ca);
-        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bs.x, Bs.y, Bs.z);
+        // the candidates are certain winners of the coming steps. All 64 lanes are active,
+        // so conditions are combined as lane masks in scalar registers.
+        const float4 A = s_cand[buf][ca], Bc = s_cand[buf][cb];
+        const int2 Bx = s_aux[buf][cb];  // the wave's second-largest minimum, its point
+        ax = A.x;
+        ay = A.y;
+        az = A.z;
+        const int va = __builtin_bit_cast(int, A.w), vb = __builtin_bit_cast(int, Bc.w);
+        // b comes before a in the reference's order: larger value, then lower position
+        // (waves hold ascending ranges of positions)
+        const unsigned long long m_before =
+            __builtin_amdgcn_ballot_w64(vb > va) | (__builtin_amdgcn_ballot_w64(vb == va) & EARLIER);
+        const unsigned long long m_live = __builtin_amdgcn_ballot_w64(va > 0);
+        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bc.x, Bc.y, Bc.z);
         // a survives b's selection: b's update leaves a's minimum alone, and b's wave
         // holds nothing else at or above it
-        const bool survives = __builtin_bit_cast(int, dab) >= va && Bs.pad[0] < va;
-        const unsigned long long m_before = __builtin_amdgcn_ballot_w64(before);
-        const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(!before || survives);
-        const int rank = __builtin_popcount((unsigned)(m_before >> (8 * ca)) & 0xffu);
-        const bool all_fine = ((unsigned)(m_fine >> (8 * ca)) & 0xffu) == 0xffu && va > 0;
-        const unsigned long long fine = __builtin_amdgcn_ballot_w64(all_fine);
-        // How many leading ranks passed (scalar work), then the winners' data: a
-        // v_readlane costs tens of clocks, so only accepted ranks are fetched.
+        const unsigned long long m_far =
+            __builtin_amdgcn_ballot_w64(__builtin_bit_cast(int, dab) >= va);
+        const unsigned long long m_alone = __builtin_amdgcn_ballot_w64(Bx.x < va);
+        const unsigned long long m_fine = ~m_before | (m_far & m_alone);
+        // byte a of a mask: candidate a against every b
+        const unsigned before_a =
+            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_before : (unsigned)(m_before >> 32),
+                                  (unsigned)(lane & 24), 8u);
+        const unsigned fine_a =
+            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_fine : (unsigned)(m_fine >> 32),
+                                  (unsigned)(lane & 24), 8u);
+        const int rank = __builtin_popcount(before_a);  // a permutation of the candidates
+        const unsigned long long fine = __builtin_amdgcn_ballot_w64(fine_a == 0xffu) & m_live;
+        // Lane (a, b) asks whether candidate a has rank b and passed; folding the bytes of
+        // that mask together gives, in bit b, whether the candidate of rank b passed.
+        unsigned long long passed = __builtin_amdgcn_ballot_w64(rank == cb) & fine;
+        passed |= passed >> 32;
+        passed |= passed >> 16;
+        passed |= passed >> 8;
         const int left = L.k - it;  // steps still wanted
-        unsigned long long row[MAXM];
-        int good = 0;               // ranks 0..good-1 passed
-        bool chain = true;
-#pragma unroll
-        for (int m = 0; m < MAXM; ++m) {
-            // the ranks are a permutation of the 8 slots, so every rank has its row
-            row[m] = __builtin_amdgcn_ballot_w64(rank == m);
-            chain = chain && (row[m] & fine) != 0ull && m < left;  // uniform
-            good += chain ? 1 : 0;
-        }
+        int good = __builtin_ctz(~(unsigned)passed | (1u << MAXM));  // ranks 0..good-1 passed
+        good = good < left ? good : left;
+        centres = __builtin_amdgcn_ballot_w64(rank < good) & FIRST_OF_EIGHT;
         if (good > 0) {  // uniform
-            int jsel = 0;  // lane m of the first wave: the point of rank m
-#pragma unroll
-            for (int m = 0; m < MAXM; ++m) {
-                if (m < good) {  // uniform
-                    // every lane reads the winner's slot (one broadcast LDS read; fetching
-                    // the four values from a lane's registers costs far more)
-                    const FpsSlot w = slots[buf][__builtin_ctzll(row[m]) >> 3];
-                    cx[m] = w.x;
-                    cy[m] = w.y;
-                    cz[m] = w.z;
-                    sel_j = w.j;
-                    jsel = lane == m ? sel_j : jsel;
-                }
+            if (wave == 0) {  // uniform
+                if (ca == cb && rank < good)
+                    out[it + rank] = (int64_t)Bx.y;
             }
-            if (tid < good)
-                out[it + tid] = (int64_t)jsel;
+            // the last point emitted, should the cloud run out of distinct points
+            last_mask = __builtin_amdgcn_ballot_w64(rank == good - 1);
+            last_j = Bx.y;
             nc = good;
         } else {
             // No point lies away from the chosen set: the previous choice is emitted again,
-            // as the reference does. Every minimum is zero already, so whatever centre the
-            // next update applies changes nothing.
+            // as the reference does. Every minimum is zero already: nothing is updated.
             if (tid == 0)
-                out[it] = (int64_t)sel_j;
+                out[it] = last_mask != 0ull
+                              ? (int64_t)read_lane(last_j, __builtin_ctzll(last_mask) >> 3)
+                              : (int64_t)0;
             nc = 1;
         }
     }
@@ -569,7 +565,8 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
     constexpr int F32_NEG1 = (int)0xbf800000;
     extern __shared__ __align__(16) unsigned char fps_region_lds[];
     unsigned long long *const keys = reinterpret_cast<unsigned long long *>(fps_region_lds);
-    __shared__ FpsSlot slots[2][8];
+    __shared__ float4 s_cand[2][8];  // a wave's candidate: x, y, z, running minimum (bits)
+    __shared__ int2 s_aux[2][8];     // the wave's second-largest minimum, the candidate's rank
     __shared__ float s_box[NW][NB][8];  // lo.xyz, hi.xyz of a wave's block
     __shared__ float s_red[NW][8];
 
@@ -713,63 +710,60 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
     for (int i = P - 1; i >= 1; --i)  // later only the touched blocks' maxima are redone
         t[i] = t[2 * i] > t[2 * i + 1] ? t[2 * i] : t[2 * i + 1];
 
-    int sel_j = 0;
-    float cx[MAXM], cy[MAXM], cz[MAXM];  // centres selected by the last exchange
+    // From here on a point is named by its rank in the sorted list; the list is consulted
+    // only where a point index is needed (output, ties).
+    __syncthreads();  // the boxes are written
+    // Lane (a, b) = (lane / 8, lane % 8) relates candidate a to candidate b after an
+    // exchange; with b < 4 it also tests candidate a against the wave's block b, whose
+    // box it keeps in registers.
+    const int ca = lane >> 3, cb = lane & 7;
+    float box_lo[3], box_hi[3];
 #pragma unroll
-    for (int m = 0; m < MAXM; ++m) {
-        cx[m] = fps_coord<SOA>(pts, L.n, 0, 0);
-        cy[m] = fps_coord<SOA>(pts, L.n, 0, 1);
-        cz[m] = fps_coord<SOA>(pts, L.n, 0, 2);
+    for (int a = 0; a < 3; ++a) {
+        box_lo[a] = s_box[wave][cb & (NB - 1)][a];
+        box_hi[a] = s_box[wave][cb & (NB - 1)][3 + a];
     }
+    // The centres of the coming update are the candidates of the lanes in `centres`
+    // (lane 8 a stands for candidate a); bit 8 a + q of `reach` says whether candidate a
+    // can lower a minimum in block q. The first update is point 0 against every block.
+    float ax = fps_coord<SOA>(pts, L.n, 0, 0);
+    float ay = fps_coord<SOA>(pts, L.n, 0, 1);
+    float az = fps_coord<SOA>(pts, L.n, 0, 2);
+    unsigned long long centres = 1ull, reach = (1ull << NB) - 1;
+    // the last point emitted is the candidate of lane ctz(last_mask) / 8's sorted rank in
+    // last_rank; no mask: point 0
+    unsigned long long last_mask = 0ull;
+    int last_rank = 0;
+    constexpr unsigned long long DIAGONAL = 0x8040201008040201ull;        // lanes a == b
+    constexpr unsigned long long FIRST_OF_EIGHT = 0x0101010101010101ull;  // lanes b == 0
+    constexpr unsigned long long BLOCK_LANES = FIRST_OF_EIGHT * ((1u << NB) - 1);  // b < NB
     int nc = 1;
-    float tau = INF;  // every running minimum is at most this
     if (tid == 0)
         out[0] = 0;
-    __syncthreads();  // the boxes are written
 
     int round = 0;
     for (int it = 1; it < L.k; it += nc, ++round) {
-        // ---- which blocks can the centres reach? lane (m, q) = (lane / 4, lane % 4) ----
-        unsigned long long reach;
-        {
-            const int m = lane >> 2, q = lane & (NB - 1);
-            float mx = cx[0], my = cy[0], mz = cz[0];
-#pragma unroll
-            for (int mm = 1; mm < MAXM; ++mm) {
-                mx = m == mm ? cx[mm] : mx;
-                my = m == mm ? cy[mm] : my;
-                mz = m == mm ? cz[mm] : mz;
-            }
-            const float *box = s_box[wave][q];
-            const float gx = __builtin_fmaxf(__builtin_fmaxf(box[0] - mx, mx - box[3]), 0.0f);
-            const float gy = __builtin_fmaxf(__builtin_fmaxf(box[1] - my, my - box[4]), 0.0f);
-            const float gz = __builtin_fmaxf(__builtin_fmaxf(box[2] - mz, mz - box[5]), 0.0f);
-            const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
-            // (a NaN bound counts as reachable)
-            reach = __builtin_amdgcn_ballot_w64(m < nc && !(bound >= tau));
-        }
-        // bit m * 4 + q of `reach`: most blocks are reached by no centre at all, so the
-        // blocks are tested first and the centres only inside a reached block
+        // ---- running minima: only the blocks a centre can reach ----
         unsigned touched = 0u;
-        constexpr unsigned long long EVERY_CENTRE = 0x111111111111111ull;  // bit 4 m, any m
+        for (unsigned long long todo = centres; todo != 0ull; todo &= todo - 1) {  // uniform
+            const int l = __builtin_ctzll(todo);
+            const unsigned blocks = (unsigned)(reach >> l) & ((1u << NB) - 1);
+            if (blocks == 0u)
+                continue;
+            const float sx = read_lane(ax, l), sy = read_lane(ay, l), sz = read_lane(az, l);
 #pragma unroll
-        for (int q = 0; q < NB; ++q) {
-            if ((reach >> q) & EVERY_CENTRE) {  // uniform
+            for (int q = 0; q < NB; ++q) {
+                if ((blocks >> q) & 1u) {  // uniform
 #pragma unroll
-                for (int m = 0; m < MAXM; ++m) {
-                    if ((reach >> (m * NB + q)) & 1ull) {  // uniform
-#pragma unroll
-                        for (int u = 0; u < PB; ++u) {
-                            const int p = q * PB + u;
-                            const float d =
-                                tk_dist2<float>(x[p], y[p], z[p], cx[m], cy[m], cz[m]);
-                            const int db = __builtin_bit_cast(int, d);
-                            t[P + p] = t[P + p] < db ? t[P + p] : db;
-                        }
+                    for (int u = 0; u < PB; ++u) {
+                        const int p = q * PB + u;
+                        const float d = tk_dist2<float>(x[p], y[p], z[p], sx, sy, sz);
+                        const int db = __builtin_bit_cast(int, d);
+                        t[P + p] = t[P + p] < db ? t[P + p] : db;
                     }
                 }
-                touched |= 1u << q;
             }
+            touched |= blocks;
         }
         // maxima of the touched blocks (node 4 + q is the root of block q), then the top
 #pragma unroll
@@ -795,7 +789,7 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
         int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
         FpsPick pick;
         FpsWalk3<P, 1>::go(t, x, y, z, wl, wmax, pick, second);  // and inside lane wl
-        pick.j = (int)(unsigned)keys[rank_of(wl, pick.j)];         // leaf -> point
+        int pick_rank = rank_of(wl, pick.j);
         if (second == wmax && wmax > 0) {  // uniform
             // The wave holds its maximum more than once: the reference takes the point with
             // the lowest position in its own order.
@@ -827,78 +821,94 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
             pick.x = read_lane(sx, wl);
             pick.y = read_lane(sy, wl);
             pick.z = read_lane(sz, wl);
-            pick.j = (int)(unsigned)keys[rank_of(wl, wp)];
+            pick_rank = rank_of(wl, wp);
         }
         const int buf = round & 1;
         if (lane == 0) {
-            FpsSlot s;
-            s.val = wmax;
-            s.j = pick.j;
-            s.x = pick.x;
-            s.y = pick.y;
-            s.z = pick.z;
-            s.pad[0] = second;
-            s.pad[1] = fps_position_of_point(pick.j, L);
-            s.pad[2] = 0;
-            slots[buf][wave] = s;
+            s_cand[buf][wave] = make_float4(pick.x, pick.y, pick.z, __builtin_bit_cast(float, wmax));
+            s_aux[buf][wave] = make_int2(second, pick_rank);
         }
         __syncthreads();
         // Every wave now works out, redundantly and without a serial chain, how many of
-        // the candidates are certain winners of the coming steps. Lane (a, b) = (lane / 8,
-        // lane % 8) relates candidate a to candidate b.
-        const int ca = lane >> 3, cb = lane & 7;
-        const FpsSlot A = slots[buf][ca], Bs = slots[buf][cb];
-        const int va = A.val, vb = Bs.val;
-        // b comes before a in the reference's order (larger value, then lower position)
-        const bool before = vb > va || (vb == va && Bs.pad[1] < A.pad[1]);
-        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bs.x, Bs.y, Bs.z);
+        // the candidates are certain winners of the coming steps. All 64 lanes are active,
+        // so conditions are combined as lane masks in scalar registers.
+        const float4 A = s_cand[buf][ca], Bc = s_cand[buf][cb];
+        const int2 Bx = s_aux[buf][cb];  // the wave's second-largest minimum, sorted rank
+        ax = A.x;
+        ay = A.y;
+        az = A.z;
+        const int va = __builtin_bit_cast(int, A.w), vb = __builtin_bit_cast(int, Bc.w);
+        const unsigned long long m_above = __builtin_amdgcn_ballot_w64(vb > va);
+        const unsigned long long m_equal = __builtin_amdgcn_ballot_w64(vb == va);
+        const unsigned long long m_live = __builtin_amdgcn_ballot_w64(va > 0);
+        // b comes before a in the reference's order: larger value, then lower position.
+        // Positions are looked up only when two candidates really hold the same value.
+        unsigned long long m_before = m_above;
+        if ((m_equal & m_live & ~DIAGONAL) != 0ull) {  // uniform
+            const int rank_a = __shfl(Bx.y, ca);  // (lane a holds candidate a as its b)
+            const int pos_a = fps_position_of_point((int)(unsigned)keys[rank_a], L);
+            const int pos_b = fps_position_of_point((int)(unsigned)keys[Bx.y], L);
+            m_before |= m_equal & __builtin_amdgcn_ballot_w64(pos_b < pos_a);
+        }
+        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bc.x, Bc.y, Bc.z);
         // a survives b's selection: b's update leaves a's minimum alone, and b's wave
         // holds nothing else at or above it
-        const bool survives = __builtin_bit_cast(int, dab) >= va && Bs.pad[0] < va;
-        const unsigned long long m_before = __builtin_amdgcn_ballot_w64(before);
-        const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(!before || survives);
-        const int rank = __builtin_popcount((unsigned)(m_before >> (8 * ca)) & 0xffu);
-        const bool all_fine = ((unsigned)(m_fine >> (8 * ca)) & 0xffu) == 0xffu && va > 0;
-        const unsigned long long fine = __builtin_amdgcn_ballot_w64(all_fine);
+        const unsigned long long m_far =
+            __builtin_amdgcn_ballot_w64(__builtin_bit_cast(int, dab) >= va);
+        const unsigned long long m_alone = __builtin_amdgcn_ballot_w64(Bx.x < va);
+        const unsigned long long m_fine = ~m_before | (m_far & m_alone);
+        // byte a of a mask: candidate a against every b
+        const unsigned before_a =
+            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_before : (unsigned)(m_before >> 32),
+                                  (unsigned)(lane & 24), 8u);
+        const unsigned fine_a =
+            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_fine : (unsigned)(m_fine >> 32),
+                                  (unsigned)(lane & 24), 8u);
+        const int rank = __builtin_popcount(before_a);
+        const unsigned long long fine = __builtin_amdgcn_ballot_w64(fine_a == 0xffu) & m_live;
+        // Candidates above zero have distinct ranks. Lane (a, b) asks whether candidate a
+        // has rank b and passed; folding the bytes of that mask together gives, in bit b,
+        // whether the candidate of rank b passed.
+        unsigned long long passed = __builtin_amdgcn_ballot_w64(rank == cb) & fine;
+        passed |= passed >> 32;
+        passed |= passed >> 16;
+        passed |= passed >> 8;
         const int left = L.k - it;  // steps still wanted
-        unsigned long long row[MAXM];
-        int good = 0;               // ranks 0..good-1 passed
-        bool chain = true;
-#pragma unroll
-        for (int m = 0; m < MAXM; ++m) {
-            // the ranks are a permutation of the 8 slots, so every rank has its row
-            row[m] = __builtin_amdgcn_ballot_w64(rank == m);
-            chain = chain && (row[m] & fine) != 0ull && m < left;  // uniform
-            good += chain ? 1 : 0;
-        }
+        int good = __builtin_ctz(~(unsigned)passed | (1u << MAXM));  // ranks 0..good-1 passed
+        good = good < left ? good : left;
+        // Every running minimum is at most tau, the value of the first winner (the largest
+        // value has nobody before it); candidate a reaches block q only if the canonical
+        // distance from it to the block's box - rounded like tk_dist2, each operation
+        // monotone, hence a lower bound for every point of the box - is below tau. (A NaN
+        // bound counts as reachable.)
+        const float tau =
+            read_lane(A.w, __builtin_ctzll(__builtin_amdgcn_ballot_w64(rank == 0)));
+        const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
+        const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
+        const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
+        const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
+        reach = __builtin_amdgcn_ballot_w64(!(bound >= tau)) & BLOCK_LANES;
+        const unsigned long long m_taken = __builtin_amdgcn_ballot_w64(rank < good);
+        centres = m_taken & FIRST_OF_EIGHT;
         if (good > 0) {  // uniform
-            // the slots of all ranks are read together (one LDS round trip), then the
-            // accepted ones are kept
-            FpsSlot w[MAXM];
-#pragma unroll
-            for (int m = 0; m < MAXM; ++m)
-                w[m] = slots[buf][__builtin_ctzll(row[m]) >> 3];
-            int jsel = 0;  // lane m of the first wave: the point of rank m
-            tau = __builtin_bit_cast(float, w[0].val);  // the largest minimum of all
-#pragma unroll
-            for (int m = 0; m < MAXM; ++m) {
-                const bool keep = m < good;  // uniform
-                cx[m] = keep ? w[m].x : cx[m];
-                cy[m] = keep ? w[m].y : cy[m];
-                cz[m] = keep ? w[m].z : cz[m];
-                sel_j = keep ? w[m].j : sel_j;
-                jsel = (keep && lane == m) ? w[m].j : jsel;
+            if (wave == 0) {  // uniform
+                if (ca == cb && rank < good)
+                    out[it + rank] = (int64_t)(unsigned)keys[Bx.y];
             }
-            if (tid < good)
-                out[it + tid] = (int64_t)jsel;
+            // the last point emitted, should the cloud run out of distinct points
+            last_mask = __builtin_amdgcn_ballot_w64(rank == good - 1);
+            last_rank = Bx.y;
             nc = good;
         } else {
             // No point lies away from the chosen set: the previous choice is emitted again,
-            // as the reference does. Every minimum is zero already: nothing is reachable.
-            if (tid == 0)
-                out[it] = (int64_t)sel_j;
+            // as the reference does. Every minimum is zero already: nothing is updated.
+            if (tid == 0) {
+                int64_t j = 0;
+                if (last_mask != 0ull)
+                    j = (int64_t)(unsigned)keys[read_lane(last_rank, __builtin_ctzll(last_mask) >> 3)];
+                out[it] = j;
+            }
             nc = 1;
-            tau = 0.0f;
         }
     }
 }
