@@ -330,7 +330,7 @@ def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
                                         (2, 300, 1000, 7), (16, 8192, 2048, 16),        # pre-filtered
                                         (2, 300, 1000, 16), (1, 100, 500, 33), (1, 64, 300, 64),
                                         (1, 40, 200, 65)])                               # copies
-def test_channels_first_clouds_are_read_in_place(cuda, b, n1, n2, k, dtype):
+def test_channels_first_clouds_are_read_in_place_or_copied(cuda, b, n1, n2, k, dtype):
     # knn_points(transpose=True) on [B,3,N] clouds: same rows as on the [B,N,3] clouds
     from torkit3d_amd import _fused
     from torkit3d_amd.ops.knn_points import knn_points
@@ -344,7 +344,13 @@ def test_channels_first_clouds_are_read_in_place(cuda, b, n1, n2, k, dtype):
     np.testing.assert_array_equal(d.cpu().numpy(), od)
     np.testing.assert_array_equal(i.cpu().numpy(), oi)
     raw = _fused.knn_distance_bcn(qt, kt, k, 1)
-    assert (raw is None) == (k > 64)
+    # fp32: the library declines where its faster kernels only read [B,N,3] (k > 16, and
+    # k = 5..16 on launches too small for the pre-filtered sweep); fp64: k > 64 only
+    if dtype == torch.float64:
+        declined = k > 64
+    else:
+        declined = k > 16 or (k > 4 and not (b * n1 >= 131072 and n2 >= 2048))
+    assert (raw is None) == declined
     if raw is not None:
         assert torch.equal(raw[0], d) and torch.equal(raw[1], i)
 

@@ -76,8 +76,9 @@ def ball_query_bcn(query, key, radius, max_neighbors):
 
 def knn_distance_bcn(query, key, k, version):
     """query [B,3,N1], key [B,3,N2] -> [distance [B,N1,k], index [B,N1,k]]; equals
-    ``_C.knn_distance_cuda`` on the transposed clouds. Returns None when the library has
-    no kernel for this k on this layout (k > 64): the caller then copies to [B,N,3]."""
+    ``_C.knn_distance_cuda`` on the transposed clouds. Returns None when the library
+    declines this k and launch size on this layout (it has a faster kernel that reads
+    [B,N,3] only, or none at all for k > 64): the caller then copies to [B,N,3]."""
     b, n1 = _cloud_dims("query", query, True)
     b2, n2 = _cloud_dims("key", key, True)
     _check_eq(b, b2, "key.size(0) == query.size(0)")
@@ -91,10 +92,11 @@ def knn_distance_bcn(query, key, k, version):
     with _lib.on_device_of(query):
         distance = torch.empty((b, n1, k), dtype=query.dtype, device=query.device)
         index = torch.empty((b, n1, k), dtype=torch.int64, device=query.device)
-        if k > 0:
-            _lib.call("tk3d_knn_distance_bcn", query, ptr(query), ptr(key), i64(b), i64(n1),
-                      i64(n2), i64(k), ctypes.c_int(int(version)), ptr(distance), ptr(index),
-                      stream_of(query))
+        if k > 0 and not _lib.call("tk3d_knn_distance_bcn", query, ptr(query), ptr(key), i64(b),
+                                   i64(n1), i64(n2), i64(k), ctypes.c_int(int(version)),
+                                   ptr(distance), ptr(index), stream_of(query),
+                                   may_decline=True):
+            return None
     return [distance, index]
 
 

@@ -75,14 +75,23 @@ def fps_workspace_bytes(b, n, element_size):
     return int(_fps_workspace_fn(i64(b), i64(n), ctypes.c_size_t(element_size)))
 
 
-def call(name, tensor_for_dtype, *args):
+ERR_UNSUPPORTED = -6  # TK3D_ERR_UNSUPPORTED
+
+
+def call(name, tensor_for_dtype, *args, may_decline=False):
+    """Call ``name`` + the dtype suffix and raise on an error code. With ``may_decline`` a
+    TK3D_ERR_UNSUPPORTED return (nothing was launched) is handed back as False instead."""
     key = (name, tensor_for_dtype.dtype)
     fn = _functions.get(key)
     if fn is None:
         fn = getattr(lib(), name + suffix(tensor_for_dtype))
         fn.restype = ctypes.c_int
         _functions[key] = fn
-    check(fn(*args), name)
+    code = fn(*args)
+    if may_decline and code == ERR_UNSUPPORTED:
+        return False
+    check(code, name)
+    return True
 
 
 class _NoSwitch:

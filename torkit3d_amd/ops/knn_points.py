@@ -15,12 +15,17 @@ class KNNDistanceFunction(NoGradient):
 
 
 class KNNDistanceChannelsFirstFunction(NoGradient):
-    """The same on [B,3,N] clouds, read in place (the reference copies them to [B,N,3]
-    first, torkit3d/ops/knn_points.py:40-45)."""
+    """The same on [B,3,N] clouds, read in place where the library has a kernel for it (the
+    reference copies them to [B,N,3] first, torkit3d/ops/knn_points.py:40-45; so does this
+    for the k and launch sizes the library declines on this layout)."""
 
     @staticmethod
     def run(query_xyz, key_xyz, k, version):
-        return _fused.knn_distance_bcn(query_xyz, key_xyz, k, version)
+        result = _fused.knn_distance_bcn(query_xyz, key_xyz, k, version)
+        if result is None:
+            result = _C.knn_distance_cuda(query_xyz.transpose(1, 2).contiguous(),
+                                          key_xyz.transpose(1, 2).contiguous(), k, version)
+        return result
 
 
 def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False, version=1):
@@ -34,7 +39,7 @@ def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False
     distance). ``version`` selects between the reference's two kernels (0 or 1); here
     both values give the same result from the same kernel.
     """
-    if (transpose and k <= 64 and query.dim() == 3 and key.dim() == 3
+    if (transpose and query.dim() == 3 and key.dim() == 3
             and query.is_contiguous() and key.is_contiguous()):
         distance, index = KNNDistanceChannelsFirstFunction.apply(query, key, k, version)
     else:
