@@ -40,7 +40,7 @@ FLOP_PER_PAIR = 8                 # 3 sub, 3 mul, 2 add
 # HBM bytes per chamfer-forward launch at B=32, N=M=16384, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
 # (profiles/chamfer_forward_filter_B32_N16384.md).
-CHAMFER_TRAFFIC_BYTES = 39.9e6
+CHAMFER_TRAFFIC_BYTES = 40.0e6
 
 
 def sphere_cloud(gen, b, n, noise=0.01):
