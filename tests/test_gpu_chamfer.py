@@ -240,12 +240,11 @@ def test_sqrt_option(cuda):
 # bit-identical to the oracle: these cases aim at its error bound, its candidate
 # bookkeeping and its fallbacks.
 
-def _clouds(kind, g):
-    b, n1, n2 = 2, 1500, 3001
+def _clouds(kind, g, b=2, n1=1500, n2=3001):
     if kind == "lattice":            # exact ties everywhere: many candidate tiles
-        return lattice_cloud(g, b, 2048, 4), lattice_cloud(g, b, 2048, 4)
+        return lattice_cloud(g, b, max(n1, 2048), 4), lattice_cloud(g, b, max(n1, 2048), 4)
     if kind == "coarse_lattice":     # 27 distinct positions: every tile ties
-        return lattice_cloud(g, b, 1100, 2), lattice_cloud(g, b, 1300, 2)
+        return lattice_cloud(g, b, n1 - 400, 2), lattice_cloud(g, b, n1 - 200, 2)
     if kind == "duplicates":
         return uniform_cloud(g, b, n1), uniform_cloud(g, b, 1).expand(b, n2, 3).contiguous()
     if kind == "far_from_origin":    # magnitude >> spacing: the bound is loose
@@ -287,8 +286,22 @@ def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
     check_forward(a.contiguous(), c.contiguous(), cuda)
 
 
+# Launches of 512 workgroups or more on clouds of 2048 points or more run the pre-filter
+# on the matrix cores (scores from two-piece 16-bit splits of the coordinates): the same
+# inputs again at a batch size and cloud lengths that reach it.
+@pytest.mark.parametrize("kind", ["lattice", "coarse_lattice", "duplicates", "far_from_origin",
+                                  "separated", "wide_range", "tiny", "huge", "overflowing",
+                                  "clusters", "nan_and_inf", "all_nan_keys"])
+def test_matrix_prefilter_is_exact_on_hard_inputs(cuda, kind):
+    b, n1, n2 = 48, 2500, 3001
+    assert min(n1 - 400, n2) >= 2048 and b * ((n1 - 400 + 511) // 512 + (n2 + 511) // 512) >= 512
+    a, c = _clouds(kind, gen(sum(map(ord, kind)) + 1), b, n1, n2)
+    check_forward(a.contiguous(), c.contiguous(), cuda)
+
+
 @pytest.mark.parametrize("b,n1,n2", [(1, 1024, 1024), (2, 1025, 4097), (3, 8191, 1031),
-                                     (1, 20000, 1024), (64, 1024, 1100)])
+                                     (1, 20000, 1024), (64, 1024, 1100),
+                                     (64, 2049, 4100), (20, 6000, 7777), (512, 2048, 2048)])
 def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
     g = gen(n1 + n2)
     check_forward(sphere_cloud(g, b, n1), sphere_cloud(g, b, n2), cuda)

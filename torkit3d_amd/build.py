@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     "-ffp-contract=off",
     "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix instructions write ordinary vector registers (no copies out of the
+    # accumulation registers before the vector ALU can use a result)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall",
     "-Wno-unused-function",
 ]

@@ -647,6 +647,422 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     }
 }
 
+// ---- fp32 forward, pre-filter on the matrix cores --------------------------------
+//
+// The score s(q,k) = |k'|^2 - 2 q'.k' of the kernel above is a dot product, and the
+// pre-filter only has to be accurate to a stated bound, so it can run as a bf16 matrix
+// product with fp32 accumulation (v_mfma_f32_32x32x16_bf16: 32 keys x 32 queries x 16
+// terms in 32 clocks, against 3 x 2 clocks of vector FMAs per 64 pairs). Every centred
+// coordinate is split into two bf16 pieces, x = xh + xl + e with |e| <= 2^-17 |x|
+// (bf16 carries 8 significant bits: |x - xh| <= 2^-8 |x| to nearest, and xl, again to
+// nearest, is within 2^-9 of that; round to nearest even is done with integer arithmetic
+// below), and |k'|^2 into three. The 16 terms of a pair are
+//     key   : xh xh xl xl  yh yh yl yl  zh zh zl zl  n0 n1 n2 0
+//     query : Xh Xl Xh Xl  Yh Yl Yh Yl  Zh Zl Zh Zl  1  1  1  0      (X = -2 q'x, ...)
+// i.e. all four piece products of every coordinate plus |k'|^2. Products of two bf16
+// values are exact in fp32. With u = 2^-24, rho = |k'| + |q'|, R = (max|k'| + |q'|)^2:
+//     pieces dropped from 2 q'.k'   2 * 2^-17 * sum |x||X| <= 2^-15 |q'||k'| <=   128 u R
+//     |k'|^2 as staged, and its pieces                                             3.2 u R
+//     the matrix core's 16 additions, two units in the last place of the largest
+//         partial sum each (round to nearest would be half a unit; measured on this
+//         GPU: at most 11 u times the largest product)                              64 u R
+//     canonical d2 against the exact distance of the centred points               7.1 u R
+// so |s + |q'|^2 - canonical d2| <= E = 203 u R, and a key whose canonical distance
+// equals the minimum has s <= min(s) + 2 E. The kernel uses slack = 512 u R = 2^-15 R
+// (+1e-36 against underflow).
+//
+// Layout. In the 32 x 32 result a lane holds 16 keys (rows 8a + 4h + c, a, c < 4, h =
+// lane / 32) of one query (column lane % 32): lanes l and l + 32 serve the same query
+// on disjoint halves of the keys, each with its own three smallest group minima, and
+// their exact results are merged at the end (smaller distance, then lower index). A
+// wave keeps NQB blocks of 32 queries, so one LDS read of a key tile (16 bytes per
+// lane, conflict-free) feeds NQB matrix instructions. The vector ALU only folds the 16
+// results of an instruction into the running minimum (8 v_min3) and, every 4 tiles
+// (a group of 128 keys), updates the three smallest group minima as above.
+// A matrix instruction and its 8 v_min3 take 32 clocks each on a SIMD.
+//
+// Everything after the sweep is the scheme of the kernel above: at most two candidate
+// groups per half are re-evaluated with the canonical arithmetic in ascending key
+// order, three or more send the query to the exact scan, non-finite or huge input takes
+// the exact sweep. Results are bit-identical to the exact sweep for every input.
+typedef __bf16 tk_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float tk_f32x16 __attribute__((ext_vector_type(16)));
+
+// bf16 (as the upper half of a float's bits) nearest to x, ties to even; x finite.
+__device__ __forceinline__ unsigned chamfer_bf16_rne(float x)
+{
+    const unsigned bits = __builtin_bit_cast(unsigned, x);
+    return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float chamfer_bf16_value(unsigned b)
+{
+    return __builtin_bit_cast(float, b << 16);
+}
+// x = hi + lo + e, |e| <= 2^-17 |x|; returns hi | lo << 16.
+__device__ __forceinline__ unsigned chamfer_split2(float x)
+{
+    const unsigned hi = chamfer_bf16_rne(x);
+    const unsigned lo = chamfer_bf16_rne(x - chamfer_bf16_value(hi));  // the difference is exact
+    return hi | (lo << 16);
+}
+
+// The two 16-byte halves of a key's 16 terms. A key past the end gets |k'|^2 = +inf.
+__device__ __forceinline__ void chamfer_key_terms(float x, float y, float z, bool exists,
+                                                  uint4 &half0, uint4 &half1)
+{
+    const float n = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+    const unsigned sx = chamfer_split2(x), sy = chamfer_split2(y), sz = chamfer_split2(z);
+    const unsigned n0 = chamfer_bf16_rne(n);
+    const float r1 = n - chamfer_bf16_value(n0);
+    const unsigned n1 = chamfer_bf16_rne(r1);
+    const unsigned n2 = chamfer_bf16_rne(r1 - chamfer_bf16_value(n1));
+    const unsigned xh = sx & 0xffffu, xl = sx >> 16, yh = sy & 0xffffu, yl = sy >> 16;
+    const unsigned zh = sz & 0xffffu, zl = sz >> 16;
+    half0 = make_uint4(xh * 0x10001u, xl * 0x10001u, yh * 0x10001u, yl * 0x10001u);
+    half1 = make_uint4(zh * 0x10001u, zl * 0x10001u, n0 | (n1 << 16), n2);
+    if (!exists) {
+        half0 = make_uint4(0u, 0u, 0u, 0u);
+        half1 = make_uint4(0u, 0u, 0x7f80u, 0u);  // n0 = +inf
+    }
+}
+
+// The query side of the 16 terms for half h of the lanes (q' = centred query).
+__device__ __forceinline__ uint4 chamfer_query_terms(float qx, float qy, float qz, int h)
+{
+    const unsigned sx = chamfer_split2(-2.0f * qx), sy = chamfer_split2(-2.0f * qy);
+    const unsigned sz = chamfer_split2(-2.0f * qz);
+    return h == 0 ? make_uint4(sx, sx, sy, sy) : make_uint4(sz, sz, 0x3f803f80u, 0x00003f80u);
+}
+
+template <int NQB, int BLOCK, int STAGE>
+__global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
+{
+    constexpr int NW = BLOCK / TK_WAVE;
+    constexpr int QB = NW * NQB * 32;  // queries per workgroup
+    constexpr int GROUP = 128;         // keys per group: 4 tiles of 32
+    constexpr int TILES = STAGE / 32;
+    constexpr int PER = STAGE / BLOCK;
+    constexpr int MAX_SCANS = 96;
+    static_assert(STAGE % GROUP == 0 && STAGE % BLOCK == 0 && QB % BLOCK == 0, "shapes");
+    // Two stage buffers of key terms, [tile][half][key in tile] x 16 bytes; the exact
+    // sweep (the way out for input the bound does not cover) reuses them.
+    __shared__ __align__(16) uint4 sterm[2 * STAGE * 2];
+    static_assert(sizeof(uint4) * 2 * STAGE * 2 >= sizeof(float) * (512 * 4 + 8), "exact sweep stage");
+    __shared__ float sred[NW][8];
+    __shared__ int sidx[NW];
+    __shared__ int s_list[MAX_SCANS];
+    __shared__ int s_count;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int wave = tid / TK_WAVE;
+    const int col = lane & 31, half = lane >> 5;
+    int b, qblock, slice;
+    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
+    const int nq = d.nq;
+    const int k0 = slice * d.slice_len;
+    const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
+    const float *__restrict__ Q = d.query + (int64_t)b * nq * 3;
+    const float *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
+    const float INF = __builtin_huge_valf();
+
+    // ---- bounding box of the key cloud -> centre; largest centred squared norm ----
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    for (int j = tid; j < nk; j += BLOCK) {
+        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const float v[3] = {p.x, p.y, p.z};
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            lo[a] = __builtin_fminf(lo[a], v[a]);
+            hi[a] = __builtin_fmaxf(hi[a], v[a]);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        lo[a] = wave_reduce_min(lo[a]);
+        hi[a] = wave_reduce_max(hi[a]);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            sred[wave][a] = lo[a];
+            sred[wave][3 + a] = hi[a];
+        }
+    }
+    if (tid == 0)
+        s_count = 0;
+    __syncthreads();
+    float cc[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float l = INF, h = -INF;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][a]);
+            h = __builtin_fmaxf(h, sred[w][3 + a]);
+        }
+        cc[a] = 0.5f * l + 0.5f * h;
+    }
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    float kmax2 = 0.0f;
+    for (int j = tid; j < nk; j += BLOCK) {
+        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const float x = p.x - c0;
+        const float y = p.y - c1;
+        const float z = p.z - c2;
+        kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
+    }
+    kmax2 = wave_reduce_max(kmax2);
+    if (lane == 0)
+        sred[wave][6] = kmax2;
+    __syncthreads();
+    kmax2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
+    const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
+                      (kmax2 < 1e30f);
+    if (!safe) {  // uniform over the workgroup
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+            d, b, qblock, slice, reinterpret_cast<float *>(sterm));
+        return;
+    }
+    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+
+    // ---- queries: block g of the wave, column `col`; both halves of the lanes load it ----
+    tk_bf16x8 qterm[NQB];
+    float slack[NQB];
+    float v0[NQB], v1[NQB], v2[NQB];
+    int id0[NQB], id1[NQB];
+#pragma unroll
+    for (int g = 0; g < NQB; ++g) {
+        const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
+        const bool ok = qi < nq;
+        const float px = (ok ? Q[(int64_t)qi * 3 + 0] : c0) - c0;
+        const float py = (ok ? Q[(int64_t)qi * 3 + 1] : c1) - c1;
+        const float pz = (ok ? Q[(int64_t)qi * 3 + 2] : c2) - c2;
+        qterm[g] = __builtin_bit_cast(tk_bf16x8, chamfer_query_terms(px, py, pz, half));
+        // slack = 512 u (max|k'| + |q'|)^2: NaN / inf for a non-finite or huge query,
+        // which the epilogue tests for
+        const float qn =
+            1.000001f * __builtin_sqrtf(__builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px)));
+        const float r = kmax + qn;
+        slack[g] = r * r * 3.0517578e-05f + 1e-36f;
+        v0[g] = v1[g] = v2[g] = INF;
+        id0[g] = id1[g] = -1;
+    }
+
+    // ---- sweep ----
+    const int nstages = (nk + STAGE - 1) / STAGE;
+    float pre[PER][3];
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int kj = st * STAGE + r * BLOCK + tid;
+            pre[r][0] = pre[r][1] = pre[r][2] = 0.0f;
+            if (kj < nk) {
+                const TkPoint3<float> p = tk_load3<float>(K + (int64_t)kj * 3);
+                pre[r][0] = p.x;
+                pre[r][1] = p.y;
+                pre[r][2] = p.z;
+            }
+        }
+    };
+    auto stash = [&](int st, int buf) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int j = r * BLOCK + tid;  // key within the stage
+            uint4 h0, h1;
+            chamfer_key_terms(pre[r][0] - c0, pre[r][1] - c1, pre[r][2] - c2,
+                              st * STAGE + j < nk, h0, h1);
+            uint4 *tile = sterm + buf * (STAGE * 2) + (j >> 5) * 64 + (j & 31);
+            tile[0] = h0;
+            tile[32] = h1;
+        }
+    };
+    __syncthreads();
+    fetch(0);
+    stash(0, 0);
+    __syncthreads();
+    const tk_f32x16 zero = {};
+    for (int st = 0; st < nstages; ++st) {
+        if (st + 1 < nstages)
+            fetch(st + 1);
+        const uint4 *sbuf = sterm + (st & 1) * (STAGE * 2) + lane;
+        const int left = nk - st * STAGE;
+        const int cnt = left < STAGE ? left : STAGE;
+        const int ntiles = (cnt + GROUP - 1) / GROUP * (GROUP / 32);  // whole groups
+        float tmin[NQB];
+#pragma unroll
+        for (int g = 0; g < NQB; ++g)
+            tmin[g] = INF;
+        // The matrix instruction of the next step is issued before the minima of the
+        // current one are taken, so the wave does not wait for its result.
+        tk_bf16x8 ka = __builtin_bit_cast(tk_bf16x8, sbuf[0]);
+        tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qterm[0], zero, 0, 0, 0);
+#pragma unroll 4
+        for (int t = 0; t < ntiles; ++t) {
+            // (the read after the last tile wraps to tile 0: one wasted instruction)
+            const tk_bf16x8 kn =
+                __builtin_bit_cast(tk_bf16x8, sbuf[((t + 1) & (TILES - 1)) * 64]);
+#pragma unroll
+            for (int g = 0; g < NQB; ++g) {
+                const tk_f32x16 next =
+                    g + 1 < NQB
+                        ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qterm[g + 1 < NQB ? g + 1 : 0],
+                                                                   zero, 0, 0, 0)
+                        : __builtin_amdgcn_mfma_f32_32x32x16_bf16(kn, qterm[0], zero, 0, 0, 0);
+                float m = tmin[g];
+#pragma unroll
+                for (int r = 0; r < 16; r += 2)
+                    m = __builtin_fminf(__builtin_fminf(m, acc[r]), acc[r + 1]);
+                tmin[g] = m;
+                if ((t & 3) == 3) {
+                    // three smallest group minima (ties keep the earlier group in front)
+                    const int group_id = st * (STAGE / GROUP) + (t >> 2);
+                    const float x = m;
+                    const bool lt0 = x < v0[g];
+                    const bool lt1 = x < v1[g];
+                    id1[g] = lt1 ? group_id : id1[g];
+                    id1[g] = lt0 ? id0[g] : id1[g];
+                    id0[g] = lt0 ? group_id : id0[g];
+                    v2[g] = __builtin_amdgcn_fmed3f(v1[g], v2[g], x);
+                    v1[g] = __builtin_amdgcn_fmed3f(v0[g], v1[g], x);
+                    v0[g] = __builtin_amdgcn_fmed3f(-INF, v0[g], x);
+                    tmin[g] = INF;
+                }
+                acc = next;
+            }
+            ka = kn;
+        }
+
+        if (st + 1 < nstages) {
+            __syncthreads();  // (the other buffer was read during the previous stage)
+            stash(st + 1, (st + 1) & 1);
+        }
+        __syncthreads();
+
+        // One look, an eighth of the way in: if a quarter of the lanes already see three
+        // groups within the slack, the cloud is quantised and will not get better.
+        if (nstages >= 8 && st == (nstages >> 3)) {
+            int tied = 0;
+#pragma unroll
+            for (int g = 0; g < NQB; ++g) {
+                const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
+                const bool t3 = qi < nq && v2[g] <= v0[g] + slack[g];
+                tied += __builtin_popcountll(__builtin_amdgcn_ballot_w64(t3));
+            }
+            if (lane == 0)
+                atomicAdd(&s_count, tied);
+            __syncthreads();
+            const int total = s_count;
+            __syncthreads();
+            if (tid == 0)
+                s_count = 0;
+            if (total * 4 > 2 * QB) {  // uniform over the workgroup
+                chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+                    d, b, qblock, slice, reinterpret_cast<float *>(sterm));
+                return;
+            }
+        }
+    }
+
+    // ---- epilogue: exact evaluation of each half's candidate groups, then the merge ----
+    const bool k_aligned = (reinterpret_cast<uintptr_t>(K) & 15) == 0;  // runs of 4 keys: 48 B
+#pragma unroll 1
+    for (int g = 0; g < NQB; ++g) {
+        const int slot = (wave * NQB + g) * 32 + col;
+        const int qi = qblock * QB + slot;
+        const bool ok = qi < nq;
+        const float best_score = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
+        const float thr = best_score + slack[g];
+        const bool usable = slack[g] < 1e30f;  // false for NaN / inf / huge
+        // No finite score at all (nk == 0 or every key NaN): the exact result is (+inf, -1).
+        const bool none = !(best_score < INF);
+        const bool crowded = v2[g] <= thr;  // three or more candidate groups in this half
+        const bool over =
+            ok && !none && (!usable || __builtin_amdgcn_ballot_w64(crowded) >> col & 0x100000001ull);
+        float bestd = INF;
+        int bestj = -1;
+        if (ok && !none && !over) {
+            const float qx = Q[(int64_t)qi * 3 + 0], qy = Q[(int64_t)qi * 3 + 1],
+                        qz = Q[(int64_t)qi * 3 + 2];
+            int ta = v0[g] <= thr ? id0[g] : -1, tb = v1[g] <= thr ? id1[g] : -1;
+            if (tb >= 0 && tb < ta) {
+                const int tmp = ta;
+                ta = tb;
+                tb = tmp;
+            }
+            for (int pass = 0; pass < 2; ++pass) {
+                const int group = pass == 0 ? ta : tb;
+                if (group < 0)
+                    continue;
+                // this half's keys of the group: runs of 4 keys, 8 keys apart
+                for (int run = 0; run < GROUP / 8; ++run) {
+                    const int j = group * GROUP + run * 8 + half * 4;
+                    if (j >= nk)
+                        break;
+                    if (k_aligned && j + 4 <= nk) {
+                        const float4 *p4 = reinterpret_cast<const float4 *>(K + (int64_t)j * 3);
+                        const float4 f0 = p4[0], f1 = p4[1], f2 = p4[2];
+                        const float dd0 = tk_dist2<float>(f0.x, f0.y, f0.z, qx, qy, qz);
+                        const float dd1 = tk_dist2<float>(f0.w, f1.x, f1.y, qx, qy, qz);
+                        const float dd2 = tk_dist2<float>(f1.z, f1.w, f2.x, qx, qy, qz);
+                        const float dd3 = tk_dist2<float>(f2.y, f2.z, f2.w, qx, qy, qz);
+                        if (dd0 < bestd) { bestd = dd0; bestj = j; }
+                        if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
+                        if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
+                        if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
+                    } else {
+                        for (int e = j; e < j + 4 && e < nk; ++e) {
+                            const TkPoint3<float> p = tk_load3<float>(K + (int64_t)e * 3);
+                            const float dd = tk_dist2<float>(p.x, p.y, p.z, qx, qy, qz);
+                            if (dd < bestd) {
+                                bestd = dd;
+                                bestj = e;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // the other half's result: smaller distance, then lower key index
+        const float od = __shfl_xor(bestd, 32);
+        const int oj = __shfl_xor(bestj, 32);
+        if (oj >= 0 && (bestj < 0 || od < bestd || (od == bestd && oj < bestj))) {
+            bestd = od;
+            bestj = oj;
+        }
+        if (half == 0) {
+            if (ok && !over)
+                chamfer_emit<float>(d, b, qi, k0, bestd, bestj);
+            if (over) {
+                const int at = atomicAdd(&s_count, 1);
+                if (at < MAX_SCANS)
+                    s_list[at] = slot;
+            }
+        }
+    }
+
+    // ---- queries with three or more candidate groups in a half ----
+    __syncthreads();
+    const int nscan = s_count;
+    if (nscan > MAX_SCANS) {  // uniform over the workgroup
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+            d, b, qblock, slice, reinterpret_cast<float *>(sterm));
+        return;
+    }
+    for (int e = 0; e < nscan; ++e) {
+        const int qi = qblock * QB + s_list[e];
+        float bd;
+        int bj;
+        chamfer_block_exact_scan<BLOCK>(K, nk, Q[(int64_t)qi * 3 + 0], Q[(int64_t)qi * 3 + 1],
+                                        Q[(int64_t)qi * 3 + 2], &sred[0][0], sidx, bd, bj);
+        if (tid == 0)
+            chamfer_emit<float>(d, b, qi, k0, bd, bj);
+    }
+}
+
 // ---- backward ----------------------------------------------------------------
 // Pass A ("own" terms): every point i of cloud 1 has exactly one term
 // 2*gd1[i]*(x1[i]-x2[idx1[i]]) addressed to itself, so it is written with a plain
@@ -1092,6 +1508,21 @@ int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t 
                                       BLOCK, a, nblocks, B, stream);
 }
 
+template <int NQB, int BLOCK = 256, int STAGE = 512>
+int chamfer_forward_mfma_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
+                                int64_t N2, float *dist1, int64_t *idx1, float *dist2,
+                                int64_t *idx2, hipStream_t stream, int slices = 1)
+{
+    ChamferFwdArgs<float> a;
+    int64_t nblocks;
+    const int rc = chamfer_fill_args<float, (BLOCK / TK_WAVE) * NQB * 32, 128>(
+        a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, slices, nblocks);
+    if (rc != TK3D_OK)
+        return rc;
+    return chamfer_forward_run<float>(chamfer_forward_mfma_kernel<NQB, BLOCK, STAGE>, BLOCK, a,
+                                      nblocks, B, stream);
+}
+
 // Estimated duration in microseconds of the pre-filtered sweep launched as `qpl`
 // queries per lane, `block` lanes per workgroup and `want_slices` key slices; used only
 // to rank launch shapes. A wave issues qpl * ipp vector instructions per key (ipp per
@@ -1147,6 +1578,11 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
         // The pre-filter pays off once the key clouds are a few hundred points long
         // (its prologue passes over the keys twice per workgroup).
         const int64_t nkmin = N1 < N2 ? N1 : N2;
+        // Matrix-core pre-filter: 512 queries per workgroup; worth it once the launch
+        // fills the chip twice over and the key clouds are a few thousand points long.
+        if (nkmin >= 2048 && B * ((N1 + 511) / 512 + (N2 + 511) / 512) >= 512)
+            return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
+                                                  s);
         if (nkmin >= 512) {
             // Launch shapes: 4 queries per lane in 512-lane workgroups is the fastest
             // sweep once it fills the chip; below that 2 queries per lane in 256-lane
