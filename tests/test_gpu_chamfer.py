@@ -275,23 +275,49 @@ def _clouds(kind, g, b=2, n1=1500, n2=3001):
         return a, c
     if kind == "all_nan_keys":
         return uniform_cloud(g, b, n1), torch.full((b, n2, 3), float("nan"))
+    if kind == "scaled_small":       # inside the range the matrix pre-filter rescales
+        return uniform_cloud(g, b, n1) * 1e-9, uniform_cloud(g, b, n2) * 1e-9
+    if kind == "scaled_large":
+        return uniform_cloud(g, b, n1) * 3e9 + 1e9, uniform_cloud(g, b, n2) * 3e9 + 1e9
+    if kind == "outliers_off_sample":
+        # The matrix pre-filter places its centre and scale from every (n/1024)-th key;
+        # keys at positions the sample skips lie far outside what it saw: a few within
+        # the range of the 16-bit pieces, in batch 1 one beyond it.
+        a, c = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
+        for cloud in (a, c):
+            n = cloud.shape[1]
+            seen = set((i * n) // 1024 for i in range(1024))
+            skipped = [j for j in range(n) if j not in seen]
+            assert len(skipped) >= 3
+            cloud[:, skipped[0]] = torch.tensor([40.0, -3.0, 0.5])
+            cloud[:, skipped[len(skipped) // 2]] *= 100.0
+            cloud[1::2, skipped[-1], 1] = 3.0e4
+        return a, c
+    if kind == "far_queries":        # some queries beyond the range of the 16-bit pieces
+        a, c = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
+        a[:, ::97] *= 1.0e5
+        a[:, 5::211, 2] += 2.0e4
+        c[:, 7::301] += 7.0e6
+        return a, c
     raise ValueError(kind)
 
 
-@pytest.mark.parametrize("kind", ["lattice", "coarse_lattice", "duplicates", "far_from_origin",
-                                  "separated", "wide_range", "tiny", "huge", "overflowing",
-                                  "clusters", "nan_and_inf", "all_nan_keys"])
+HARD_KINDS = ["lattice", "coarse_lattice", "duplicates", "far_from_origin", "separated",
+              "wide_range", "tiny", "huge", "overflowing", "clusters", "nan_and_inf",
+              "all_nan_keys", "scaled_small", "scaled_large", "outliers_off_sample",
+              "far_queries"]
+
+
+@pytest.mark.parametrize("kind", HARD_KINDS)
 def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
     a, c = _clouds(kind, gen(sum(map(ord, kind))))
     check_forward(a.contiguous(), c.contiguous(), cuda)
 
 
 # Launches of 512 workgroups or more on clouds of 2048 points or more run the pre-filter
-# on the matrix cores (scores from two-piece 16-bit splits of the coordinates): the same
-# inputs again at a batch size and cloud lengths that reach it.
-@pytest.mark.parametrize("kind", ["lattice", "coarse_lattice", "duplicates", "far_from_origin",
-                                  "separated", "wide_range", "tiny", "huge", "overflowing",
-                                  "clusters", "nan_and_inf", "all_nan_keys"])
+# on the matrix cores (scores from two-piece fp16 splits of the centred, rescaled
+# coordinates): the same inputs again at a batch size and cloud lengths that reach it.
+@pytest.mark.parametrize("kind", HARD_KINDS)
 def test_matrix_prefilter_is_exact_on_hard_inputs(cuda, kind):
     b, n1, n2 = 48, 2500, 3001
     assert min(n1 - 400, n2) >= 2048 and b * ((n1 - 400 + 511) // 512 + (n2 + 511) // 512) >= 512
@@ -314,19 +340,22 @@ def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
 # lowest key index among equals, (inf, -1) without a finite distance.
 
 @pytest.mark.parametrize("b,n1,n2", [(1, 4096, 4096), (2, 3000, 5000), (1, 20000, 700),
-                                     (1, 777, 65536 + 5), (4, 512, 512), (1, 16384, 16384)])
+                                     (1, 777, 65536 + 5), (4, 512, 512), (1, 16384, 16384),
+                                     (1, 8192, 8192), (2, 16384, 9000), (1, 2048, 65536 + 5)])
 def test_split_sweep_shapes(cuda, b, n1, n2):
     g = gen(n1 * 3 + n2)
     check_forward(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), cuda)
 
 
-def test_split_sweep_ties_across_slices_keep_the_lowest_index(cuda):
+@pytest.mark.parametrize("n1,n2,spots", [
+    (2048, 8192, (100, 101, 3000, 3001, 8000, 8191)),        # vector pre-filter, sliced
+    (4096, 16384, (100, 101, 7000, 7001, 16000, 16383))])    # matrix pre-filter, sliced
+def test_split_sweep_ties_across_slices_keep_the_lowest_index(cuda, n1, n2, spots):
     from torkit3d_amd import _C
 
     g = gen(77)
-    a, c = uniform_cloud(g, 1, 2048), uniform_cloud(g, 1, 8192) + 5.0
+    a, c = uniform_cloud(g, 1, n1), uniform_cloud(g, 1, n2) + 5.0
     # The same three points sit in the first, a middle and the last part of the key cloud.
-    spots = (100, 101, 3000, 3001, 8000, 8191)
     for j in spots:
         c[0, j] = torch.tensor([0.25, -0.5, 0.125]) if j % 2 == 0 else torch.tensor([-0.5, 0.5, 0.75])
     c[0, 4000] = c[0, 100]
@@ -341,11 +370,13 @@ def test_split_sweep_ties_across_slices_keep_the_lowest_index(cuda):
         assert torch.equal(m[0], o[0]) and torch.equal(m[95], o[0])
 
 
-def test_split_sweep_with_slices_that_hold_no_finite_distance(cuda):
+@pytest.mark.parametrize("n1,n2", [(1500, 6000),       # vector pre-filter, sliced
+                                   (4096, 16384)])     # matrix pre-filter, sliced
+def test_split_sweep_with_slices_that_hold_no_finite_distance(cuda, n1, n2):
     g = gen(78)
-    a, c = uniform_cloud(g, 2, 1500), uniform_cloud(g, 2, 6000)
-    c[0, :2500] = float("nan")          # leading slices without a candidate
-    c[0, 5000:, 1] = float("inf")       # trailing slices at infinite distance
+    a, c = uniform_cloud(g, 2, n1), uniform_cloud(g, 2, n2)
+    c[0, :n2 * 5 // 12] = float("nan")          # leading slices without a candidate
+    c[0, n2 * 5 // 6:, 1] = float("inf")        # trailing slices at infinite distance
     c[1] = float("nan")                 # a cloud without any candidate: (inf, -1) everywhere
     a[0, 7] = float("nan")
     check_forward(a, c, cuda)

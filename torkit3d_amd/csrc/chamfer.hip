@@ -650,26 +650,38 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
 // ---- fp32 forward, pre-filter on the matrix cores --------------------------------
 //
 // The score s(q,k) = |k'|^2 - 2 q'.k' of the kernel above is a dot product, and the
-// pre-filter only has to be accurate to a stated bound, so it can run as a bf16 matrix
-// product with fp32 accumulation (v_mfma_f32_32x32x16_bf16: 32 keys x 32 queries x 16
-// terms in 32 clocks, against 3 x 2 clocks of vector FMAs per 64 pairs). Every centred
-// coordinate is split into two bf16 pieces, x = xh + xl + e with |e| <= 2^-17 |x|
-// (bf16 carries 8 significant bits: |x - xh| <= 2^-8 |x| to nearest, and xl, again to
-// nearest, is within 2^-9 of that; round to nearest even is done with integer arithmetic
-// below), and |k'|^2 into three. The 16 terms of a pair are
+// pre-filter only has to be accurate to a stated bound, so it can run as an fp16 matrix
+// product with fp32 accumulation (v_mfma_f32_32x32x16_f16: 32 keys x 32 queries x 16
+// terms in 32 clocks, against 3 x 2 clocks of vector FMAs per 64 pairs).
+//
+// Coordinates are centred on c and multiplied by a power of two 2^-e (exact), so that the
+// key cloud's extent is of order 1 and fp16's range is not an issue; c and e come from a
+// strided sample of 1024 keys and need not be accurate: the bound below uses the largest
+// centred norm of *all* keys, which the staging computes on the way, and input that leaves
+// the range (|k'| > 181, the extent's exponent outside [-40, 40], anything non-finite in
+// the sample) takes the exact sweep. From here on k', q' are the centred, scaled points.
+// Every coordinate is split into two fp16 pieces, x = xh + xl + e with |e| <= 2^-23 |x|
+// + 2^-25 (fp16 has 11 significant bits: |x - xh| <= 2^-11 |x| to nearest and xl, again
+// to nearest, is within 2^-12 of that, or within half the subnormal spacing 2^-24; the
+// matrix cores of this GPU take subnormal fp16 input as it is - measured, and flushing
+// would put errors of 2^-14 |X| into the scores of every uniform cloud, far beyond the
+// slack, so the parity tests on such clouds would fail), and |k'|^2 into
+// three. The 16 terms of a pair are
 //     key   : xh xh xl xl  yh yh yl yl  zh zh zl zl  n0 n1 n2 0
 //     query : Xh Xl Xh Xl  Yh Yl Yh Yl  Zh Zl Zh Zl  1  1  1  0      (X = -2 q'x, ...)
-// i.e. all four piece products of every coordinate plus |k'|^2. Products of two bf16
-// values are exact in fp32. With u = 2^-24, rho = |k'| + |q'|, R = (max|k'| + |q'|)^2:
-//     pieces dropped from 2 q'.k'   2 * 2^-17 * sum |x||X| <= 2^-15 |q'||k'| <=   128 u R
-//     |k'|^2 as staged, and its pieces                                             3.2 u R
-//     the matrix core's 16 additions, two units in the last place of the largest
-//         partial sum each (round to nearest would be half a unit; measured on this
-//         GPU: at most 11 u times the largest product)                              64 u R
+// i.e. all four piece products of every coordinate plus |k'|^2. Products of two fp16
+// values are exact in fp32. With u = 2^-24, R = (max|k'| + |q'|)^2:
+//     pieces dropped from 2 q'.k'    2 * 2^-23 * sum |x||X| <= 2^-21 |q'||k'| <=    2 u R
+//     subnormal pieces               2^-25 * (sum |X| + sum |x|)              <=      1 u R
+//     |k'|^2 as staged                                                            3.2 u R
+//     the matrix core's 16 additions, one unit in the last place of the largest
+//         partial sum each (round to nearest would be half a unit; measured on
+//         this GPU: at most 9.3 u times the largest product)                        32 u R
 //     canonical d2 against the exact distance of the centred points               7.1 u R
-// so |s + |q'|^2 - canonical d2| <= E = 203 u R, and a key whose canonical distance
-// equals the minimum has s <= min(s) + 2 E. The kernel uses slack = 512 u R = 2^-15 R
-// (+1e-36 against underflow).
+// so |s + |q'|^2 - canonical d2| <= E = 45.3 u R, and a key whose canonical distance
+// equals the minimum has s <= min(s) + 2 E. The kernel uses slack = 128 u R = 2^-17 R
+// (+ 1e-36 in the caller's units against underflow of the canonical distance).
+// A query beyond fp16's range (|q'| > 16000) goes to the exact scan.
 //
 // Layout. In the 32 x 32 result a lane holds 16 keys (rows 8a + 4h + c, a, c < 4, h =
 // lane / 32) of one query (column lane % 32): lanes l and l + 32 serve the same query
@@ -678,64 +690,74 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
 // wave keeps NQB blocks of 32 queries, so one LDS read of a key tile (16 bytes per
 // lane, conflict-free) feeds NQB matrix instructions. The vector ALU only folds the 16
 // results of an instruction into the running minimum (8 v_min3) and, every 4 tiles
-// (a group of 128 keys), updates the three smallest group minima as above.
-// A matrix instruction and its 8 v_min3 take 32 clocks each on a SIMD.
+// (a group of 128 keys), updates the three smallest group minima as above. A matrix
+// instruction and its 8 v_min3 take 32 clocks each on a SIMD and run side by side: the
+// loop issues the matrix instruction of the next step into a second set of result
+// registers before it folds the current set.
 //
 // Everything after the sweep is the scheme of the kernel above: at most two candidate
 // groups per half are re-evaluated with the canonical arithmetic in ascending key
-// order, three or more send the query to the exact scan, non-finite or huge input takes
-// the exact sweep. Results are bit-identical to the exact sweep for every input.
-typedef __bf16 tk_bf16x8 __attribute__((ext_vector_type(8)));
+// order, three or more send the query to the exact scan, non-finite or out-of-range input
+// takes the exact sweep. Results are bit-identical to the exact sweep for every input.
+typedef _Float16 tk_f16x8 __attribute__((ext_vector_type(8)));
 typedef float tk_f32x16 __attribute__((ext_vector_type(16)));
 
-// bf16 (as the upper half of a float's bits) nearest to x, ties to even; x finite.
-__device__ __forceinline__ unsigned chamfer_bf16_rne(float x)
+__device__ __forceinline__ unsigned chamfer_f16_bits(float x)  // nearest fp16
 {
-    const unsigned bits = __builtin_bit_cast(unsigned, x);
-    return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+    return (unsigned)__builtin_bit_cast(unsigned short, (_Float16)x);
 }
-__device__ __forceinline__ float chamfer_bf16_value(unsigned b)
+__device__ __forceinline__ float chamfer_f16_value(unsigned b)
 {
-    return __builtin_bit_cast(float, b << 16);
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)b);
 }
-// x = hi + lo + e, |e| <= 2^-17 |x|; returns hi | lo << 16.
+// x = hi + lo + e, |e| <= 2^-23 |x| + 2^-25; returns hi | lo << 16.
 __device__ __forceinline__ unsigned chamfer_split2(float x)
 {
-    const unsigned hi = chamfer_bf16_rne(x);
-    const unsigned lo = chamfer_bf16_rne(x - chamfer_bf16_value(hi));  // the difference is exact
+    const unsigned hi = chamfer_f16_bits(x);
+    const unsigned lo = chamfer_f16_bits(x - chamfer_f16_value(hi));  // the difference is exact
     return hi | (lo << 16);
 }
 
-// The two 16-byte halves of a key's 16 terms. A key past the end gets |k'|^2 = +inf.
-__device__ __forceinline__ void chamfer_key_terms(float x, float y, float z, bool exists,
+// The two 16-byte halves of a key's 16 terms; n = |k'|^2. A key past the end gets
+// |k'|^2 = +inf.
+__device__ __forceinline__ void chamfer_key_terms(float x, float y, float z, float n, bool exists,
                                                   uint4 &half0, uint4 &half1)
 {
-    const float n = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
     const unsigned sx = chamfer_split2(x), sy = chamfer_split2(y), sz = chamfer_split2(z);
-    const unsigned n0 = chamfer_bf16_rne(n);
-    const float r1 = n - chamfer_bf16_value(n0);
-    const unsigned n1 = chamfer_bf16_rne(r1);
-    const unsigned n2 = chamfer_bf16_rne(r1 - chamfer_bf16_value(n1));
+    const unsigned n0 = chamfer_f16_bits(n);
+    const float r1 = n - chamfer_f16_value(n0);
+    const unsigned n1 = chamfer_f16_bits(r1);
+    const unsigned n2 = chamfer_f16_bits(r1 - chamfer_f16_value(n1));
     const unsigned xh = sx & 0xffffu, xl = sx >> 16, yh = sy & 0xffffu, yl = sy >> 16;
     const unsigned zh = sz & 0xffffu, zl = sz >> 16;
     half0 = make_uint4(xh * 0x10001u, xl * 0x10001u, yh * 0x10001u, yl * 0x10001u);
     half1 = make_uint4(zh * 0x10001u, zl * 0x10001u, n0 | (n1 << 16), n2);
     if (!exists) {
         half0 = make_uint4(0u, 0u, 0u, 0u);
-        half1 = make_uint4(0u, 0u, 0x7f80u, 0u);  // n0 = +inf
+        half1 = make_uint4(0u, 0u, 0x7c00u, 0u);  // n0 = +inf
     }
 }
 
-// The query side of the 16 terms for half h of the lanes (q' = centred query).
+// The query side of the 16 terms for half h of the lanes (q' = centred, scaled query).
 __device__ __forceinline__ uint4 chamfer_query_terms(float qx, float qy, float qz, int h)
 {
     const unsigned sx = chamfer_split2(-2.0f * qx), sy = chamfer_split2(-2.0f * qy);
     const unsigned sz = chamfer_split2(-2.0f * qz);
-    return h == 0 ? make_uint4(sx, sx, sy, sy) : make_uint4(sz, sz, 0x3f803f80u, 0x00003f80u);
+    return h == 0 ? make_uint4(sx, sx, sy, sy) : make_uint4(sz, sz, 0x3c003c00u, 0x00003c00u);
+}
+
+// Folds the 16 results of a matrix instruction into m.
+__device__ __forceinline__ float chamfer_fold16(float m, const tk_f32x16 &acc)
+{
+#pragma unroll
+    for (int r = 0; r < 16; r += 2)
+        m = __builtin_fminf(__builtin_fminf(m, acc[r]), acc[r + 1]);
+    return m;
 }
 
 template <int NQB, int BLOCK, int STAGE>
-__global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
+chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
 {
     constexpr int NW = BLOCK / TK_WAVE;
     constexpr int QB = NW * NQB * 32;  // queries per workgroup
@@ -743,7 +765,9 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
     constexpr int TILES = STAGE / 32;
     constexpr int PER = STAGE / BLOCK;
     constexpr int MAX_SCANS = 96;
+    constexpr int SAMPLES = 4;         // keys per lane in the sample that places the centre
     static_assert(STAGE % GROUP == 0 && STAGE % BLOCK == 0 && QB % BLOCK == 0, "shapes");
+    static_assert(NQB % 2 == 0, "the loop alternates between two sets of result registers");
     // Two stage buffers of key terms, [tile][half][key in tile] x 16 bytes; the exact
     // sweep (the way out for input the bound does not cover) reuses them.
     __shared__ __align__(16) uint4 sterm[2 * STAGE * 2];
@@ -766,21 +790,35 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
     const float *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
     const float INF = __builtin_huge_valf();
 
-    // ---- bounding box of the key cloud -> centre; largest centred squared norm ----
+    // ---- centre and scale from a strided sample of the key cloud ----
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
-    for (int j = tid; j < nk; j += BLOCK) {
-        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
-        const float v[3] = {p.x, p.y, p.z};
+    if (nk > 0) {
+        TkPoint3<float> sp[SAMPLES];
 #pragma unroll
-        for (int a = 0; a < 3; ++a) {
-            lo[a] = __builtin_fminf(lo[a], v[a]);
-            hi[a] = __builtin_fmaxf(hi[a], v[a]);
+        for (int r = 0; r < SAMPLES; ++r) {
+            const int j = (int)(((int64_t)(r * BLOCK + tid) * nk) / (SAMPLES * BLOCK));
+            sp[r] = tk_load3<float>(K + (int64_t)j * 3);
+        }
+#pragma unroll
+        for (int r = 0; r < SAMPLES; ++r) {
+            const float v[3] = {sp[r].x, sp[r].y, sp[r].z};
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                // (not fmin / fmax: a NaN must reach the test below)
+                lo[a] = v[a] < lo[a] ? v[a] : (v[a] == v[a] ? lo[a] : v[a]);
+                hi[a] = v[a] > hi[a] ? v[a] : (v[a] == v[a] ? hi[a] : v[a]);
+            }
         }
     }
+    // NaN-propagating reductions: min / max of (value, partner) written with compares
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        lo[a] = wave_reduce_min(lo[a]);
-        hi[a] = wave_reduce_max(hi[a]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ol = __shfl_xor(lo[a], o), oh = __shfl_xor(hi[a], o);
+            lo[a] = (ol < lo[a] || ol != ol) ? ol : lo[a];
+            hi[a] = (oh > hi[a] || oh != oh) ? oh : hi[a];
+        }
     }
     if (lane == 0) {
 #pragma unroll
@@ -792,62 +830,53 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
     if (tid == 0)
         s_count = 0;
     __syncthreads();
-    float cc[3];
+    float cc[3], ext = 0.0f;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        float l = INF, h = -INF;
+        float l = sred[0][a], h = sred[0][3 + a];
 #pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            l = __builtin_fminf(l, sred[w][a]);
-            h = __builtin_fmaxf(h, sred[w][3 + a]);
+        for (int w = 1; w < NW; ++w) {
+            const float ol = sred[w][a], oh = sred[w][3 + a];
+            l = (ol < l || ol != ol) ? ol : l;
+            h = (oh > h || oh != oh) ? oh : h;
         }
         cc[a] = 0.5f * l + 0.5f * h;
+        const float e = 0.5f * h - 0.5f * l;
+        ext = (e > ext || e != e) ? e : ext;
     }
     const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
-    float kmax2 = 0.0f;
-    for (int j = tid; j < nk; j += BLOCK) {
-        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
-        const float x = p.x - c0;
-        const float y = p.y - c1;
-        const float z = p.z - c2;
-        kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
-    }
-    kmax2 = wave_reduce_max(kmax2);
-    if (lane == 0)
-        sred[wave][6] = kmax2;
-    __syncthreads();
-    kmax2 = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w)
-        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
-    const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
-                      (kmax2 < 1e30f);
+    // scale = 2^-(exponent of the sampled half extent), the exponent within [-40, 40]
+    // (a sample of identical points: scale 1). Outside, or with anything non-finite in
+    // the sample: exact sweep.
+    const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
+    const bool safe = nk > 0 && (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
+                      (ext - ext == 0.0f) && (ext == 0.0f || (ebits >= -40 && ebits <= 40));
     if (!safe) {  // uniform over the workgroup
         chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
     }
-    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+    const float scale =
+        ext == 0.0f ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
 
     // ---- queries: block g of the wave, column `col`; both halves of the lanes load it ----
-    tk_bf16x8 qterm[NQB];
-    float slack[NQB];
+    tk_f16x8 qterm[NQB];
+    float qnorm[NQB];  // |q'| with a margin for its rounding; > 16000 or NaN: not filtered
     float v0[NQB], v1[NQB], v2[NQB];
     int id0[NQB], id1[NQB];
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
         const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
         const bool ok = qi < nq;
-        const float px = (ok ? Q[(int64_t)qi * 3 + 0] : c0) - c0;
-        const float py = (ok ? Q[(int64_t)qi * 3 + 1] : c1) - c1;
-        const float pz = (ok ? Q[(int64_t)qi * 3 + 2] : c2) - c2;
-        qterm[g] = __builtin_bit_cast(tk_bf16x8, chamfer_query_terms(px, py, pz, half));
-        // slack = 512 u (max|k'| + |q'|)^2: NaN / inf for a non-finite or huge query,
-        // which the epilogue tests for
-        const float qn =
+        const float px = ((ok ? Q[(int64_t)qi * 3 + 0] : c0) - c0) * scale;
+        const float py = ((ok ? Q[(int64_t)qi * 3 + 1] : c1) - c1) * scale;
+        const float pz = ((ok ? Q[(int64_t)qi * 3 + 2] : c2) - c2) * scale;
+        qnorm[g] =
             1.000001f * __builtin_sqrtf(__builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px)));
-        const float r = kmax + qn;
-        slack[g] = r * r * 3.0517578e-05f + 1e-36f;
+        const bool in_range = qnorm[g] <= 16000.0f;  // false for NaN
+        qterm[g] = __builtin_bit_cast(
+            tk_f16x8, chamfer_query_terms(in_range ? px : 0.0f, in_range ? py : 0.0f,
+                                          in_range ? pz : 0.0f, half));
         v0[g] = v1[g] = v2[g] = INF;
         id0[g] = id1[g] = -1;
     }
@@ -855,11 +884,14 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
     // ---- sweep ----
     const int nstages = (nk + STAGE - 1) / STAGE;
     float pre[PER][3];
+    float kmax2 = 0.0f;  // largest |k'|^2 this lane has staged (NaN keys never match: skipped)
     auto fetch = [&](int st) {
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             const int kj = st * STAGE + r * BLOCK + tid;
-            pre[r][0] = pre[r][1] = pre[r][2] = 0.0f;
+            pre[r][0] = c0;
+            pre[r][1] = c1;
+            pre[r][2] = c2;
             if (kj < nk) {
                 const TkPoint3<float> p = tk_load3<float>(K + (int64_t)kj * 3);
                 pre[r][0] = p.x;
@@ -872,9 +904,13 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             const int j = r * BLOCK + tid;  // key within the stage
+            const float x = (pre[r][0] - c0) * scale;
+            const float y = (pre[r][1] - c1) * scale;
+            const float z = (pre[r][2] - c2) * scale;
+            const float n = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+            kmax2 = __builtin_fmaxf(kmax2, n);
             uint4 h0, h1;
-            chamfer_key_terms(pre[r][0] - c0, pre[r][1] - c1, pre[r][2] - c2,
-                              st * STAGE + j < nk, h0, h1);
+            chamfer_key_terms(x, y, z, n, st * STAGE + j < nk, h0, h1);
             uint4 *tile = sterm + buf * (STAGE * 2) + (j >> 5) * 64 + (j & 31);
             tile[0] = h0;
             tile[32] = h1;
@@ -896,26 +932,26 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
 #pragma unroll
         for (int g = 0; g < NQB; ++g)
             tmin[g] = INF;
-        // The matrix instruction of the next step is issued before the minima of the
-        // current one are taken, so the wave does not wait for its result.
-        tk_bf16x8 ka = __builtin_bit_cast(tk_bf16x8, sbuf[0]);
-        tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qterm[0], zero, 0, 0, 0);
+        // Two sets of result registers: the matrix instruction of the next step is
+        // issued before the minima of the current one are taken (the barriers keep the
+        // compiler from putting the two back in sequence on one set).
+        tk_f16x8 ka = __builtin_bit_cast(tk_f16x8, sbuf[0]);
+        tk_f32x16 acc[2];
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qterm[0], zero, 0, 0, 0);
 #pragma unroll 4
         for (int t = 0; t < ntiles; ++t) {
             // (the read after the last tile wraps to tile 0: one wasted instruction)
-            const tk_bf16x8 kn =
-                __builtin_bit_cast(tk_bf16x8, sbuf[((t + 1) & (TILES - 1)) * 64]);
+            const tk_f16x8 kn =
+                __builtin_bit_cast(tk_f16x8, sbuf[((t + 1) & (TILES - 1)) * 64]);
 #pragma unroll
             for (int g = 0; g < NQB; ++g) {
-                const tk_f32x16 next =
+                acc[(g + 1) & 1] =
                     g + 1 < NQB
-                        ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qterm[g + 1 < NQB ? g + 1 : 0],
-                                                                   zero, 0, 0, 0)
-                        : __builtin_amdgcn_mfma_f32_32x32x16_bf16(kn, qterm[0], zero, 0, 0, 0);
-                float m = tmin[g];
-#pragma unroll
-                for (int r = 0; r < 16; r += 2)
-                    m = __builtin_fminf(__builtin_fminf(m, acc[r]), acc[r + 1]);
+                        ? __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qterm[g + 1 < NQB ? g + 1 : 0],
+                                                                  zero, 0, 0, 0)
+                        : __builtin_amdgcn_mfma_f32_32x32x16_f16(kn, qterm[0], zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                const float m = chamfer_fold16(tmin[g], acc[g & 1]);
                 tmin[g] = m;
                 if ((t & 3) == 3) {
                     // three smallest group minima (ties keep the earlier group in front)
@@ -931,7 +967,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
                     v0[g] = __builtin_amdgcn_fmed3f(-INF, v0[g], x);
                     tmin[g] = INF;
                 }
-                acc = next;
+                __builtin_amdgcn_sched_barrier(0);
             }
             ka = kn;
         }
@@ -943,13 +979,24 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
         __syncthreads();
 
         // One look, an eighth of the way in: if a quarter of the lanes already see three
-        // groups within the slack, the cloud is quantised and will not get better.
+        // groups within the slack (taken with the largest key norm so far), the cloud is
+        // quantised and will not get better.
         if (nstages >= 8 && st == (nstages >> 3)) {
+            const float kmax_wave = wave_reduce_max(kmax2);
+            if (lane == 0)
+                sred[wave][6] = kmax_wave;
+            __syncthreads();
+            float kmax_now = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                kmax_now = __builtin_fmaxf(kmax_now, sred[w][6]);
+            kmax_now = __builtin_sqrtf(kmax_now) * 1.000001f;
             int tied = 0;
 #pragma unroll
             for (int g = 0; g < NQB; ++g) {
                 const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
-                const bool t3 = qi < nq && v2[g] <= v0[g] + slack[g];
+                const float r = kmax_now + qnorm[g];
+                const bool t3 = qi < nq && v2[g] <= v0[g] + r * r * 7.6293945e-06f;
                 tied += __builtin_popcountll(__builtin_amdgcn_ballot_w64(t3));
             }
             if (lane == 0)
@@ -967,28 +1014,53 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
         }
     }
 
+    // ---- the largest centred key norm; a key cloud that left fp16's range ----
+    kmax2 = wave_reduce_max(kmax2);
+    if (lane == 0)
+        sred[wave][6] = kmax2;
+    __syncthreads();
+    kmax2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
+    if (!(kmax2 <= 32768.0f)) {  // uniform over the workgroup (also +inf)
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+            d, b, qblock, slice, reinterpret_cast<float *>(sterm));
+        return;
+    }
+    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+    const float guard = 1e-36f * scale * scale;  // scale^2 <= 2^80
+
     // ---- epilogue: exact evaluation of each half's candidate groups, then the merge ----
     const bool k_aligned = (reinterpret_cast<uintptr_t>(K) & 15) == 0;  // runs of 4 keys: 48 B
-#pragma unroll 1
+    float qx[NQB], qy[NQB], qz[NQB];
+#pragma unroll
+    for (int g = 0; g < NQB; ++g) {
+        const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
+        const bool ok = qi < nq;
+        qx[g] = ok ? Q[(int64_t)qi * 3 + 0] : 0.0f;
+        qy[g] = ok ? Q[(int64_t)qi * 3 + 1] : 0.0f;
+        qz[g] = ok ? Q[(int64_t)qi * 3 + 2] : 0.0f;
+    }
+#pragma unroll
     for (int g = 0; g < NQB; ++g) {
         const int slot = (wave * NQB + g) * 32 + col;
         const int qi = qblock * QB + slot;
         const bool ok = qi < nq;
         const float best_score = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
-        const float thr = best_score + slack[g];
-        const bool usable = slack[g] < 1e30f;  // false for NaN / inf / huge
+        const float r = kmax + qnorm[g];
+        const float thr = best_score + (r * r * 7.6293945e-06f + guard);  // 2^-17 R
+        const bool filtered = qnorm[g] <= 16000.0f;  // false for NaN / inf / out of range
         // No finite score at all (nk == 0 or every key NaN): the exact result is (+inf, -1).
-        const bool none = !(best_score < INF);
+        const bool none = filtered && !(best_score < INF);
         const bool crowded = v2[g] <= thr;  // three or more candidate groups in this half
         const bool over =
-            ok && !none && (!usable || __builtin_amdgcn_ballot_w64(crowded) >> col & 0x100000001ull);
+            ok && !none && (!filtered || (__builtin_amdgcn_ballot_w64(crowded) >> col & 0x100000001ull));
         float bestd = INF;
         int bestj = -1;
         if (ok && !none && !over) {
-            const float qx = Q[(int64_t)qi * 3 + 0], qy = Q[(int64_t)qi * 3 + 1],
-                        qz = Q[(int64_t)qi * 3 + 2];
             int ta = v0[g] <= thr ? id0[g] : -1, tb = v1[g] <= thr ? id1[g] : -1;
-            if (tb >= 0 && tb < ta) {
+            if (tb >= 0 && (ta < 0 || tb < ta)) {
                 const int tmp = ta;
                 ta = tb;
                 tb = tmp;
@@ -998,25 +1070,38 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
                 if (group < 0)
                     continue;
                 // this half's keys of the group: runs of 4 keys, 8 keys apart
-                for (int run = 0; run < GROUP / 8; ++run) {
-                    const int j = group * GROUP + run * 8 + half * 4;
-                    if (j >= nk)
-                        break;
-                    if (k_aligned && j + 4 <= nk) {
-                        const float4 *p4 = reinterpret_cast<const float4 *>(K + (int64_t)j * 3);
-                        const float4 f0 = p4[0], f1 = p4[1], f2 = p4[2];
-                        const float dd0 = tk_dist2<float>(f0.x, f0.y, f0.z, qx, qy, qz);
-                        const float dd1 = tk_dist2<float>(f0.w, f1.x, f1.y, qx, qy, qz);
-                        const float dd2 = tk_dist2<float>(f1.z, f1.w, f2.x, qx, qy, qz);
-                        const float dd3 = tk_dist2<float>(f2.y, f2.z, f2.w, qx, qy, qz);
-                        if (dd0 < bestd) { bestd = dd0; bestj = j; }
-                        if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
-                        if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
-                        if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
-                    } else {
+                if (k_aligned && (group + 1) * GROUP <= nk) {
+                    const float4 *p4 =
+                        reinterpret_cast<const float4 *>(K + (int64_t)(group * GROUP + half * 4) * 3);
+#pragma unroll
+                    for (int r0 = 0; r0 < GROUP / 8; r0 += 4) {
+                        float4 f[4][3];
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) {  // a run is 48 bytes, runs 96 bytes apart
+                            f[rr][0] = p4[(r0 + rr) * 6 + 0];
+                            f[rr][1] = p4[(r0 + rr) * 6 + 1];
+                            f[rr][2] = p4[(r0 + rr) * 6 + 2];
+                        }
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) {
+                            const int j = group * GROUP + (r0 + rr) * 8 + half * 4;
+                            const float4 f0 = f[rr][0], f1 = f[rr][1], f2 = f[rr][2];
+                            const float dd0 = tk_dist2<float>(f0.x, f0.y, f0.z, qx[g], qy[g], qz[g]);
+                            const float dd1 = tk_dist2<float>(f0.w, f1.x, f1.y, qx[g], qy[g], qz[g]);
+                            const float dd2 = tk_dist2<float>(f1.z, f1.w, f2.x, qx[g], qy[g], qz[g]);
+                            const float dd3 = tk_dist2<float>(f2.y, f2.z, f2.w, qx[g], qy[g], qz[g]);
+                            if (dd0 < bestd) { bestd = dd0; bestj = j; }
+                            if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
+                            if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
+                            if (dd3 < bestd) { bestd = dd3; bestj = j + 3; }
+                        }
+                    }
+                } else {
+                    for (int run = 0; run < GROUP / 8; ++run) {
+                        const int j = group * GROUP + run * 8 + half * 4;
                         for (int e = j; e < j + 4 && e < nk; ++e) {
                             const TkPoint3<float> p = tk_load3<float>(K + (int64_t)e * 3);
-                            const float dd = tk_dist2<float>(p.x, p.y, p.z, qx, qy, qz);
+                            const float dd = tk_dist2<float>(p.x, p.y, p.z, qx[g], qy[g], qz[g]);
                             if (dd < bestd) {
                                 bestd = dd;
                                 bestj = e;
@@ -1044,7 +1129,7 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_mfma_kernel(ChamferFwdA
         }
     }
 
-    // ---- queries with three or more candidate groups in a half ----
+    // ---- queries with three or more candidate groups in a half, or out of range ----
     __syncthreads();
     const int nscan = s_count;
     if (nscan > MAX_SCANS) {  // uniform over the workgroup
@@ -1578,11 +1663,19 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
         // The pre-filter pays off once the key clouds are a few hundred points long
         // (its prologue passes over the keys twice per workgroup).
         const int64_t nkmin = N1 < N2 ? N1 : N2;
-        // Matrix-core pre-filter: 512 queries per workgroup; worth it once the launch
-        // fills the chip twice over and the key clouds are a few thousand points long.
-        if (nkmin >= 2048 && B * ((N1 + 511) / 512 + (N2 + 511) / 512) >= 512)
-            return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
-                                                  s);
+        // Matrix-core pre-filter, 512 queries per workgroup: the fastest sweep from about a
+        // hundred workgroups on key clouds of 1024 points or more (1.3-2.2x over the
+        // vector pre-filter). Smaller launches cut the key clouds into slices of 1024
+        // keys or more until 256 workgroups are there.
+        if (nkmin >= 1024) {
+            const int64_t blocks = B * ((N1 + 511) / 512 + (N2 + 511) / 512);
+            int slices = 1;
+            while (blocks * slices < 256 && slices < 16 && nkmin / (slices * 2) >= 1024)
+                slices *= 2;
+            if (blocks * slices >= 96)
+                return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+                                                      idx2, s, slices);
+        }
         if (nkmin >= 512) {
             // Launch shapes: 4 queries per lane in 512-lane workgroups is the fastest
             // sweep once it fills the chip; below that 2 queries per lane in 256-lane
