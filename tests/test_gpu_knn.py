@@ -247,6 +247,14 @@ def _filter_case(kind, g, k):
         q, key = q * 1e18, key * 1e18
     elif kind == "huge_queries":                 # only the queries are beyond the bound
         q = q * 3e18
+    elif kind == "scaled_small":                 # inside the range the matrix scores rescale
+        q, key = q * 1e-9, key * 1e-9
+    elif kind == "scaled_large":
+        q, key = q * 3e9 + 1e9, key * 3e9 + 1e9
+    elif kind == "far_queries":                  # some queries beyond the fp16 pieces' range
+        q[:, ::97] *= 400.0                      # (200 times the key cloud's extent)
+        q[:, 5::211, 2] += 2.0e4
+        q[:, 11::301] *= 150.0                   # inside the range, thresholds of order 1e4
     elif kind == "clusters":
         centres = uniform_cloud(g, b, 8) * 100.0
         def mk(n):
@@ -273,6 +281,7 @@ def _filter_case(kind, g, k):
 @pytest.mark.parametrize("k", [1, 3, 4, 7, 16])
 @pytest.mark.parametrize("kind", ["uniform", "lattice", "far_to_near", "near_to_far",
                                   "far_from_origin", "separated", "tiny", "huge", "huge_queries",
+                                  "scaled_small", "scaled_large", "far_queries",
                                   "clusters", "duplicates", "nan_and_inf"])
 def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
     q, key = _filter_case(kind, gen(sum(map(ord, kind)) + k), k)

@@ -699,35 +699,16 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
 // groups per half are re-evaluated with the canonical arithmetic in ascending key
 // order, three or more send the query to the exact scan, non-finite or out-of-range input
 // takes the exact sweep. Results are bit-identical to the exact sweep for every input.
-typedef _Float16 tk_f16x8 __attribute__((ext_vector_type(8)));
-typedef float tk_f32x16 __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ unsigned chamfer_f16_bits(float x)  // nearest fp16
-{
-    return (unsigned)__builtin_bit_cast(unsigned short, (_Float16)x);
-}
-__device__ __forceinline__ float chamfer_f16_value(unsigned b)
-{
-    return (float)__builtin_bit_cast(_Float16, (unsigned short)b);
-}
-// x = hi + lo + e, |e| <= 2^-23 |x| + 2^-25; returns hi | lo << 16.
-__device__ __forceinline__ unsigned chamfer_split2(float x)
-{
-    const unsigned hi = chamfer_f16_bits(x);
-    const unsigned lo = chamfer_f16_bits(x - chamfer_f16_value(hi));  // the difference is exact
-    return hi | (lo << 16);
-}
-
 // The two 16-byte halves of a key's 16 terms; n = |k'|^2. A key past the end gets
 // |k'|^2 = +inf.
 __device__ __forceinline__ void chamfer_key_terms(float x, float y, float z, float n, bool exists,
                                                   uint4 &half0, uint4 &half1)
 {
-    const unsigned sx = chamfer_split2(x), sy = chamfer_split2(y), sz = chamfer_split2(z);
-    const unsigned n0 = chamfer_f16_bits(n);
-    const float r1 = n - chamfer_f16_value(n0);
-    const unsigned n1 = chamfer_f16_bits(r1);
-    const unsigned n2 = chamfer_f16_bits(r1 - chamfer_f16_value(n1));
+    const unsigned sx = tk_f16_split2(x), sy = tk_f16_split2(y), sz = tk_f16_split2(z);
+    const unsigned n0 = tk_f16_bits(n);
+    const float r1 = n - tk_f16_value(n0);
+    const unsigned n1 = tk_f16_bits(r1);
+    const unsigned n2 = tk_f16_bits(r1 - tk_f16_value(n1));
     const unsigned xh = sx & 0xffffu, xl = sx >> 16, yh = sy & 0xffffu, yl = sy >> 16;
     const unsigned zh = sz & 0xffffu, zl = sz >> 16;
     half0 = make_uint4(xh * 0x10001u, xl * 0x10001u, yh * 0x10001u, yl * 0x10001u);
@@ -741,8 +722,8 @@ __device__ __forceinline__ void chamfer_key_terms(float x, float y, float z, flo
 // The query side of the 16 terms for half h of the lanes (q' = centred, scaled query).
 __device__ __forceinline__ uint4 chamfer_query_terms(float qx, float qy, float qz, int h)
 {
-    const unsigned sx = chamfer_split2(-2.0f * qx), sy = chamfer_split2(-2.0f * qy);
-    const unsigned sz = chamfer_split2(-2.0f * qz);
+    const unsigned sx = tk_f16_split2(-2.0f * qx), sy = tk_f16_split2(-2.0f * qy);
+    const unsigned sz = tk_f16_split2(-2.0f * qz);
     return h == 0 ? make_uint4(sx, sx, sy, sy) : make_uint4(sz, sz, 0x3c003c00u, 0x00003c00u);
 }
 

@@ -411,8 +411,35 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 // Per 2048 keys a wave runs 68 steps at k = 3 and 145 at k = 16 instead of 142 and 253
 // rounds. Keys are centred and staged in LDS as (x', y', z', |k'|^2); a lane serves QPL
 // queries, so one LDS read feeds QPL pairs and the steps of its queries interleave.
-template <int KMAX, int QPL, bool SOA, bool WEIGHTS>
-__global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
+//
+// MATRIX. The scores of a chunk of 32 keys come from the matrix cores instead: one
+// v_mfma_f32_32x32x16_f16 gives t = s - thr for 32 keys x 32 queries as a 16-term dot
+// product of fp16 pieces, and a lane only has to collect the 16 sign bits it is handed
+// (1.1 vector instructions per pair instead of 5). Coordinates are centred and multiplied
+// by a power of two that brings the largest centred key norm into [1, 2) (exact; outside
+// 2^-40 .. 2^40 the workgroup takes the exact sweep), then split into two fp16 pieces
+// each, x = xh + xl + e with |e| <= 2^-23 |x| + 2^-25, |k'|^2 into two and -thr into two:
+//     key   : xh xh xl  yh yh yl  1  1  | zh zh zl  n0 n1 0  1  1
+//     query : Xh Xl Xh  Yh Yl Yh  T0 T1 | Zh Zl Zh  1  1  0  T0 T1        (X = -2 q'x)
+// In the 32 x 32 result lane l holds rows (keys) 16 h .. 16 h + 15, h = l / 32, of column
+// (query) l % 32; the keys of a tile are stored in that row order, so the sign bits of a
+// lane are 16 consecutive bits of the chunk mask. The wave's 128 queries are four blocks
+// of 32; lane l owns the queries of column l % 32 in blocks h and 2 + h, computes their
+// thr and writes -thr into the T terms of its own half only (the other half holds zeros
+// there), so no thr crosses lanes; the two halves of a mask meet through one exchange
+// between lanes l and l ^ 32 per chunk. Error budget in the rescaled units, on top of the
+// one above (products of the second pieces are left out, thr is rounded to two pieces):
+//     pieces dropped from 2 q'.k', subnormal pieces                       5 u R
+//     |k'|^2 and thr in two pieces                           4 u R + 4 u (M + R)
+//     the matrix core's 16 additions, one unit in the last place of the largest
+//         partial sum each (measured: at most 9.3 u times the largest product)
+//                                                                    32 u (M + R)
+//     canonical d2, |k'|^2 as staged, thr itself             10 u R + 3 u (M + R)
+// below 58 u R + 39 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
+// from the centre (rescaled; thr would leave fp16's range) take every key as a candidate.
+template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX>
+__global__ __launch_bounds__(KNN_BLOCK)
+    __attribute__((amdgpu_waves_per_eu(MATRIX && KMAX <= 4 ? 3 : 1))) void knn_filter_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
     float eps, int blocks_per_batch, int n1, int n2, int k)
@@ -429,11 +456,16 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
                   "the staging buffers double as the exact sweep's stage");
     // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
     // the sweep runs into), then two of raw keys (x, y, z, 0) for the service steps.
-    constexpr int STAGING_FLOATS = 2 * STAGE * 4 + 32 + 2 * STAGE * 4;
+    // (MATRIX: two stage buffers of key terms, [tile][half][row] x 16 bytes, instead.)
+    static_assert(!MATRIX || QPL == 2, "four blocks of 32 queries per wave");
+    constexpr int SCORE_FLOATS = MATRIX ? 2 * STAGE * 8 : 2 * STAGE * 4 + 32;
+    constexpr int STAGING_FLOATS = SCORE_FLOATS + 2 * STAGE * 4;
     constexpr int TRANSPOSE_FLOATS = NW * 2 * TK_WAVE * (KMAX + 1);  // see the end of the kernel
     __shared__ __align__(16) float
         skey[STAGING_FLOATS > TRANSPOSE_FLOATS ? STAGING_FLOATS : TRANSPOSE_FLOATS];
-    float4 *const sraw = reinterpret_cast<float4 *>(skey + 2 * STAGE * 4 + 32);
+    float4 *const sraw = reinterpret_cast<float4 *>(skey + SCORE_FLOATS);
+    uint4 *const sterm = reinterpret_cast<uint4 *>(skey);
+    const int half = (threadIdx.x >> 5) & 1;
     __shared__ float sred[NW][8];
     const int tid = threadIdx.x;
     const int lane = tid & (TK_WAVE - 1);
@@ -499,8 +531,15 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
 #pragma unroll
     for (int w = 0; w < NW; ++w)
         kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
-    const bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
-                      (kmax2 < 1e30f);
+    bool safe = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) && (kmax2 < 1e30f);
+    float scale = 1.0f;  // MATRIX: 2^-(exponent of the largest centred key norm)
+    if constexpr (MATRIX) {
+        const float ext = __builtin_sqrtf(kmax2);
+        const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
+        safe = safe && (ext == 0.0f || (ebits >= -40 && ebits <= 40));
+        scale = (!safe || ext == 0.0f) ? 1.0f
+                                       : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
+    }
     if (!safe) {  // uniform over the workgroup
 #pragma unroll 1
         for (int i = 0; i < QPL; ++i)
@@ -509,7 +548,8 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
                                                  skey);
         return;
     }
-    const float kmax = __builtin_sqrtf(kmax2) * 1.000001f;
+    const float kmax = __builtin_sqrtf(kmax2) * scale * 1.000001f;
+    const float scale2 = scale * scale;  // <= 2^80
 
     // ---- queries ----
     float qx[QPL], qy[QPL], qz[QPL], ax[QPL], ay[QPL], az[QPL], qn[QPL], slack_r[QPL];
@@ -542,14 +582,23 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
         qx[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 0) : c0;
         qy[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 1) : c1;
         qz[i] = active[i] ? knn_coord<SOA>(Q, n1, qi, 2) : c2;
-        const float px = qx[i] - c0, py = qy[i] - c1, pz = qz[i] - c2;
+        const float px = (qx[i] - c0) * scale, py = (qy[i] - c1) * scale, pz = (qz[i] - c2) * scale;
         ax[i] = -2.0f * px;
         ay[i] = -2.0f * py;
         az[i] = -2.0f * pz;
         qn[i] = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px));
-        const float r = kmax + __builtin_sqrtf(qn[i]) * 1.000001f;
-        slack_r[i] = r * r * 1.9073486e-06f + 1e-37f;  // 32 u R
-        usable[i] = slack_r[i] < 1e30f;                  // false for NaN / inf / huge
+        const float qnorm = __builtin_sqrtf(qn[i]) * 1.000001f;
+        const float r = kmax + qnorm;
+        if constexpr (MATRIX) {
+            slack_r[i] = r * r * 3.8146973e-06f + 1e-37f * scale2;  // 64 u R
+            usable[i] = qnorm <= 200.0f;                            // false for NaN
+            ax[i] = usable[i] ? ax[i] : 0.0f;
+            ay[i] = usable[i] ? ay[i] : 0.0f;
+            az[i] = usable[i] ? az[i] : 0.0f;
+        } else {
+            slack_r[i] = r * r * 1.9073486e-06f + 1e-37f;  // 32 u R
+            usable[i] = slack_r[i] < 1e30f;                  // false for NaN / inf / huge
+        }
         // fill: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots stay at -inf
         max_key[i] = 0.0f;
         max_idx[i] = 0;
@@ -578,6 +627,29 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
         pq[i] = Pending{0u, 0u, 0u, 0u, 0, 0, 0, 0};
         qlen[i] = 0;
         pending[i] = 0;
+    }
+
+    // MATRIX: the query side of the 16 terms for the wave's four blocks of 32 queries.
+    // Block 2 i + h' holds query i of the lanes of half h'; this lane supplies terms
+    // 8 h .. 8 h + 7 of column lane % 32 in every block, from its own coordinates or, for
+    // the other half's blocks, its partner's. The T terms (.w) are written per chunk.
+    uint4 qterm[MATRIX ? 2 * QPL : 1];
+    if constexpr (MATRIX) {
+#pragma unroll
+        for (int i = 0; i < QPL; ++i) {
+            const float ox = __shfl_xor(ax[i], 32), oy = __shfl_xor(ay[i], 32),
+                        oz = __shfl_xor(az[i], 32);
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {  // the block owned by half hb
+                const bool own = half == hb;
+                const float X = own ? ax[i] : ox, Y = own ? ay[i] : oy, Z = own ? az[i] : oz;
+                const unsigned sx = tk_f16_split2(X), sy = tk_f16_split2(Y), sz = tk_f16_split2(Z);
+                const unsigned xh = sx & 0xffffu, yh = sy & 0xffffu, zh = sz & 0xffffu;
+                qterm[2 * i + hb] =
+                    half == 0 ? make_uint4(sx, xh | (yh << 16), (sy >> 16) | (yh << 16), 0u)
+                              : make_uint4(sz, zh | 0x3c000000u, 0x00003c00u, 0u);
+            }
+        }
     }
 
     // One service step: every query with a pending candidate takes its first one. Written
@@ -703,8 +775,26 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
     auto stash = [&](int buf) {
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
-            reinterpret_cast<float4 *>(skey)[buf * STAGE + r * BLOCK + tid] = pre[r];
-            sraw[buf * STAGE + r * BLOCK + tid] = pre_raw[r];
+            const int j = r * BLOCK + tid;  // key within the stage
+            if constexpr (MATRIX) {
+                const float4 e = pre[r];
+                const float x = e.x * scale, y = e.y * scale, z = e.z * scale;
+                const float n = e.w * scale2;  // (+inf past the end)
+                const unsigned sx = tk_f16_split2(x), sy = tk_f16_split2(y), sz = tk_f16_split2(z);
+                const unsigned xh = sx & 0xffffu, yh = sy & 0xffffu, zh = sz & 0xffffu;
+                const unsigned sn = tk_f16_split2(n);
+                const bool exists = e.w < INF || e.w != e.w;
+                const unsigned n0 = exists ? (sn & 0xffffu) : 0x7c00u, n1 = exists ? (sn >> 16) : 0u;
+                // row of the tile: lane half h of the result holds rows 8 a + 4 h + c
+                const int row = ((j & 12) << 1) | ((j & 16) >> 2) | (j & 3);
+                uint4 *t = sterm + buf * (STAGE * 2) + (j >> 5) * 64 + row;
+                t[0] = make_uint4(xh * 0x10001u, (sx >> 16) | (yh << 16), yh | (sy & 0xffff0000u),
+                                  0x3c003c00u);
+                t[32] = make_uint4(zh * 0x10001u, (sz >> 16) | (n0 << 16), n1, 0x3c003c00u);
+            } else {
+                reinterpret_cast<float4 *>(skey)[buf * STAGE + j] = pre[r];
+            }
+            sraw[buf * STAGE + j] = pre_raw[r];
         }
     };
     __syncthreads();
@@ -724,9 +814,47 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
             unsigned mask[QPL];
 #pragma unroll
             for (int i = 0; i < QPL; ++i) {
-                thr[i] = (max_key[i] - qn[i]) + __builtin_fmaf(max_key[i], 9.5367432e-07f, slack_r[i]);
+                if constexpr (MATRIX) {  // rescaled units; slack 64 u R + 48 u M
+                    const float m = max_key[i] * scale2;
+                    thr[i] = (m - qn[i]) + __builtin_fmaf(m, 2.8610229e-06f, slack_r[i]);
+                } else {
+                    thr[i] = (max_key[i] - qn[i]) +
+                             __builtin_fmaf(max_key[i], 9.5367432e-07f, slack_r[i]);
+                }
                 mask[i] = 0u;
             }
+            if constexpr (MATRIX) {
+                const tk_f16x8 ka = __builtin_bit_cast(
+                    tk_f16x8, sterm[(st & 1) * (STAGE * 2) + (c0k >> 5) * 64 + lane]);
+#pragma unroll
+                for (int i = 0; i < QPL; ++i) {
+                    const unsigned tp = tk_f16_split2(-thr[i]);
+                    qterm[2 * i].w = half == 0 ? tp : 0u;
+                    qterm[2 * i + 1].w = half == 1 ? tp : 0u;
+                }
+                const tk_f32x16 zero = {};
+                unsigned m16[2 * QPL];
+#pragma unroll
+                for (int g = 0; g < 2 * QPL; ++g) {
+                    const tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        ka, __builtin_bit_cast(tk_f16x8, qterm[g]), zero, 0, 0, 0);
+                    unsigned m = 0u;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float t = acc[r];  // (a bit_cast applied to acc[r] itself reads element 0)
+                        m = __builtin_amdgcn_alignbit(m, __builtin_bit_cast(unsigned, t), 31);
+                    }
+                    m16[g] = m;
+                }
+                // rows of this half: keys 16 h .. 16 h + 15 of the chunk, first key in the
+                // highest bit; the other half's rows of this lane's blocks come from lane ^ 32
+                const unsigned send = half == 0 ? (m16[1] | (m16[3] << 16)) : (m16[0] | (m16[2] << 16));
+                const unsigned recv = __shfl_xor(send, 32);
+                const unsigned own0 = half == 0 ? m16[0] : m16[1], own1 = half == 0 ? m16[2] : m16[3];
+                const unsigned oth0 = recv & 0xffffu, oth1 = recv >> 16;
+                mask[0] = half == 0 ? ((own0 << 16) | oth0) : ((oth0 << 16) | own0);
+                mask[1] = half == 0 ? ((own1 << 16) | oth1) : ((oth1 << 16) | own1);
+            } else {
             const float4 *ck = sbuf + c0k;
             // Groups of G keys: the next group is read from LDS before the current one is
             // used, and the G scores of a query are independent chains.
@@ -764,6 +892,7 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
 #pragma unroll
                 for (int g = 0; g < G; ++g)
                     cur[g] = nxt[g];
+            }
             }
             // Keys that do not exist, or that the fill phase took, are no candidates.
             int vlo = k - first;
@@ -1690,20 +1819,18 @@ void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64
 // The pre-filtered kernel pays when the launch fills the chip with two queries per lane
 // and the key cloud is long enough to amortise its prologue (two passes over the keys per
 // workgroup); TK3D_ERR_UNSUPPORTED otherwise. Thresholds from timing it against the
-// kernels above on an MI355X for k = 1..16, 32768 to 524288 queries, 256 to 8192 keys:
-// 1.1-1.8 times faster inside them, 0.6-1.0 outside.
+// kernels above on an MI355X for k = 1..16, 16384 to 524288 queries, 256 to 8192 keys:
+// 1.05-1.5 times faster inside them, 0.6-1.0 outside.
 inline bool knn_filter_pays(int64_t queries, int n2, int k)
 {
-    if (n2 >= 8192)
-        return queries >= 32768;
     if (n2 >= 2048)
-        return queries >= (k <= 5 ? 65536 : 131072);
+        return queries >= 32768;
     if (n2 >= 1024)
         return queries >= 262144;
-    return n2 >= 512 && k <= 4 && queries >= 262144;
+    return n2 >= 512 && queries >= (k <= 4 ? 131072 : k <= 8 ? 262144 : 524288);
 }
 
-template <int KMAX, bool SOA, bool WEIGHTS>
+template <int KMAX, bool SOA, bool WEIGHTS, bool MATRIX = true>
 int knn_filter_launch(const float *query, const float *key, float *distance, int64_t *index,
                       float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
@@ -1711,7 +1838,7 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
     const int64_t bpb = ((int64_t)n1 + QPL * KNN_BLOCK - 1) / (QPL * KNN_BLOCK);
     if (!knn_filter_pays(B * n1, n2, k) || B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, QPL, SOA, WEIGHTS>), dim3((unsigned)(B * bpb)),
+    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, QPL, SOA, WEIGHTS, MATRIX>), dim3((unsigned)(B * bpb)),
                        dim3(KNN_BLOCK), 0, s, query, key, distance, index, weight, eps, (int)bpb,
                        n1, n2, k);
     return tk_launch_status();

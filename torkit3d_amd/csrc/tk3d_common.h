@@ -73,6 +73,30 @@ template <typename T> __device__ __forceinline__ TkPoint3<T> tk_load3(const T *p
     return *reinterpret_cast<const TkPoint3<T> *>(p);
 }
 
+// ---- fp16 pieces for scores computed on the matrix cores ------------------------------
+
+typedef _Float16 tk_f16x8 __attribute__((ext_vector_type(8)));
+typedef float tk_f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ unsigned tk_f16_bits(float x)  // nearest fp16
+{
+    return (unsigned)__builtin_bit_cast(unsigned short, (_Float16)x);
+}
+__device__ __forceinline__ float tk_f16_value(unsigned b)
+{
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)b);
+}
+// x = hi + lo + e with |e| <= 2^-23 |x| + 2^-25 (fp16 has 11 significant bits: the first
+// piece is within 2^-11 |x| of x, the second within 2^-12 of the rest or within half the
+// subnormal spacing 2^-24); returns hi | lo << 16. x beyond +-65504 gives an infinite hi
+// and a NaN lo.
+__device__ __forceinline__ unsigned tk_f16_split2(float x)
+{
+    const unsigned hi = tk_f16_bits(x);
+    const unsigned lo = tk_f16_bits(x - tk_f16_value(hi));  // the difference is exact
+    return hi | (lo << 16);
+}
+
 // ---- host side --------------------------------------------------------------
 
 static inline int tk_launch_status()
