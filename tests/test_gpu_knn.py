@@ -95,6 +95,23 @@ def test_non_finite_keys_follow_mink(cuda, k):
     check_raw(q, key, k, cuda)
 
 
+@pytest.mark.parametrize("b,n1,n2,k", [(1, 200, 3000, 17), (2, 100, 500, 64), (2, 200, 700, 128),
+                                        (1, 70, 70000, 20), (2, 33, 40, 40), (1, 100, 400, 129)])
+def test_fp64_beyond_16_neighbours_keeps_mink_order(cuda, b, n1, n2, k):
+    # fp64 with k = 17..128 keeps its slots in LDS as a tournament tree, as fp32 does
+    g = gen(k + 1)
+    q, key = uniform_cloud(g, b, n1).double(), uniform_cloud(g, b, n2).double()
+    check_raw(q, key, k, cuda)
+    q, key = lattice_cloud(g, b, n1, 4).double(), lattice_cloud(g, b, n2, 4).double()
+    check_raw(q, key, k, cuda)                     # exact ties everywhere
+    key = uniform_cloud(g, b, n2).double()
+    key[0, 0, 1] = float("nan")                    # slot 0 of the fill: nothing is inserted later
+    key[-1, 2, 0] = float("nan")                   # a later fill slot keeps its NaN
+    key[-1, n2 // 2, 2] = float("nan")             # beyond the fill: never inserted
+    key[0, 1, 0] = float("inf")
+    check_raw(q, key, k, cuda)
+
+
 def test_k1_equals_chamfer_argmin(cuda):
     from torkit3d_amd import _C
 

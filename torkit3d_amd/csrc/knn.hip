@@ -1030,23 +1030,23 @@ __global__ __launch_bounds__(KNN_BLOCK)
 // maximum). MinK never selects such a slot as maximum unless it is slot 0, in which
 // case it never inserts again. Here a NaN in slot 0 freezes the lane; a NaN elsewhere
 // plays the tournament as -inf and is recomputed when the results are written.
-template <int KMAX, bool IDX16> struct KnnTreeLayout {
+template <int KMAX, bool IDX16, typename T = float> struct KnnTreeLayout {
     static constexpr int NT = 64;
     using Idx = typename std::conditional<IDX16, unsigned short, int>::type;
-    static constexpr int LEAF_BYTES = 4 * KMAX * NT;
+    static constexpr int LEAF_BYTES = (int)sizeof(T) * KMAX * NT;
     static constexpr int KIDX_BYTES = (int)sizeof(Idx) * KMAX * NT;
-    static constexpr int IVAL_BYTES = 4 * (KMAX / 2) * NT;
+    static constexpr int IVAL_BYTES = (int)sizeof(T) * (KMAX / 2) * NT;
     static constexpr int IARG_BYTES = (KMAX / 2) * NT;
     static constexpr int BYTES = LEAF_BYTES + KIDX_BYTES + IVAL_BYTES + IARG_BYTES;
 };
 
-template <int KMAX, bool IDX16>
-__global__ __launch_bounds__(64) void knn_tree_kernel_f32(
-    const float *__restrict__ query, const float *__restrict__ key,
-    float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
+template <typename T, int KMAX, bool IDX16>
+__global__ __launch_bounds__(64) void knn_tree_kernel(
+    const T *__restrict__ query, const T *__restrict__ key,
+    T *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
     int n2, int k)
 {
-    using Lay = KnnTreeLayout<KMAX, IDX16>;
+    using Lay = KnnTreeLayout<KMAX, IDX16, T>;
     using Idx = typename Lay::Idx;
     constexpr int CHUNK = 32;
     constexpr int NT = 64;
@@ -1057,29 +1057,29 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     static_assert(KMAX <= 256, "slot numbers are kept in one byte");
     extern __shared__ __align__(16) unsigned char knn_tree_lds[];
     const int lane = threadIdx.x;
-    float *const leaf = reinterpret_cast<float *>(knn_tree_lds) + lane;
+    T *const leaf = reinterpret_cast<T *>(knn_tree_lds) + lane;
     Idx *const kidx = reinterpret_cast<Idx *>(knn_tree_lds + Lay::LEAF_BYTES) + lane;
-    float *const ival =
-        reinterpret_cast<float *>(knn_tree_lds + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
+    T *const ival =
+        reinterpret_cast<T *>(knn_tree_lds + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
     unsigned char *const iarg =
         knn_tree_lds + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
 
     const int b = blockIdx.x / blocks_per_batch;
     const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
     const bool active = qi < n1;
-    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
-    float qx = 0, qy = 0, qz = 0;
+    const T *__restrict__ K = key + (int64_t)b * n2 * 3;
+    T qx = 0, qy = 0, qz = 0;
     if (active) {
-        const float *q = query + ((int64_t)b * n1 + qi) * 3;
+        const T *q = query + ((int64_t)b * n1 + qi) * 3;
         qx = q[0];
         qy = q[1];
         qz = q[2];
     }
 
     // Value and first slot of a node whose children are leaves.
-    auto leaf_parent = [&](int n, float &v, int &a) {
+    auto leaf_parent = [&](int n, T &v, int &a) {
         const int s = 2 * n - KMAX;
-        const float lv = leaf[s * NT], rv = leaf[(s + 1) * NT];
+        const T lv = leaf[s * NT], rv = leaf[(s + 1) * NT];
         const bool right = rv > lv;
         v = right ? rv : lv;
         a = right ? s + 1 : s;
@@ -1088,19 +1088,19 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     // Fill phase: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots hold -inf.
     bool frozen = false;
     for (int s = 0; s < KMAX; ++s) {
-        float d = -__builtin_huge_valf();
+        T d = -tk_inf<T>();
         if (s < k) {
-            d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            d = tk_dist2<T>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
             if (d != d) {
                 frozen |= s == 0;
-                d = -__builtin_huge_valf();  // marks the slot: no real distance is -inf
+                d = -tk_inf<T>();  // marks the slot: no real distance is -inf
             }
         }
         leaf[s * NT] = d;
         kidx[s * NT] = (Idx)s;
     }
     for (int n = HALF - 1; n >= 1; --n) {
-        float lv, rv;
+        T lv, rv;
         int la, ra;
         if (2 * n >= HALF) {
             leaf_parent(2 * n, lv, la);
@@ -1115,29 +1115,37 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         ival[n * NT] = right ? rv : lv;
         iarg[n * NT] = (unsigned char)(right ? ra : la);
     }
-    float max_key = frozen ? -__builtin_huge_valf() : ival[NT];
+    T max_key = frozen ? -tk_inf<T>() : ival[NT];
     int max_idx = iarg[NT];
 
     for (int first = 0; first < n2; first += CHUNK) {  // `first` = key index of bit 31
         // ---- sweep: bit (31 - i) of `mask` <=> key first+i is below the maximum ----
-        const int maxbits = __builtin_bit_cast(int, max_key);
+        // (fp32: squared distances are non-negative, their bit patterns order as integers
+        // and the sign of the difference is shifted in with one instruction)
+        auto below_max = [&](unsigned m, T d) {
+            if constexpr (sizeof(T) == 4) {
+                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) -
+                                                 __builtin_bit_cast(int, max_key));
+                return __builtin_amdgcn_alignbit(m, diff, 31);  // (m << 1) | sign
+            } else {
+                return (m << 1) | (d < max_key ? 1u : 0u);
+            }
+        };
         unsigned mask = 0u;
         if (first + CHUNK <= n2) {
-            const float *__restrict__ g = K + (int64_t)first * 3;
+            const T *__restrict__ g = K + (int64_t)first * 3;
 #pragma unroll
             for (int i = 0; i < CHUNK; ++i) {
-                const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
+                const T d = tk_dist2<T>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
                                                 qy, qz);
-                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
-                mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
+                mask = below_max(mask, d);
             }
         } else {
             for (int i = 0; i < CHUNK; ++i) {
                 const int j = first + i < n2 ? first + i : n2 - 1;  // clamped, masked below
-                const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
+                const T d = tk_dist2<T>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
                                                 K[(int64_t)j * 3 + 2], qx, qy, qz);
-                const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
-                mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                mask = below_max(mask, d);
             }
         }
         // Keys that do not exist, or that the fill phase took, are no candidates.
@@ -1150,23 +1158,23 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
         mask &= valid;
 
         // ---- insertion rounds, the next candidate's key in flight during the current ----
-        const float *__restrict__ ck = K + (int64_t)first * 3;
+        const T *__restrict__ ck = K + (int64_t)first * 3;
         bool has = mask != 0u;
         int i = has ? __builtin_clz(mask) : 0;
-        float ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
+        T ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
             mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
             const bool has_next = mask != 0u;
             const int i_next = has_next ? __builtin_clz(mask) : 0;
-            const float nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
+            const T nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
                         nz = ck[3 * i_next + 2];
-            const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+            const T d = tk_dist2<T>(ex, ey, ez, qx, qy, qz);
             if (has && d < max_key) {
                 const int p = max_idx;
                 leaf[p * NT] = d;
                 kidx[p * NT] = (Idx)(first + i);
                 // the other side of every match on the path, fetched together
-                float sv[LEVELS];
+                T sv[LEVELS];
                 int sa[LEVELS];
                 sv[0] = leaf[(p ^ 1) * NT];
                 sa[0] = p ^ 1;
@@ -1177,7 +1185,7 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
                     sv[l] = ival[sib * NT];
                     sa[l] = iarg[sib * NT];
                 }
-                float v = d;
+                T v = d;
                 int a = p;
 #pragma unroll
                 for (int l = 0; l < LEVELS; ++l) {
@@ -1204,12 +1212,12 @@ __global__ __launch_bounds__(64) void knn_tree_kernel_f32(
     }
 
     if (active) {
-        float *od = distance + ((int64_t)b * n1 + qi) * k;
+        T *od = distance + ((int64_t)b * n1 + qi) * k;
         int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
         for (int s = 0; s < k; ++s) {
-            float d = leaf[s * NT];
-            if (d == -__builtin_huge_valf())  // a NaN of the fill phase, still in its slot
-                d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            T d = leaf[s * NT];
+            if (d == -tk_inf<T>())  // a NaN of the fill phase, still in its slot
+                d = tk_dist2<T>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
             od[s] = d;
             oi[s] = (int64_t)kidx[s * NT];
         }
@@ -1325,7 +1333,7 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     int max_idx = iarg[NT];
     int logged = 0;  // entries this lane wrote to its log (may exceed CAP: overflow)
 
-    // MinK's insertion of key j at distance d < max_key (see knn_tree_kernel_f32).
+    // MinK's insertion of key j at distance d < max_key (see knn_tree_kernel).
     auto insert = [&](float d, int j) {
         const int p = max_idx;
         leaf[p * NT] = d;
@@ -1500,32 +1508,32 @@ int knn_tree_split_launch(const float *query, const float *key, float *distance,
     return tk_launch_status();
 }
 
-template <int KMAX, bool IDX16>
-int knn_tree_launch_as(const float *query, const float *key, float *distance, int64_t *index,
+template <int KMAX, bool IDX16, typename T = float>
+int knn_tree_launch_as(const T *query, const T *key, T *distance, int64_t *index,
                        int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    constexpr int LDS_BYTES = KnnTreeLayout<KMAX, IDX16>::BYTES;
+    constexpr int LDS_BYTES = KnnTreeLayout<KMAX, IDX16, T>::BYTES;
     if (LDS_BYTES > 48 * 1024) {
         const int allowed =
-            tk_allow_dynamic_lds<knn_tree_kernel_f32<KMAX, IDX16>>(LDS_BYTES);
+            tk_allow_dynamic_lds<knn_tree_kernel<T, KMAX, IDX16>>(LDS_BYTES);
         if (allowed != TK3D_OK)
             return allowed;
     }
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     if (B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_tree_kernel_f32<KMAX, IDX16>), dim3((unsigned)(B * bpb)), dim3(64),
+    hipLaunchKernelGGL((knn_tree_kernel<T, KMAX, IDX16>), dim3((unsigned)(B * bpb)), dim3(64),
                        LDS_BYTES, s, query, key, distance, index, (int)bpb, n1, n2, k);
     return tk_launch_status();
 }
 
-template <int KMAX>
-int knn_tree_launch(const float *query, const float *key, float *distance, int64_t *index,
+template <int KMAX, typename T = float>
+int knn_tree_launch(const T *query, const T *key, T *distance, int64_t *index,
                     int64_t B, int n1, int n2, int k, hipStream_t s)
 {
     if (n2 <= 65536)
-        return knn_tree_launch_as<KMAX, true>(query, key, distance, index, B, n1, n2, k, s);
-    return knn_tree_launch_as<KMAX, false>(query, key, distance, index, B, n1, n2, k, s);
+        return knn_tree_launch_as<KMAX, true, T>(query, key, distance, index, B, n1, n2, k, s);
+    return knn_tree_launch_as<KMAX, false, T>(query, key, distance, index, B, n1, n2, k, s);
 }
 
 // Any k: the structure lives in the output rows in global memory.
@@ -1933,14 +1941,18 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
                                dim3(KNN_BLOCK), 0, s, query, key, distance, index, (int)bpb,
                                n1, n2, kk);
     } else {
+        // fp64: slots in registers up to k = 16, the LDS tree beyond (k = 64 at B=32,
+        // 2048 x 8192: the register variant pays 2 k selects per insertion on 64-bit values)
         if (k <= 8)
             knn_launch<T, 8>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
         else if (k <= 16)
             knn_launch<T, 16>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
         else if (k <= 32)
-            knn_launch<T, 32>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+            return knn_tree_launch<32, T>(query, key, distance, index, B, n1, n2, kk, s);
         else if (k <= 64)
-            knn_launch<T, 64>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
+            return knn_tree_launch<64, T>(query, key, distance, index, B, n1, n2, kk, s);
+        else if (k <= 128)
+            return knn_tree_launch<128, T>(query, key, distance, index, B, n1, n2, kk, s);
         else
             hipLaunchKernelGGL((knn_global_kernel<T>), dim3((unsigned)(B * bpb)),
                                dim3(KNN_BLOCK), 0, s, query, key, distance, index, (int)bpb,
