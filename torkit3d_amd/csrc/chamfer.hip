@@ -737,7 +737,7 @@ __device__ __forceinline__ float chamfer_fold16(float m, const tk_f32x16 &acc)
 }
 
 template <int NQB, int BLOCK, int STAGE>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(NQB <= 4 ? 4 : 3, NQB <= 4 ? 4 : 3))) void
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(NQB <= 4 ? 4 : 2, NQB <= 4 ? 4 : 2))) void
 chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
 {
     constexpr int NW = BLOCK / TK_WAVE;
@@ -1659,11 +1659,11 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
             int slices = 1;
             while (blocks * slices < 256 && slices < 16 && nkmin / (slices * 2) >= 1024)
                 slices *= 2;
-            // Launches of five workgroups per CU or more even so: six blocks of 32 queries
-            // per wave (768 per workgroup, three waves per SIMD): the key terms a workgroup
-            // stages serve half as many queries again (4.6 % at B=32, N=M=16384).
-            if (slices == 1 && B * ((N1 + 767) / 768 + (N2 + 767) / 768) >= 1280)
-                return chamfer_forward_mfma_launch<6>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+            // Launches that still fill the chip with 1024 queries per workgroup run eight
+            // blocks of 32 queries per wave (two waves per SIMD): the key terms a workgroup
+            // stages then serve twice the queries (8-10 % at B=32, N=M=16384).
+            if (slices == 1 && B * ((N1 + 1023) / 1024 + (N2 + 1023) / 1024) >= 1024)
+                return chamfer_forward_mfma_launch<8>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                                       idx2, s);
             if (blocks * slices >= 96)
                 return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
