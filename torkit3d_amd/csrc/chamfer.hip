@@ -737,7 +737,7 @@ __device__ __forceinline__ float chamfer_fold16(float m, const tk_f32x16 &acc)
 }
 
 template <int NQB, int BLOCK, int STAGE>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(NQB <= 4 ? 4 : 2, NQB <= 4 ? 4 : 2))) void
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
 {
     constexpr int NW = BLOCK / TK_WAVE;
@@ -771,10 +771,6 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
     const float *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
     const float INF = __builtin_huge_valf();
 
-    // Older waves win the issue arbitration, so a wave that starts while three others
-    // sweep on its SIMD waits through their sweeps for every instruction of its prologue:
-    // the phases that are short and latency-bound run at a raised priority.
-    __builtin_amdgcn_s_setprio(2);
     // ---- centre and scale from a strided sample of the key cloud ----
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
     if (nk > 0) {
@@ -905,7 +901,6 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
     fetch(0);
     stash(0, 0);
     __syncthreads();
-    __builtin_amdgcn_s_setprio(0);
     const tk_f32x16 zero = {};
     for (int st = 0; st < nstages; ++st) {
         if (st + 1 < nstages)
@@ -1000,7 +995,6 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
         }
     }
 
-    __builtin_amdgcn_s_setprio(2);
     // ---- the largest centred key norm; a key cloud that left fp16's range ----
     kmax2 = wave_reduce_max(kmax2);
     if (lane == 0)
@@ -1659,12 +1653,6 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
             int slices = 1;
             while (blocks * slices < 256 && slices < 16 && nkmin / (slices * 2) >= 1024)
                 slices *= 2;
-            // Launches that still fill the chip with 1024 queries per workgroup run eight
-            // blocks of 32 queries per wave (two waves per SIMD): the key terms a workgroup
-            // stages then serve twice the queries (8-10 % at B=32, N=M=16384).
-            if (slices == 1 && B * ((N1 + 1023) / 1024 + (N2 + 1023) / 1024) >= 1024)
-                return chamfer_forward_mfma_launch<8>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
-                                                      idx2, s);
             if (blocks * slices >= 96)
                 return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                                       idx2, s, slices);
