@@ -41,8 +41,8 @@ MATRIX_FLOP_PER_PAIR = 32         # executed: a 16-term dot product per pair in 
 
 # HBM bytes per chamfer-forward launch at B=32, N=M=16384, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
-# (profiles/chamfer_forward_filter_B32_N16384.md).
-CHAMFER_TRAFFIC_BYTES = 40.0e6
+# (profiles/chamfer_forward_mfma_B32_N16384.md).
+CHAMFER_TRAFFIC_BYTES = 46.7e6
 
 
 def sphere_cloud(gen, b, n, noise=0.01):
@@ -383,7 +383,7 @@ def secondary_metrics(dev, steps, warmup, cpu):
             lambda: _C.sample_farthest_points_cuda(ap, kk), max(3, steps // 10), 1)
 
     # Roofline per op: algorithmic work of one launch over its measured duration.
-    valu = "fp32 vector ALU, 8 FLOP per pair-distance (top-k upkeep not counted)"
+    valu = "8 algorithmic fp32 FLOP per pair-distance against the fp32 vector peak (the sweep itself runs as fp16 dot products on the matrix cores; top-k upkeep, the rest of the time, on the vector ALUs)"
     roof = {
         "fps_B16_N4096_K1024": dict(
             op_roofline("hbm", "serial chain of 1023 selection steps: latency bound, neither "
