@@ -238,8 +238,7 @@ def test_slot_order_of_the_hand_worked_mink_run(cuda, k, dtype):
 # queues, its stage boundaries and its fallbacks. (Sizes are chosen inside the range where
 # the dispatcher takes this kernel: 65536 queries or more against 2048 keys or more.) ----
 
-def _filter_case(kind, g, k):
-    b, n1, n2 = 8, 8192 + 5, 2048 + 37          # ragged: partial workgroup, partial chunk
+def _filter_case(kind, g, k, b=8, n1=8192 + 5, n2=2048 + 37):  # ragged: partial workgroup, partial chunk
     q, key = uniform_cloud(g, b, n1), uniform_cloud(g, b, n2)
     if kind == "uniform":
         pass
@@ -303,6 +302,27 @@ def _filter_case(kind, g, k):
 def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
     q, key = _filter_case(kind, gen(sum(map(ord, kind)) + k), k)
     check_raw(q, key, k, cuda)
+
+
+# ---- k = 17..32 with 32768 to 131071 queries against 4096 keys or more: the same matrix
+# sweep feeding the LDS tournament tree (one query per lane, two blocks of 32 per wave) ----
+
+@pytest.mark.parametrize("k", [17, 32])
+@pytest.mark.parametrize("kind", ["uniform", "lattice", "far_to_near", "near_to_far",
+                                  "far_from_origin", "separated", "tiny", "huge", "huge_queries",
+                                  "scaled_small", "scaled_large", "far_queries",
+                                  "clusters", "duplicates", "nan_and_inf"])
+def test_tree_kernel_with_matrix_sweep_on_hard_inputs(cuda, kind, k):
+    q, key = _filter_case(kind, gen(sum(map(ord, kind)) + k), k, b=8, n1=4096 + 5, n2=4096 + 37)
+    assert 32768 <= q.shape[0] * q.shape[1] < 131072 and key.shape[1] >= 4096
+    check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("b,n1,n2,k", [(32, 2048, 8192, 32), (16, 2048, 4096, 20), (5, 8000, 4097, 31),
+                                        (2, 20000, 65536, 24), (33, 1000, 4096 + 255, 18)])
+def test_tree_kernel_with_matrix_sweep_shapes(cuda, b, n1, n2, k):
+    g = gen(n1 + n2 + k)
+    check_raw(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), k, cuda)
 
 
 @pytest.mark.parametrize("b,n1,n2,k", [(4, 8192, 8192, 12),     # 32768 queries, long key cloud

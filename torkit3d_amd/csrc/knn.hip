@@ -1224,6 +1224,366 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
     }
 }
 
+// fp32, 17 <= k <= 32 on launches of a chip's worth of queries: the sweep of the pre-filtered kernel
+// on the matrix cores (see knn_filter_kernel_f32, MATRIX) feeding the LDS tournament tree
+// of knn_tree_kernel. A lane owns one query; a wave's 64 queries are two blocks of 32
+// (block h = the lanes of half h), so a chunk of 32 keys is two matrix instructions, the
+// lane collects the 16 sign bits of its rows in both blocks, keeps those of its own block
+// and hands the other 16 to lane ^ 32. The mask is a superset of the keys below the
+// query's maximum (slack 64 u R + 48 u M as above); every candidate is re-evaluated with
+// the canonical arithmetic and inserted under MinK's strict test in ascending key order
+// by the rounds of the tree kernel, so the slots go through exactly MinK's states. A key
+// cloud outside the range of the fp16 pieces (or non-finite) makes the workgroup compute
+// its masks with the exact distances instead, as the tree kernel does; a query outside it
+// takes every key as a candidate.
+template <int KMAX, bool IDX16, int NW>
+__global__ __launch_bounds__(64 * NW) void knn_tree_matrix_kernel_f32(
+    const float *__restrict__ query, const float *__restrict__ key,
+    float *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
+    int n2, int k)
+{
+    using Lay = KnnTreeLayout<KMAX, IDX16>;
+    using Idx = typename Lay::Idx;
+    constexpr int CHUNK = 32;
+    constexpr int NT = 64;
+    constexpr int BLOCK = 64 * NW;
+    constexpr int STAGE = 256;
+    constexpr int PER = (STAGE + BLOCK - 1) / BLOCK;
+    constexpr int HALF = KMAX / 2;
+    constexpr int LEVELS = KMAX == 8 ? 3 : KMAX == 16 ? 4 : KMAX == 32 ? 5 : 6;
+    static_assert((1 << LEVELS) == KMAX, "KMAX must be a power of two from 8 to 64");
+    constexpr int TERM_BYTES = 2 * STAGE * 32;  // two stage buffers of key terms
+    extern __shared__ __align__(16) unsigned char knn_tm_lds[];
+    __shared__ float sred[NW][8];
+    uint4 *const sterm = reinterpret_cast<uint4 *>(knn_tm_lds);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    unsigned char *const mine = knn_tm_lds + TERM_BYTES + wave * Lay::BYTES;
+    float *const leaf = reinterpret_cast<float *>(mine) + lane;
+    Idx *const kidx = reinterpret_cast<Idx *>(mine + Lay::LEAF_BYTES) + lane;
+    float *const ival = reinterpret_cast<float *>(mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES) + lane;
+    unsigned char *const iarg =
+        mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
+
+    const int b = blockIdx.x / blocks_per_batch;
+    const int qi = (blockIdx.x - b * blocks_per_batch) * BLOCK + tid;
+    const bool active = qi < n1;
+    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
+    const float INF = __builtin_huge_valf();
+    float qx = 0, qy = 0, qz = 0;
+    if (active) {
+        const float *q = query + ((int64_t)b * n1 + qi) * 3;
+        qx = q[0];
+        qy = q[1];
+        qz = q[2];
+    }
+
+    // ---- bounding box of the key cloud -> centre; largest centred norm -> scale ----
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    for (int j = tid; j < n2; j += BLOCK) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const float v = K[(int64_t)j * 3 + a];
+            lo[a] = __builtin_fminf(lo[a], v);
+            hi[a] = __builtin_fmaxf(hi[a], v);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            lo[a] = __builtin_fminf(lo[a], __shfl_xor(lo[a], o));
+            hi[a] = __builtin_fmaxf(hi[a], __shfl_xor(hi[a], o));
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            sred[wave][a] = lo[a];
+            sred[wave][3 + a] = hi[a];
+        }
+    }
+    __syncthreads();
+    float cc[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float l = INF, h = -INF;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][a]);
+            h = __builtin_fmaxf(h, sred[w][3 + a]);
+        }
+        cc[a] = 0.5f * l + 0.5f * h;
+    }
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    float kmax2 = 0.0f;
+    for (int j = tid; j < n2; j += BLOCK) {
+        const float x = K[(int64_t)j * 3 + 0] - c0, y = K[(int64_t)j * 3 + 1] - c1,
+                    z = K[(int64_t)j * 3 + 2] - c2;
+        kmax2 = __builtin_fmaxf(kmax2, __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        kmax2 = __builtin_fmaxf(kmax2, __shfl_xor(kmax2, o));
+    if (lane == 0)
+        sred[wave][6] = kmax2;
+    __syncthreads();
+    kmax2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
+    // (a NaN or infinite key coordinate is skipped by the reductions above or makes the
+    // centre non-finite; either way such keys never compare below a maximum and the exact
+    // masks below handle the cloud)
+    const float ext = __builtin_sqrtf(kmax2);
+    const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
+    const bool matrix = (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
+                        (kmax2 < 1e30f) && (ext == 0.0f || (ebits >= -40 && ebits <= 40));  // uniform
+    const float scale =
+        (!matrix || ext == 0.0f) ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
+    const float scale2 = scale * scale;
+    const float kmax = ext * scale * 1.000001f;
+
+    // ---- the query in rescaled units; its terms for both blocks of the wave ----
+    const float px = (qx - c0) * scale, py = (qy - c1) * scale, pz = (qz - c2) * scale;
+    const float qn = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px));
+    const float qnorm = __builtin_sqrtf(qn) * 1.000001f;
+    const bool usable = matrix && qnorm <= 200.0f;  // false for NaN
+    const float rr = kmax + qnorm;
+    const float slack_r = rr * rr * 3.8146973e-06f + 1e-37f * scale2;  // 64 u R
+    uint4 qterm[2];
+    {
+        const float ax = usable ? -2.0f * px : 0.0f, ay = usable ? -2.0f * py : 0.0f,
+                    az = usable ? -2.0f * pz : 0.0f;
+        const float ox = __shfl_xor(ax, 32), oy = __shfl_xor(ay, 32), oz = __shfl_xor(az, 32);
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {  // block hb: the queries of the lanes of half hb
+            const bool own = half == hb;
+            const float X = own ? ax : ox, Y = own ? ay : oy, Z = own ? az : oz;
+            const unsigned sx = tk_f16_split2(X), sy = tk_f16_split2(Y), sz = tk_f16_split2(Z);
+            const unsigned xh = sx & 0xffffu, yh = sy & 0xffffu, zh = sz & 0xffffu;
+            qterm[hb] = half == 0 ? make_uint4(sx, xh | (yh << 16), (sy >> 16) | (yh << 16), 0u)
+                                  : make_uint4(sz, zh | 0x3c000000u, 0x00003c00u, 0u);
+        }
+    }
+
+    auto leaf_parent = [&](int n, float &v, int &a) {
+        const int s = 2 * n - KMAX;
+        const float lv = leaf[s * NT], rv = leaf[(s + 1) * NT];
+        const bool right = rv > lv;
+        v = right ? rv : lv;
+        a = right ? s + 1 : s;
+    };
+
+    // Fill phase: keys 0..k-1 go to slots 0..k-1 (mink.cuh:63-72); unused slots hold -inf.
+    bool frozen = false;
+    for (int s = 0; s < KMAX; ++s) {
+        float d = -INF;
+        if (s < k) {
+            d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            if (d != d) {
+                frozen |= s == 0;
+                d = -INF;  // marks the slot: no real distance is -inf
+            }
+        }
+        leaf[s * NT] = d;
+        kidx[s * NT] = (Idx)s;
+    }
+    for (int n = HALF - 1; n >= 1; --n) {
+        float lv, rv;
+        int la, ra;
+        if (2 * n >= HALF) {
+            leaf_parent(2 * n, lv, la);
+            leaf_parent(2 * n + 1, rv, ra);
+        } else {
+            lv = ival[2 * n * NT];
+            rv = ival[(2 * n + 1) * NT];
+            la = iarg[2 * n * NT];
+            ra = iarg[(2 * n + 1) * NT];
+        }
+        const bool right = rv > lv;
+        ival[n * NT] = right ? rv : lv;
+        iarg[n * NT] = (unsigned char)(right ? ra : la);
+    }
+    float max_key = frozen ? -INF : ival[NT];
+    int max_idx = iarg[NT];
+
+    // ---- key terms, staged STAGE keys at a time in two buffers ----
+    const int nstages = (n2 + STAGE - 1) / STAGE;
+    float pre[PER][3];
+    auto fetch = [&](int st) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int j = r * BLOCK + tid;
+            const int kj = st * STAGE + j;
+            pre[r][0] = pre[r][1] = pre[r][2] = INF;  // past the end
+            if (j < STAGE && kj < n2) {
+                pre[r][0] = K[(int64_t)kj * 3 + 0];
+                pre[r][1] = K[(int64_t)kj * 3 + 1];
+                pre[r][2] = K[(int64_t)kj * 3 + 2];
+            }
+        }
+    };
+    auto stash = [&](int st, int buf) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int j = r * BLOCK + tid;  // key within the stage
+            if (j >= STAGE)
+                continue;
+            const bool exists = st * STAGE + j < n2;
+            const float x = exists ? (pre[r][0] - c0) * scale : 0.0f;
+            const float y = exists ? (pre[r][1] - c1) * scale : 0.0f;
+            const float z = exists ? (pre[r][2] - c2) * scale : 0.0f;
+            const float n = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+            const unsigned sx = tk_f16_split2(x), sy = tk_f16_split2(y), sz = tk_f16_split2(z);
+            const unsigned xh = sx & 0xffffu, yh = sy & 0xffffu, zh = sz & 0xffffu;
+            const unsigned sn = tk_f16_split2(n);
+            const unsigned n0 = exists ? (sn & 0xffffu) : 0x7c00u, n1p = exists ? (sn >> 16) : 0u;
+            // row of the tile: lane half h of the result holds rows 8 a + 4 h + c
+            const int row = ((j & 12) << 1) | ((j & 16) >> 2) | (j & 3);
+            uint4 *t = sterm + buf * (STAGE * 2) + (j >> 5) * 64 + row;
+            t[0] = make_uint4(xh * 0x10001u, (sx >> 16) | (yh << 16), yh | (sy & 0xffff0000u),
+                              0x3c003c00u);
+            t[32] = make_uint4(zh * 0x10001u, (sz >> 16) | (n0 << 16), n1p, 0x3c003c00u);
+        }
+    };
+    if (matrix) {  // uniform
+        __syncthreads();
+        fetch(0);
+        stash(0, 0);
+        __syncthreads();
+    }
+    for (int st = 0; st < nstages; ++st) {
+        const int stage0 = st * STAGE;
+        if (matrix && st + 1 < nstages)
+            fetch(st + 1);
+        const int left = n2 - stage0;
+        const int cnt = left < STAGE ? left : STAGE;
+        for (int c0k = 0; c0k < cnt; c0k += CHUNK) {
+            const int first = stage0 + c0k;  // key index of bit 31
+            unsigned mask = 0u;
+            if (matrix) {
+                const float m = max_key * scale2;
+                const float thr = (m - qn) + __builtin_fmaf(m, 2.8610229e-06f, slack_r);
+                const unsigned tp = tk_f16_split2(-thr);
+                qterm[0].w = half == 0 ? tp : 0u;
+                qterm[1].w = half == 1 ? tp : 0u;
+                const tk_f16x8 ka = __builtin_bit_cast(
+                    tk_f16x8, sterm[(st & 1) * (STAGE * 2) + (c0k >> 5) * 64 + lane]);
+                const tk_f32x16 zero = {};
+                unsigned m16[2];
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        ka, __builtin_bit_cast(tk_f16x8, qterm[g]), zero, 0, 0, 0);
+                    unsigned mm = 0u;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float t = acc[r];
+                        mm = __builtin_amdgcn_alignbit(mm, __builtin_bit_cast(unsigned, t), 31);
+                    }
+                    m16[g] = mm;
+                }
+                const unsigned own = half == 0 ? m16[0] : m16[1];
+                const unsigned recv = __shfl_xor(half == 0 ? m16[1] : m16[0], 32);
+                mask = half == 0 ? ((own << 16) | recv) : ((recv << 16) | own);
+                mask = usable ? mask : 0xffffffffu;
+            } else {
+                const int maxbits = __builtin_bit_cast(int, max_key);
+                for (int i = 0; i < CHUNK; ++i) {
+                    const int j = first + i < n2 ? first + i : n2 - 1;  // clamped, masked below
+                    const float d = tk_dist2<float>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
+                                                    K[(int64_t)j * 3 + 2], qx, qy, qz);
+                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
+                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
+                }
+            }
+            // Keys that do not exist, or that the fill phase took, are no candidates.
+            int vlo = k - first;
+            vlo = vlo < 0 ? 0 : (vlo > CHUNK ? CHUNK : vlo);
+            int vhi = n2 - first;
+            vhi = vhi > CHUNK ? CHUNK : vhi;
+            unsigned valid = (vlo >= CHUNK) ? 0u : (0xffffffffu >> vlo);
+            valid &= (vhi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> vhi);
+            mask = active ? (mask & valid) : 0u;
+
+            // ---- insertion rounds, the next candidate's key in flight during the current ----
+            const float *__restrict__ ck = K + (int64_t)first * 3;
+            bool has = mask != 0u;
+            int i = has ? __builtin_clz(mask) : 0;
+            float ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
+            while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+                mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
+                const bool has_next = mask != 0u;
+                const int i_next = has_next ? __builtin_clz(mask) : 0;
+                const float nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
+                            nz = ck[3 * i_next + 2];
+                const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+                if (has && d < max_key) {
+                    const int p = max_idx;
+                    leaf[p * NT] = d;
+                    kidx[p * NT] = (Idx)(first + i);
+                    // the other side of every match on the path, fetched together
+                    float sv[LEVELS];
+                    int sa[LEVELS];
+                    sv[0] = leaf[(p ^ 1) * NT];
+                    sa[0] = p ^ 1;
+                    leaf_parent(((KMAX + p) >> 1) ^ 1, sv[1], sa[1]);
+#pragma unroll
+                    for (int l = 2; l < LEVELS; ++l) {
+                        const int sib = ((KMAX + p) >> l) ^ 1;
+                        sv[l] = ival[sib * NT];
+                        sa[l] = iarg[sib * NT];
+                    }
+                    float v = d;
+                    int a = p;
+#pragma unroll
+                    for (int l = 0; l < LEVELS; ++l) {
+                        const int node = (KMAX + p) >> l;
+                        // the other side wins from the right only when strictly greater
+                        const bool take = (node & 1) ? !(v > sv[l]) : (sv[l] > v);
+                        v = take ? sv[l] : v;
+                        a = take ? sa[l] : a;
+                        // parents of leaves are not stored; the root lives in max_key / max_idx
+                        if (l >= 1 && l + 1 < LEVELS) {
+                            ival[(node >> 1) * NT] = v;
+                            iarg[(node >> 1) * NT] = (unsigned char)a;
+                        }
+                    }
+                    max_key = v;
+                    max_idx = v != d ? a : p;
+                }
+                has = has_next;
+                i = i_next;
+                ex = nx;
+                ey = ny;
+                ez = nz;
+            }
+        }
+        if (matrix) {
+            if (st + 1 < nstages) {
+                __syncthreads();  // every wave is done with the buffer of the previous stage
+                stash(st + 1, (st + 1) & 1);
+            }
+            __syncthreads();
+        }
+    }
+
+    if (active) {
+        float *od = distance + ((int64_t)b * n1 + qi) * k;
+        int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
+        for (int s = 0; s < k; ++s) {
+            float d = leaf[s * NT];
+            if (d == -INF)  // a NaN of the fill phase, still in its slot
+                d = tk_dist2<float>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            od[s] = d;
+            oi[s] = (int64_t)kidx[s * NT];
+        }
+    }
+}
+
 // The tree kernel for launches with few queries. One wave per 64 queries leaves most of
 // the chip idle when B * N1 is small, and the keys cannot simply be divided among waves:
 // the slot order MinK leaves behind depends on every insertion in key order. But a key
@@ -1534,6 +1894,31 @@ int knn_tree_launch(const T *query, const T *key, T *distance, int64_t *index,
     if (n2 <= 65536)
         return knn_tree_launch_as<KMAX, true, T>(query, key, distance, index, B, n1, n2, k, s);
     return knn_tree_launch_as<KMAX, false, T>(query, key, distance, index, B, n1, n2, k, s);
+}
+
+// The tree kernel with the matrix-core sweep: pays where the launch fills the chip and the
+// key cloud amortises the prologue (two passes over the keys per workgroup).
+// Timed against the plain tree kernel on an MI355X for k = 17..32: 1.1-1.5 times faster
+// for 32768 to 65536 queries against 4096 keys or more, slower with more queries (fewer
+// waves fit beside the staged terms, and a workgroup's waves wait for each other at every
+// stage) and no faster on shorter key clouds; for k <= 16 the register kernel above wins.
+template <int KMAX, int NW>
+int knn_tree_matrix_launch(const float *query, const float *key, float *distance,
+                           int64_t *index, int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    if (n2 > 65536 || n2 < 4096 || B * n1 < 32768 || B * n1 >= 131072)
+        return TK3D_ERR_UNSUPPORTED;
+    constexpr int LDS_BYTES = 2 * 256 * 32 + NW * KnnTreeLayout<KMAX, true>::BYTES;
+    constexpr auto kernel = knn_tree_matrix_kernel_f32<KMAX, true, NW>;
+    const int allowed = tk_allow_dynamic_lds<kernel>(LDS_BYTES);
+    if (allowed != TK3D_OK)
+        return allowed;
+    const int64_t bpb = ((int64_t)n1 + 64 * NW - 1) / (64 * NW);
+    if (B * bpb > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(64 * NW), LDS_BYTES, s, query, key,
+                       distance, index, (int)bpb, n1, n2, k);
+    return tk_launch_status();
 }
 
 // Any k: the structure lives in the output rows in global memory.
@@ -1907,6 +2292,13 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
             // log gets all the spare LDS (1.15-1.5 times faster from 8192 keys on)
             const int rc = knn_tree_split_launch<32, 2, 896>(query, key, distance, index, B, n1,
                                                              n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
+        if (k > 16 && k <= 32) {
+            // a chip's worth of queries on long key clouds: matrix-core sweep into the tree
+            const int rc = knn_tree_matrix_launch<32, 2>(query, key, distance, index, B, n1, n2,
+                                                         kk, s);
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
