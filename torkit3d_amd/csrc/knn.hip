@@ -438,8 +438,7 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 // below 58 u R + 39 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
 // from the centre (rescaled; thr would leave fp16's range) take every key as a candidate.
 template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX>
-__global__ __launch_bounds__(KNN_BLOCK)
-    __attribute__((amdgpu_waves_per_eu(MATRIX && KMAX <= 4 ? 3 : 1))) void knn_filter_kernel_f32(
+__global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
     float eps, int blocks_per_batch, int n1, int n2, int k)
