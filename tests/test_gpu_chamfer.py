@@ -341,7 +341,11 @@ def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
 
 @pytest.mark.parametrize("b,n1,n2", [(1, 4096, 4096), (2, 3000, 5000), (1, 20000, 700),
                                      (1, 777, 65536 + 5), (4, 512, 512), (1, 16384, 16384),
-                                     (1, 8192, 8192), (2, 16384, 9000), (1, 2048, 65536 + 5)])
+                                     (1, 8192, 8192), (2, 16384, 9000), (1, 2048, 65536 + 5),
+                                     # clouds of very different lengths: each direction gets
+                                     # its own number of key slices
+                                     (1, 20000, 2048), (2, 1500, 70000), (3, 100000, 1024),
+                                     (32, 8192, 1024), (1, 1024, 300000)])
 def test_split_sweep_shapes(cuda, b, n1, n2):
     g = gen(n1 * 3 + n2)
     check_forward(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), cuda)
@@ -371,7 +375,8 @@ def test_split_sweep_ties_across_slices_keep_the_lowest_index(cuda, n1, n2, spot
 
 
 @pytest.mark.parametrize("n1,n2", [(1500, 6000),       # vector pre-filter, sliced
-                                   (4096, 16384)])     # matrix pre-filter, sliced
+                                   (4096, 16384),      # matrix pre-filter, sliced
+                                   (1024, 60000)])     # one direction in 59 slices, the other whole
 def test_split_sweep_with_slices_that_hold_no_finite_distance(cuda, n1, n2):
     g = gen(78)
     a, c = uniform_cloud(g, 2, n1), uniform_cloud(g, 2, n2)
