@@ -288,6 +288,8 @@ def _clouds(kind, g, b=2, n1=1500, n2=3001):
             n = cloud.shape[1]
             seen = set((i * n) // 1024 for i in range(1024))
             skipped = [j for j in range(n) if j not in seen]
+            if n <= 1024:            # every point is in the sample
+                continue
             assert len(skipped) >= 3
             cloud[:, skipped[0]] = torch.tensor([40.0, -3.0, 0.5])
             cloud[:, skipped[len(skipped) // 2]] *= 100.0
@@ -318,6 +320,18 @@ def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind):
 # on the matrix cores (scores from two-piece fp16 splits of the centred, rescaled
 # coordinates): the same inputs again at a batch size and cloud lengths that reach it.
 @pytest.mark.parametrize("kind", HARD_KINDS)
+def test_matrix_prefilter_with_a_short_cloud_on_hard_inputs(cuda, kind):
+    # one cloud of a few hundred points against one of a few thousand: the long cloud is cut
+    # into key slices for the short cloud's queries, the short one fills half a stage
+    b, n1, n2 = 40, 2900, 200
+    a, c = _clouds(kind, gen(sum(map(ord, kind)) + 2), b, n1, n2)
+    if kind in ("lattice", "coarse_lattice"):
+        c = c[:, :n2].contiguous()
+    assert b * ((a.shape[1] + 511) // 512 + (c.shape[1] + 511) // 512) >= 96 and a.shape[1] >= 1024
+    check_forward(a.contiguous(), c.contiguous(), cuda)
+
+
+@pytest.mark.parametrize("kind", HARD_KINDS)
 def test_matrix_prefilter_is_exact_on_hard_inputs(cuda, kind):
     b, n1, n2 = 48, 2500, 3001
     assert min(n1 - 400, n2) >= 2048 and b * ((n1 - 400 + 511) // 512 + (n2 + 511) // 512) >= 512
@@ -345,7 +359,10 @@ def test_prefiltered_kernel_shapes(cuda, b, n1, n2):
                                      # clouds of very different lengths: each direction gets
                                      # its own number of key slices
                                      (1, 20000, 2048), (2, 1500, 70000), (3, 100000, 1024),
-                                     (32, 8192, 1024), (1, 1024, 300000)])
+                                     (32, 8192, 1024), (1, 1024, 300000),
+                                     # ... down to key clouds of a few points on one side
+                                     (1, 200000, 512), (1, 100000, 100), (8, 16384, 256),
+                                     (16, 4096, 5), (2, 50000, 1), (3, 70000, 33)])
 def test_split_sweep_shapes(cuda, b, n1, n2):
     g = gen(n1 * 3 + n2)
     check_forward(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), cuda)

@@ -1653,7 +1653,7 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
         // a few workgroups with most of the work: a direction's key cloud is then cut
         // into slices no longer than 1/256 of all the sweeping (and no shorter than 1024
         // keys), each direction on its own (B=1, 200000 x 2048: 1.99 -> 0.07 ms).
-        if (nkmin >= 1024) {
+        if (nkmin >= 1 && (N1 > N2 ? N1 : N2) >= 1024) {
             const int64_t qb[2] = {B * ((N1 + 511) / 512), B * ((N2 + 511) / 512)};
             const int64_t nk[2] = {N2, N1};
             const double sweep = (double)qb[0] * (double)nk[0] + (double)qb[1] * (double)nk[1];
