@@ -332,6 +332,13 @@ def secondary_metrics(dev, steps, warmup, cpu):
         m2 = torch.rand(bb, nn, 3, generator=g).to(dev)
         out["chamfer_fwd_B%d_N%d_ms" % (bb, nn)] = gpu_time_ms(
             lambda: _C.chamfer_distance_forward_cuda(m1, m2), steps, 3)
+    # Clouds of very different lengths (a scan against a model): each direction's key cloud
+    # is sliced on its own, so the short cloud's few queries do not sweep the long one alone.
+    for bb, n1, n2 in ((1, 200000, 2048), (32, 16384, 2048)):
+        m1 = torch.rand(bb, n1, 3, generator=g).to(dev)
+        m2 = torch.rand(bb, n2, 3, generator=g).to(dev)
+        out["chamfer_fwd_B%d_N%d_M%d_ms" % (bb, n1, n2)] = gpu_time_ms(
+            lambda: _C.chamfer_distance_forward_cuda(m1, m2), steps, 3)
 
     # Set-abstraction chain of the stress configuration: B=8, three levels of farthest
     # point sampling, ball query and grouping, each level on the previous level's picks.
