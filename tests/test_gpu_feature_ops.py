@@ -248,7 +248,7 @@ def test_fp32_backward_is_bit_reproducible(cuda):
         assert torch.equal(again[0], cfirst[0]) and torch.equal(again[1], cfirst[1])
 
 
-@pytest.mark.parametrize("where", [100, 2500, 4095])
+@pytest.mark.parametrize("where", [100, 200, 2500, 4095])
 def test_scatter_outlier_missed_by_the_magnitude_sample(cuda, where):
     # The fixed-point scale comes from a 1-in-8 sample of the gradient; a term far above
     # the sampled maximum must send the workgroup through its exact second pass.
@@ -348,3 +348,60 @@ def test_forward_from_rows_longer_than_64_kib(cuda, n1):
     for i in range(3):
         want += torch.gather(feat, 2, index3[:, None, :, i].expand(2, 6, 3000)) * weight[:, None, :, i]
     assert torch.equal(_C.interpolate_forward_cuda(feat, index3, weight), want)
+
+
+@pytest.mark.parametrize("b,c,n1,n2", [
+    (40, 64, 300, 1000),    # 640 jobs of 4 rows: workgroups take a second job
+    (3, 7, 2000, 777),      # a channel group of 3 at the tail, points not a multiple of 64
+    (1, 4, 300, 100000),    # one job per batch: the points are split and merged with atomics
+    (2, 5, 5000, 3000),     # rows of 40 KB: one workgroup of 1024 lanes per CU, 2 rows each
+    (2, 3, 16000, 500),     # one row fills the LDS
+    (1, 1, 1, 1), (2, 2, 5, 63), (1, 130, 64, 65)])
+def test_whole_row_scatter_shapes_retries_and_bad_indices(cuda, b, c, n1, n2):
+    """The whole-row fp32 scatter: shapes on either side of its launch choices, indices
+    outside the row (they contribute nothing), gradients far above the sampled magnitude
+    in some rows (those rows are repeated with exact bounds, in a workgroup's first job and
+    in a later one) and a NaN and an inf in others (those rows are summed in floating
+    point), for interpolation (3 weighted neighbours) and grouping (flattened [n2, 4])."""
+    from torkit3d_amd import _C
+
+    g = gen(b * 1000 + c)
+    # few jobs: the points are split, and the partial sums (each rounded to fp32) meet in
+    # float atomics, a few units in the last place of sums of a thousand terms
+    atol = 2e-5 if n2 >= 100000 else ATOL
+    for k, weighted in ((3, True), (4, False)):
+        index = torch.randint(0, n1, (b, n2, k), generator=g)
+        bad = torch.rand(b, n2, k, generator=g) < 0.02
+        index[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, -1, n1 + 5)
+        go = torch.randn(b, c, n2, generator=g) if weighted else torch.randn(b, c, n2, k, generator=g)
+        flat = go.view(b, c, -1)
+        big = [(0, 0), (b - 1, c - 1), (b // 2, c // 2), (b - 1, 0)]
+        for n, (bi, ci) in enumerate(big):
+            flat[bi, ci, (97 * (n + 1)) % flat.shape[2]] = 3.0e7 * (n + 1)
+        odd = []
+        if b * c > 8:
+            odd = [(0, c - 1, float("nan")), (b - 1, c // 3, float("inf"))]
+            for bi, ci, v in odd:
+                flat[bi, ci, flat.shape[2] // 2] = v
+        if weighted:
+            weight = torch.rand(b, n2, k, generator=g) + 0.05
+            got = _C.interpolate_backward_cuda(go.to(cuda), index.to(cuda), weight.to(cuda), n1)
+            want = oracle.interpolate_backward(go.numpy(), index.numpy(), weight.numpy(), n1, wide=True)
+        else:
+            got = _C.group_points_backward_cuda(go.to(cuda), index.to(cuda), n1)
+            want = oracle.group_backward(go.numpy(), index.numpy(), n1, wide=True)
+        got = got.cpu().numpy()
+        for bi, ci, _ in odd:
+            assert np.array_equal(np.isnan(got[bi, ci]), np.isnan(want[bi, ci]))
+            assert np.array_equal(np.isposinf(got[bi, ci]), np.isposinf(want[bi, ci]))
+            keep = np.isfinite(want[bi, ci])
+            np.testing.assert_allclose(got[bi, ci][keep], want[bi, ci][keep], rtol=RTOL, atol=atol)
+            got[bi, ci] = want[bi, ci]
+        for bi, ci in big:
+            if (bi, ci) in [(o[0], o[1]) for o in odd]:
+                continue
+            # a row is resolved to 2^-40 of its largest term per sum
+            top = float(np.abs(flat[bi, ci].numpy()).max()) * (1.05 if weighted else 1.0)
+            np.testing.assert_allclose(got[bi, ci], want[bi, ci], rtol=RTOL, atol=top * 2.0 ** -40 + atol)
+            got[bi, ci] = want[bi, ci]
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=atol)

@@ -16,15 +16,20 @@
 // (group_points_kernel.cu:26-29).
 //
 // scatter: a workgroup owns CG destination rows [CG][N1] in LDS, streams its
-// share of p with coalesced reads of gout and accumulates with LDS float atomics
-// (ds_add), then writes the rows out with plain coalesced stores - no global
-// atomics and no zero-fill when one workgroup covers all p. When B*C is too
-// small to fill the chip the p range is split over several workgroups that merge
-// into a zero-filled output with global atomics. Rows too long for LDS use
-// global atomics directly. Summation order differs from run to run exactly as in
-// the reference (which uses one global atomicAdd per element,
-// group_points_kernel.cu:63, interpolate_kernel.cu:142).
+// share of p with coalesced reads of gout and accumulates with LDS atomics, then
+// writes the rows out with plain coalesced stores - no global atomics and no
+// zero-fill when one workgroup covers all p. fp32 accumulates in 64-bit fixed point
+// (integer LDS atomics: fast, and the sums do not depend on the order of arrival);
+// fp64, and fp32 rows holding NaN or inf, use floating-point LDS atomics, whose
+// summation order differs from run to run exactly as in the reference (one global
+// atomicAdd per element, group_points_kernel.cu:63, interpolate_kernel.cu:142).
+// When B*C is too small to fill the chip the p range is split over several
+// workgroups that merge into a zero-filled output with global atomics. Rows too
+// long for LDS are accumulated in windows of destinations or, longer still, with
+// global atomics directly.
+
 #include "tk3d_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -339,151 +344,216 @@ __global__ __launch_bounds__(NT) void scatter_lds_kernel(
 // Largest value of a wave, in every lane. Called by whole waves only.
 __device__ __forceinline__ unsigned wave_max_u32(unsigned v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const unsigned t = (unsigned)__shfl_xor((int)v, o);
+    // within rows of 16 lanes through the data-parallel-primitive lane selects (lane ^ 1,
+    // lane ^ 2, mirrored in 8, mirrored in 16), then the four rows through scalar registers
+    auto fold = [&](auto ctrl) {
+        const unsigned t =
+            (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, decltype(ctrl)::value, 0xf, 0xf, false);
         v = t > v ? t : v;
-    }
-    return v;
+    };
+    fold(std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+    fold(std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+    fold(std::integral_constant<int, 0x141>{});  // row_half_mirror
+    fold(std::integral_constant<int, 0x140>{});  // row_mirror
+    const unsigned r0 = (unsigned)__builtin_amdgcn_readlane((int)v, 0);
+    const unsigned r1 = (unsigned)__builtin_amdgcn_readlane((int)v, 16);
+    const unsigned r2 = (unsigned)__builtin_amdgcn_readlane((int)v, 32);
+    const unsigned r3 = (unsigned)__builtin_amdgcn_readlane((int)v, 48);
+    const unsigned a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
 }
 
 
-template <int KK, bool HAS_W, int V, int NT, int CGMAX>
-__global__ __launch_bounds__(NT) void scatter_fixed_kernel(
-    const float *__restrict__ gout, const int64_t *__restrict__ idx,
-    const float *__restrict__ w, float *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg,
-    int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count, int groups, int window)
-{
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);  // [cg][nr]
-    __shared__ unsigned s_maxg[CGMAX];  // bit patterns of non-negative floats order as integers
-    __shared__ unsigned s_maxw;
-    __shared__ int s_kexp[CGMAX];
-    __shared__ double s_scale[CGMAX];
-    __shared__ float s_bound[CGMAX];
-    __shared__ int s_finite, s_exceeded;
-    // Workgroups are handed to the 8 XCDs round-robin by linear id. Every workgroup of a
-    // batch streams that batch's index and weight arrays, so each XCD takes a contiguous
-    // range of logical workgroups (batch slowest): a batch's arrays then come from HBM
-    // once and from one XCD's L2 afterwards, instead of once per XCD.
-    int b, by, bx;
-    {
-        const unsigned long long gx = gridDim.x, gyy = gridDim.y;
-        const unsigned long long total = gx * gyy * gridDim.z;
-        unsigned long long lin = blockIdx.x + gx * (blockIdx.y + gyy * blockIdx.z);
-        const unsigned long long per = total >> 3, full = per << 3;
-        if (lin < full)
-            lin = (lin & 7ull) * per + (lin >> 3);
-        const unsigned long long rest = lin / gx;
-        bx = (int)(lin - rest * gx);
-        by = (int)(rest % gyy);
-        b = (int)(rest / gyy);
-    }
-    // by = destination window * groups + channel group; a workgroup accumulates the
-    // destinations [d0, d0 + nr) of its channels (the whole row when it fits in LDS)
-    const int win = by / groups;
-    const int c0 = (by - win * groups) * cg;
-    const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
-    const int d0 = win * window;
-    const int nr = (d0 + window < n1) ? window : n1 - d0;
-    const int64_t ps = (int64_t)bx * seg_len;
-    const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
-    const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
-    for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
-        __syncthreads();
-        for (int i = threadIdx.x; i < nc * nr; i += NT)
-            acc[i] = 0ull;
-        if (threadIdx.x < CGMAX)
-            s_maxg[threadIdx.x] = 0u;
-        if (threadIdx.x == 0) {
-            s_finite = 1;
-            s_exceeded = 0;
-            s_maxw = HAS_W ? 0u : 0x3f800000u;
-        }
-        __syncthreads();
+template <int CGMAX>
+struct ScatterFixedShared {
+    unsigned maxg[CGMAX];  // bit patterns of non-negative floats order as integers
+    unsigned maxw;
+    int kexp[CGMAX];
+    double scale[CGMAX];
+    float bound[CGMAX];
+    int finite, exceeded;
+};
 
-        // ---- magnitudes: every 8th group first, everything on the second attempt ----
-        if (HAS_W) {
-            // first attempt: one run of 64 consecutive weights in every 512
-            unsigned mw = 0u;
-            const int64_t ne = (pe - ps) * KK;
-            for (int64_t t = threadIdx.x;; t += NT) {
-                const int64_t e = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
-                if (e >= ne)
-                    break;
-                const unsigned bits =
-                    __builtin_bit_cast(unsigned, w[((int64_t)b * np + ps) * KK + e]) & 0x7fffffffu;
-                mw = bits > mw ? bits : mw;
-            }
-            // one LDS atomic per wave: 64 lanes on one address would be served one by one
-            mw = wave_max_u32(mw);
-            if ((threadIdx.x & 63) == 0 && mw != 0u)
-                atomicMax(&s_maxw, mw);
+// Workgroups are handed to the 8 XCDs round-robin by linear id. Every workgroup of a
+// batch streams that batch's index and weight arrays, so each XCD takes a contiguous
+// range of logical workgroups (batch slowest): a batch's arrays then come from HBM
+// once and from one XCD's L2 afterwards, instead of once per XCD.
+__device__ __forceinline__ void scatter_fixed_block(int &b, int &by, int &bx)
+{
+    const unsigned long long gx = gridDim.x, gyy = gridDim.y;
+    const unsigned long long total = gx * gyy * gridDim.z;
+    unsigned long long lin = blockIdx.x + gx * (blockIdx.y + gyy * blockIdx.z);
+    const unsigned long long per = total >> 3, full = per << 3;
+    if (lin < full)
+        lin = (lin & 7ull) * per + (lin >> 3);
+    const unsigned long long rest = lin / gx;
+    bx = (int)(lin - rest * gx);
+    by = (int)(rest % gyy);
+    b = (int)(rest / gyy);
+}
+
+// Clears `acc_elems` accumulators and the shared magnitudes; barriers before and after.
+template <bool HAS_W, int NT, int CGMAX>
+__device__ __forceinline__ void scatter_fixed_clear(ScatterFixedShared<CGMAX> &sh,
+                                                    unsigned long long *acc, int acc_elems)
+{
+    __syncthreads();
+    for (int i = threadIdx.x; i < acc_elems; i += NT)
+        acc[i] = 0ull;
+    if (threadIdx.x < CGMAX)
+        sh.maxg[threadIdx.x] = 0u;
+    if (threadIdx.x == 0) {
+        sh.finite = 1;
+        sh.exceeded = 0;
+        sh.maxw = HAS_W ? 0u : 0x3f800000u;
+    }
+    __syncthreads();
+}
+
+// Bound and scale of each row from the magnitudes in sh.maxg / sh.maxw, which came from a
+// sample (`headroom` 8) or from all the data (just above 1); barriers before and after.
+// sh.finite tells whether every bound is a finite number.
+template <int CGMAX>
+__device__ __forceinline__ void scatter_fixed_scales(ScatterFixedShared<CGMAX> &sh,
+                                                     float headroom, int log2_count)
+{
+    __syncthreads();
+    if (threadIdx.x < CGMAX) {  // lane c works out row c
+        const float maxw = __builtin_bit_cast(float, sh.maxw);
+        const float bound = __builtin_bit_cast(float, sh.maxg[threadIdx.x]) * maxw * headroom;
+        if (!(bound < 3.0e38f))  // NaN or inf (NaN has the largest bit pattern)
+            sh.finite = 0;
+        int e = 0;
+        (void)__builtin_frexpf(bound, &e);  // bound < 2^e (bound == 0 gives e = 0)
+        // one term stays below 2^50 (the conversion is exact to 2^51) and the sum of
+        // `count` terms below 2^62
+        sh.kexp[threadIdx.x] = (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
+        sh.scale[threadIdx.x] = __builtin_ldexp(1.0, sh.kexp[threadIdx.x]);
+        sh.bound[threadIdx.x] = bound;
+    }
+    __syncthreads();
+}
+
+// Clears `acc_elems` accumulators and works out the bound and scale of each of the `nc`
+// rows starting at row `row0` of batch b (points [ps, pe)): from a sample on attempt 0
+// (every 8th run of 64 loads, 8 times headroom), from all the data on attempt 1. Ends
+// with a barrier; sh.finite tells whether every bound is a finite number.
+template <int KK, bool HAS_W, int NT, int CGMAX>
+__device__ __forceinline__ void scatter_fixed_prepare(
+    ScatterFixedShared<CGMAX> &sh, unsigned long long *acc, int acc_elems, int attempt,
+    const float *__restrict__ gout, const float *__restrict__ w, int b, int wc_total, int row0,
+    int nc, int64_t np, int64_t ps, int64_t pe, int vec_ok, int log2_count)
+{
+    constexpr int V = 4;  // points per 16-byte load of the sampler
+    scatter_fixed_clear<HAS_W, NT, CGMAX>(sh, acc, acc_elems);
+
+    if (HAS_W) {
+        // first attempt: one run of 64 consecutive weights in every 512
+        unsigned mw = 0u;
+        const int64_t ne = (pe - ps) * KK;
+        for (int64_t t = threadIdx.x;; t += NT) {
+            const int64_t e = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
+            if (e >= ne)
+                break;
+            const unsigned bits =
+                __builtin_bit_cast(unsigned, w[((int64_t)b * np + ps) * KK + e]) & 0x7fffffffu;
+            mw = bits > mw ? bits : mw;
         }
-        {
-            // first attempt: one run of 64 consecutive 16-byte groups in every 512
-            unsigned mg[CGMAX];
+        // one LDS atomic per wave: 64 lanes on one address would be served one by one
+        mw = wave_max_u32(mw);
+        if ((threadIdx.x & 63) == 0 && mw != 0u)
+            atomicMax(&sh.maxw, mw);
+    }
+    {
+        // first attempt: one run of 64 consecutive 16-byte groups in every 512
+        unsigned mg[CGMAX];
 #pragma unroll
-            for (int c = 0; c < CGMAX; ++c)
-                mg[c] = 0u;
-            for (int64_t t = threadIdx.x;; t += NT) {
-                const int64_t gi = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
-                const int64_t p0 = ps + gi * V;
-                if (p0 >= pe)
-                    break;
-                const bool full = (p0 + V <= pe);
-#pragma unroll
-                for (int c = 0; c < CGMAX; ++c) {
-                    if (c >= nc)
-                        break;
-                    const float *__restrict__ grow = gout + ((int64_t)b * wc_total + wc_off + c0 + c) * np;
-                    float g[V];
-                    if (full && vec_ok && V == 4) {
-                        const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
-                        g[0] = pack.x;
-                        g[1 % V] = pack.y;
-                        g[2 % V] = pack.z;
-                        g[3 % V] = pack.w;
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < V; ++v)
-                            g[v] = (p0 + v < pe) ? grow[p0 + v] : 0.0f;
-                    }
-#pragma unroll
-                    for (int v = 0; v < V; ++v) {
-                        const unsigned bits = __builtin_bit_cast(unsigned, g[v]) & 0x7fffffffu;
-                        mg[c] = bits > mg[c] ? bits : mg[c];
-                    }
-                }
-            }
+        for (int c = 0; c < CGMAX; ++c)
+            mg[c] = 0u;
+        for (int64_t t = threadIdx.x;; t += NT) {
+            const int64_t gi = attempt == 0 ? (t >> 6) * 512 + (t & 63) : t;
+            const int64_t p0 = ps + gi * V;
+            if (p0 >= pe)
+                break;
+            const bool full = (p0 + V <= pe);
 #pragma unroll
             for (int c = 0; c < CGMAX; ++c) {
-                if (c >= nc)  // uniform
+                if (c >= nc)
                     break;
-                const unsigned m = wave_max_u32(mg[c]);
-                if ((threadIdx.x & 63) == 0 && m != 0u)
-                    atomicMax(&s_maxg[c], m);
+                const float *__restrict__ grow = gout + ((int64_t)b * wc_total + row0 + c) * np;
+                float g[V];
+                if (full && vec_ok) {
+                    const float4 pack = *reinterpret_cast<const float4 *>(grow + p0);
+                    g[0] = pack.x;
+                    g[1] = pack.y;
+                    g[2] = pack.z;
+                    g[3] = pack.w;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        g[v] = (p0 + v < pe) ? grow[p0 + v] : 0.0f;
+                }
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    const unsigned bits = __builtin_bit_cast(unsigned, g[v]) & 0x7fffffffu;
+                    mg[c] = bits > mg[c] ? bits : mg[c];
+                }
             }
         }
-        __syncthreads();
-
-        // ---- bounds and scales: lane c < CGMAX works out row c ----
-        if (threadIdx.x < CGMAX) {
-            const float maxw = __builtin_bit_cast(float, s_maxw);
-            const float headroom = attempt == 0 ? 8.0f : 1.000001f;
-            const float bound = __builtin_bit_cast(float, s_maxg[threadIdx.x]) * maxw * headroom;
-            if (!(bound < 3.0e38f))  // NaN or inf (NaN has the largest bit pattern)
-                s_finite = 0;
-            int e = 0;
-            (void)__builtin_frexpf(bound, &e);  // bound < 2^e (bound == 0 gives e = 0)
-            // one term stays below 2^50 (the conversion below is exact to 2^51) and the
-            // sum of `count` terms below 2^62
-            s_kexp[threadIdx.x] = (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
-            s_scale[threadIdx.x] = __builtin_ldexp(1.0, s_kexp[threadIdx.x]);
-            s_bound[threadIdx.x] = bound;
+#pragma unroll
+        for (int c = 0; c < CGMAX; ++c) {
+            if (c >= nc)  // uniform
+                break;
+            const unsigned m = wave_max_u32(mg[c]);
+            if ((threadIdx.x & 63) == 0 && m != 0u)
+                atomicMax(&sh.maxg[c], m);
         }
-        __syncthreads();
-        if (!s_finite)
+    }
+    scatter_fixed_scales<CGMAX>(sh, attempt == 0 ? 8.0f : 1.000001f, log2_count);
+}
+
+// Rows of fixed-point sums back to fp32 and out to memory; `stride` accumulators per row
+// in LDS, the first `nr` of them destinations d0, d0 + 1, ...
+template <int NT, int CGMAX>
+__device__ __forceinline__ void scatter_fixed_write(const ScatterFixedShared<CGMAX> &sh,
+                                                    const unsigned long long *acc, int stride,
+                                                    float *__restrict__ gin, int64_t row0,
+                                                    int nc, int n1, int d0, int nr,
+                                                    int merge_with_atomics)
+{
+    for (int c = 0; c < nc; ++c) {
+        float *__restrict__ dstrow = gin + (row0 + c) * n1 + d0;
+        const unsigned long long *__restrict__ row = acc + c * stride;
+        const int kexp = sh.kexp[c];
+        for (int i = threadIdx.x; i < nr; i += NT) {
+            const float v = (float)__builtin_ldexp((double)(long long)row[i], -kexp);
+            if (merge_with_atomics) {
+                if (v != 0.0f)
+                    unsafeAtomicAdd(&dstrow[i], v);
+            } else {
+                dstrow[i] = v;
+            }
+        }
+    }
+}
+
+// The general procedure for the destinations [d0, d0 + nr) of rows c0 .. c0 + nc - 1 of
+// batch b: attempts `first_attempt` .. 1 in fixed point, then floating point.
+template <int KK, bool HAS_W, int V, int NT, int CGMAX>
+__device__ __forceinline__ void scatter_fixed_attempts(
+    ScatterFixedShared<CGMAX> &sh, unsigned char *smem_raw, int first_attempt,
+    const float *__restrict__ gout, const int64_t *__restrict__ idx,
+    const float *__restrict__ w, float *__restrict__ gin, int b, int c_total, int wc_total,
+    int wc_off, int c0, int nc, int n1, int d0, int nr, int64_t np, int64_t ps, int64_t pe,
+    int merge_with_atomics, int vec_ok, int log2_count)
+{
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);  // [nc][nr]
+    const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+    for (int attempt = first_attempt; attempt < 2; ++attempt) {  // uniform over the workgroup
+        scatter_fixed_prepare<KK, HAS_W, NT, CGMAX>(sh, acc, nc * nr, attempt, gout, w, b,
+                                                    wc_total, wc_off + c0, nc, np, ps, pe,
+                                                    vec_ok, log2_count);
+        if (!sh.finite)
             break;
         struct RowScale {
             double scale;
@@ -494,8 +564,8 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
             gout, idx, w, b, wc_total, c0 + wc_off, nc, d0, nr, np, ps, pe, vec_ok,
             [&](int c) {
                 RowScale r;
-                r.scale = s_scale[c];
-                r.bound = s_bound[c];
+                r.scale = sh.scale[c];
+                r.bound = sh.bound[c];
                 return r;
             },
             [&](const RowScale &r, int c, int dst, float g, float ww) {
@@ -507,23 +577,11 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
                 atomicAdd(&acc[c * nr + dst], q);
             });
         if (exceeded)
-            s_exceeded = 1;
+            sh.exceeded = 1;
         __syncthreads();
-        if (!s_exceeded) {
-            for (int c = 0; c < nc; ++c) {
-                float *__restrict__ dstrow = gin + ((int64_t)b * c_total + c0 + c) * n1 + d0;
-                const unsigned long long *__restrict__ row = acc + c * nr;
-                const int kexp = s_kexp[c];
-                for (int i = threadIdx.x; i < nr; i += NT) {
-                    const float v = (float)__builtin_ldexp((double)(long long)row[i], -kexp);
-                    if (merge_with_atomics) {
-                        if (v != 0.0f)
-                            unsafeAtomicAdd(&dstrow[i], v);
-                    } else {
-                        dstrow[i] = v;
-                    }
-                }
-            }
+        if (!sh.exceeded) {
+            scatter_fixed_write<NT, CGMAX>(sh, acc, nr, gin, (int64_t)b * c_total + c0, nc, n1,
+                                           d0, nr, merge_with_atomics);
             return;
         }
     }
@@ -554,6 +612,313 @@ __global__ __launch_bounds__(NT) void scatter_fixed_kernel(
         }
     }
 }
+
+// Any number of neighbours, rows of any length (in windows of destinations).
+// grid = (segments, windows * channel groups, B).
+template <int KK, bool HAS_W, int V, int NT, int CGMAX>
+__global__ __launch_bounds__(NT) void scatter_fixed_kernel(
+    const float *__restrict__ gout, const int64_t *__restrict__ idx,
+    const float *__restrict__ w, float *__restrict__ gin, int c_total, int wc_total, int wc_off, int n1, int64_t np, int cg,
+    int64_t seg_len, int merge_with_atomics, int vec_ok, int log2_count, int groups, int window)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    __shared__ ScatterFixedShared<CGMAX> sh;
+    int b, by, bx;
+    scatter_fixed_block(b, by, bx);
+    // by = destination window * groups + channel group; a workgroup accumulates the
+    // destinations [d0, d0 + nr) of its channels (the whole row when it fits in LDS)
+    const int win = by / groups;
+    const int c0 = (by - win * groups) * cg;
+    const int nc = (c0 + cg < c_total) ? cg : c_total - c0;
+    const int d0 = win * window;
+    const int nr = (d0 + window < n1) ? window : n1 - d0;
+    const int64_t ps = (int64_t)bx * seg_len;
+    const int64_t pe = (ps + seg_len < np) ? ps + seg_len : np;
+    scatter_fixed_attempts<KK, HAS_W, V, NT, CGMAX>(sh, smem_raw, 0, gout, idx, w, gin, b, c_total,
+                                                    wc_total, wc_off, c0, nc, n1, d0, nr, np, ps,
+                                                    pe, merge_with_atomics, vec_ok, log2_count);
+}
+
+// A value every lane holds, moved to scalar registers.
+__device__ __forceinline__ double scatter_uniform(double v)
+{
+    const unsigned long long bits = __builtin_bit_cast(unsigned long long, v);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)bits);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(bits >> 32));
+    return __builtin_bit_cast(double, ((unsigned long long)hi << 32) | lo);
+}
+
+// Whole rows in LDS, the shapes the layers produce (one neighbour without weights, three
+// with). The general kernel above spends its time waiting: every contribution sits in a
+// branch of its own behind a wait for all loads and all LDS traffic in flight, and each
+// workgroup pays the latencies of clearing, sampling, streaming and writing one after the
+// other. Here:
+//   * a wave takes a run of consecutive chunks of 64 * V points, lane l the points l,
+//     l + 64, ... of a chunk. The indices, weights and the values of all rows for the
+//     next chunk are requested before the current chunk is accumulated; the loop over a
+//     chunk has no branch and no wait on LDS;
+//   * a lane past the end of the points, or an index outside the row, adds into a spare
+//     accumulator of its lane behind the row (64 per row, never read) instead of being
+//     skipped;
+//   * the first chunk of every wave doubles as the sample for the magnitudes (runs of
+//     64 * V points spread evenly over the points), so no separate sampling pass;
+//   * instead of comparing every term with the bound of its row, a lane keeps the largest
+//     |value| per row and the largest |weight| it has seen and compares their product at
+//     the end (NaN and inf have the largest bit patterns). That is stricter than the
+//     term-by-term test, so a pass may be repeated where the general kernel would not
+//     repeat it; a pass that is kept adds exactly the same integers;
+//   * a workgroup works through several jobs (a job = the rows of one channel group of
+//     one batch over one segment of points). Writing a job's rows out also clears the
+//     accumulators, and the first chunks of the next job are requested before that, so
+//     clearing and the first trip to memory cost nothing from the second job on.
+// A repeated pass, and rows with NaN or inf, take the general procedure.
+// grid = (workgroups); jobs = segments * channel groups * B, job j of `gx * gy * gz` has
+// x fastest; LDS = cg * (n1 + 64) accumulators.
+template <int KK, bool HAS_W, int NT, int CG, int V>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
+scatter_fixed_rows_kernel(const float *__restrict__ gout, const int64_t *__restrict__ idx,
+                          const float *__restrict__ w, float *__restrict__ gin, int c_total,
+                          int wc_total, int wc_off, int n1, int64_t np, int cg, int64_t seg_len,
+                          int merge_with_atomics, int vec_ok, int log2_count, unsigned gx,
+                          unsigned gy, unsigned gz)
+{
+    constexpr int NW = NT / 64, SPARE = 64;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(smem_raw);
+    __shared__ ScatterFixedShared<CG> sh;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int stride = n1 + SPARE;
+
+    // Workgroups go to the 8 XCDs round-robin by id. Every job of a batch streams that
+    // batch's index and weight arrays, so each XCD takes a contiguous range of the jobs
+    // (batch slowest) and a batch's arrays come from HBM once, then from one XCD's L2.
+    const unsigned total = gx * gy * gz;
+    unsigned job, job_end, job_step;
+    if (gridDim.x % 8 == 0 && total % 8 == 0) {
+        const unsigned per = total / 8, x = blockIdx.x & 7;
+        job = x * per + (blockIdx.x >> 3);
+        job_end = (x + 1) * per;
+        job_step = gridDim.x >> 3;
+    } else {
+        job = blockIdx.x;
+        job_end = total;
+        job_step = gridDim.x;
+    }
+
+    // what a lane has asked for and not yet used: one chunk of indices, weights and values
+    struct Stage {
+        int64_t j[V][KK];
+        float w[V][KK], g[CG][V];
+    };
+    struct Job {
+        int b, c0, nc;
+        int64_t ps;
+        unsigned len, first, last;  // points, and this wave's chunks [first, last)
+        const float *gbase, *wbase;
+        const int64_t *ibase;
+    };
+    auto decode = [&](unsigned j) {
+        Job jb;
+        const unsigned rest = j / gx;
+        const int bx = (int)(j - rest * gx);
+        jb.b = (int)(rest / gy);
+        jb.c0 = (int)(rest % gy) * cg;
+        jb.nc = (jb.c0 + cg < c_total) ? cg : c_total - jb.c0;
+        jb.ps = (int64_t)bx * seg_len;
+        const int64_t pe = (jb.ps + seg_len < np) ? jb.ps + seg_len : np;
+        jb.len = (unsigned)(pe - jb.ps);  // the host keeps len * KK below 2^31
+        const unsigned nchunks = (jb.len + 64 * V - 1) / (64 * V);
+        const unsigned per_wave = (nchunks + NW - 1) / NW;
+        jb.first = wave * per_wave;
+        jb.last = jb.first + per_wave < nchunks ? jb.first + per_wave : nchunks;
+        jb.gbase = gout + ((int64_t)jb.b * wc_total + wc_off + jb.c0) * np + jb.ps;
+        jb.ibase = idx + ((int64_t)jb.b * np + jb.ps) * KK;
+        jb.wbase = HAS_W ? w + ((int64_t)jb.b * np + jb.ps) * KK : nullptr;
+        return jb;
+    };
+    auto request = [&](Stage &st, const Job &jb, unsigned chunk) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            unsigned po = chunk * (64 * V) + v * 64 + lane;
+            po = po < jb.len ? po : jb.len - 1;
+#pragma unroll
+            for (int i = 0; i < KK; ++i) {
+                st.j[v][i] = jb.ibase[po * KK + i];
+                st.w[v][i] = HAS_W ? jb.wbase[po * KK + i] : 1.0f;
+            }
+#pragma unroll
+            for (int c = 0; c < CG; ++c)
+                if (c < jb.nc)  // uniform
+                    st.g[c][v] = (jb.gbase + (int64_t)c * np)[po];
+        }
+    };
+
+    Stage sa;
+    bool prepared = false;  // accumulators are zero and the first chunk is on its way
+    for (; job < job_end; job += job_step) {
+        const Job jb = decode(job);
+        const int nc = jb.nc;
+        if (!prepared) {
+            if (jb.first < jb.last)
+                request(sa, jb, jb.first);
+            scatter_fixed_clear<HAS_W, NT, CG>(sh, acc, cg * stride);
+        } else {
+            // the barrier that ended the last job's writing is behind us
+            if (threadIdx.x < CG)
+                sh.maxg[threadIdx.x] = 0u;
+            if (threadIdx.x == 0) {
+                sh.finite = 1;
+                sh.exceeded = 0;
+                sh.maxw = HAS_W ? 0u : 0x3f800000u;
+            }
+            __syncthreads();
+        }
+        prepared = false;
+        // magnitudes from the first chunk of every wave
+        if (jb.first < jb.last) {
+            if (HAS_W) {
+                unsigned mw = 0u;
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+#pragma unroll
+                    for (int i = 0; i < KK; ++i) {
+                        const unsigned bits = __builtin_bit_cast(unsigned, sa.w[v][i]) & 0x7fffffffu;
+                        mw = bits > mw ? bits : mw;
+                    }
+                mw = wave_max_u32(mw);
+                if (lane == 0 && mw != 0u)
+                    atomicMax(&sh.maxw, mw);
+            }
+#pragma unroll
+            for (int c = 0; c < CG; ++c) {
+                if (c >= nc)  // uniform
+                    break;
+                unsigned m = 0u;
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    const unsigned bits = __builtin_bit_cast(unsigned, sa.g[c][v]) & 0x7fffffffu;
+                    m = bits > m ? bits : m;
+                }
+                m = wave_max_u32(m);
+                if (lane == 0 && m != 0u)
+                    atomicMax(&sh.maxg[c], m);
+            }
+        }
+        scatter_fixed_scales<CG>(sh, 8.0f, log2_count);
+        bool done = false;
+        if (sh.finite) {
+            const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+            double scale[CG];
+#pragma unroll
+            for (int c = 0; c < CG; ++c)
+                scale[c] = scatter_uniform(sh.scale[c < nc ? c : 0]);
+            unsigned gbits[CG];
+#pragma unroll
+            for (int c = 0; c < CG; ++c)
+                gbits[c] = 0u;
+            unsigned wbits = HAS_W ? 0u : 0x3f800000u;
+            for (unsigned chunk = jb.first; chunk < jb.last; ++chunk) {
+                // copy the chunk out of `sa`, ask for the next one into it, accumulate
+                unsigned slot[V][KK];
+                float wt[V][KK], g[CG][V];
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    const bool inside = chunk * (64 * V) + v * 64 + lane < jb.len;
+#pragma unroll
+                    for (int i = 0; i < KK; ++i) {
+                        const int64_t j = sa.j[v][i];
+                        slot[v][i] = (inside && (unsigned long long)j < (unsigned long long)n1)
+                                         ? (unsigned)j
+                                         : (unsigned)n1 + lane;
+                        wt[v][i] = sa.w[v][i];
+                        if (HAS_W) {
+                            const unsigned bits =
+                                __builtin_bit_cast(unsigned, wt[v][i]) & 0x7fffffffu;
+                            wbits = bits > wbits ? bits : wbits;
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < CG; ++c)
+                        g[c][v] = sa.g[c][v];
+                }
+                if (chunk + 1 < jb.last)  // uniform
+                    request(sa, jb, chunk + 1);
+#pragma unroll
+                for (int c = 0; c < CG; ++c) {
+                    if (c >= nc)  // uniform
+                        break;
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const unsigned bits = __builtin_bit_cast(unsigned, g[c][v]) & 0x7fffffffu;
+                        gbits[c] = bits > gbits[c] ? bits : gbits[c];
+#pragma unroll
+                        for (int i = 0; i < KK; ++i) {
+                            const float term = HAS_W ? g[c][v] * wt[v][i] : g[c][v];
+                            const double d = __builtin_fma((double)term, scale[c], MAGIC);
+                            const unsigned long long q =
+                                __builtin_bit_cast(unsigned long long, d) -
+                                __builtin_bit_cast(unsigned long long, MAGIC);
+                            atomicAdd(&acc[(unsigned)c * (unsigned)stride + slot[v][i]], q);
+                        }
+                    }
+                }
+            }
+            bool exceeded = false;
+#pragma unroll
+            for (int c = 0; c < CG; ++c)
+                if (c < nc)
+                    exceeded = exceeded || !(__builtin_bit_cast(float, gbits[c]) *
+                                                 __builtin_bit_cast(float, wbits) <=
+                                             sh.bound[c]);  // also NaN
+            if (exceeded)
+                sh.exceeded = 1;
+            __syncthreads();
+            done = !sh.exceeded;
+        }
+        const bool more = job + job_step < job_end;
+        if (done) {
+            // the next job's first chunks fly while this job's rows are written and cleared
+            if (more) {
+                const Job nx = decode(job + job_step);
+                if (nx.first < nx.last)
+                    request(sa, nx, nx.first);
+                prepared = true;
+            }
+            for (int c = 0; c < nc; ++c) {
+                float *__restrict__ dstrow = gin + ((int64_t)jb.b * c_total + jb.c0 + c) * n1;
+                unsigned long long *__restrict__ row = acc + c * stride;
+                const int kexp = sh.kexp[c];
+                for (int i = threadIdx.x; i < n1; i += NT) {
+                    const unsigned long long q = row[i];
+                    row[i] = 0ull;
+                    // (double)(long long)q in one rounding: high word times 2^32 is exact
+                    const double d = __builtin_fma((double)(int)(unsigned)(q >> 32), 4294967296.0,
+                                                   (double)(unsigned)q);
+                    const float v = (float)__builtin_ldexp(d, -kexp);
+                    if (merge_with_atomics) {
+                        if (v != 0.0f)
+                            unsafeAtomicAdd(&dstrow[i], v);
+                    } else {
+                        dstrow[i] = v;
+                    }
+                }
+            }
+            __syncthreads();
+        } else {
+            const int64_t pe = jb.ps + jb.len;
+            scatter_fixed_attempts<KK, HAS_W, 4, NT, CG>(sh, smem_raw, 1, gout, idx, w, gin, jb.b,
+                                                         c_total, wc_total, wc_off, jb.c0, nc, n1,
+                                                         0, n1, np, jb.ps, pe, merge_with_atomics,
+                                                         vec_ok, log2_count);
+        }
+    }
+}
+
+// The kernel above as a type, for the launch helper of the host code.
+template <int KK, bool HAS_W, int NT, int CG, int V>
+using ScatterRowsKernel =
+    std::integral_constant<decltype(&scatter_fixed_rows_kernel<KK, HAS_W, NT, CG, V>),
+                           &scatter_fixed_rows_kernel<KK, HAS_W, NT, CG, V>>;
 
 // Rows too long for LDS: one global atomic per contribution into a zero-filled
 // output.
@@ -703,8 +1068,67 @@ int scatter(const T *gout, const int64_t *idx, const T *w, int64_t B, int64_t C,
         const int64_t windows = (N1 + MAX_WINDOW - 1) / MAX_WINDOW;
         const int64_t window = ((N1 + windows - 1) / windows + 3) / 4 * 4;
         const int64_t acc_row = window * 8;
+        const int vec_ok = (((uintptr_t)gout & 15) == 0) && ((NP * 4) % 16 == 0);
+        if constexpr ((KK == 1 && !HAS_W) || (KK == 3 && HAS_W)) {
+            // Whole rows in LDS: the branch-free kernel, as two workgroups of 512 lanes and
+            // up to 4 rows per CU when four rows fit in 72 KiB, else one workgroup of 1024
+            // lanes with as many rows (4 at most) as fit in 132 KiB. The grid is what the
+            // chip holds at once; the workgroups share out the jobs.
+            constexpr int64_t ROWS_LDS = 132 * 1024, HALF_LDS = 72 * 1024;
+            constexpr int PTS = KK == 1 ? 2 : 1;  // points per lane and chunk
+            const int64_t row = (N1 + 64) * 8;
+            if (windows == 1 && row <= ROWS_LDS) {
+                const bool two = 4 * row <= HALF_LDS;
+                const int64_t nt = two ? 512 : 1024;
+                int cg = 4;
+                while (cg > 1 && (cg * row > (two ? HALF_LDS : ROWS_LDS) || cg > C))
+                    cg /= 2;
+                // Prefer more jobs over wider channel groups until every CU has work.
+                while (cg > 2 && B * ((C + cg - 1) / cg) < (two ? 512 : 256))
+                    cg /= 2;
+                const int64_t gy = (C + cg - 1) / cg;
+                int64_t nseg = 1;
+                const int64_t groups = B * gy;
+                if (groups < 128) {
+                    nseg = (256 + groups - 1) / groups;
+                    const int64_t max_seg = (NP + 8 * nt - 1) / (8 * nt);
+                    if (nseg > max_seg)
+                        nseg = max_seg;
+                    if (nseg < 1)
+                        nseg = 1;
+                }
+                int64_t seg_len = (NP + nseg - 1) / nseg;
+                seg_len = (seg_len + 15) / 16 * 16;
+                nseg = (NP + seg_len - 1) / seg_len;
+                const int64_t jobs = nseg * gy * B;
+                if (jobs < ((int64_t)1 << 31) && seg_len * KK < ((int64_t)1 << 31)) {
+                    int log2_count = 1;
+                    while (((int64_t)1 << log2_count) < seg_len * KK + 1)
+                        ++log2_count;
+                    if (nseg > 1)
+                        hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)zero_blocks),
+                                           dim3(GS_BLOCK), 0, s, gin, out_elems);
+                    const int64_t resident = (int64_t)tk_cu_count() * (two ? 2 : 1);
+                    const int64_t wgs = jobs < resident ? jobs : resident;
+                    auto launch = [&](auto kernel_tag, int threads) {
+                        constexpr auto kernel = decltype(kernel_tag)::value;
+                        const int allowed = tk_allow_dynamic_lds<kernel>((int)ROWS_LDS);
+                        if (allowed != TK3D_OK)
+                            return allowed;
+                        hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(threads),
+                                           (size_t)(cg * row), s, gout, idx, w, gin, (int)C,
+                                           (int)wc_total, (int)wc_off, (int)N1, NP, cg, seg_len,
+                                           nseg > 1 ? 1 : 0, vec_ok, log2_count, (unsigned)nseg,
+                                           (unsigned)gy, (unsigned)B);
+                        return tk_launch_status();
+                    };
+                    if (two)
+                        return launch(ScatterRowsKernel<KK, HAS_W, 512, 4, PTS>{}, 512);
+                    return launch(ScatterRowsKernel<KK, HAS_W, 1024, 4, PTS>{}, 1024);
+                }
+            }
+        }
         if (windows <= MAX_WINDOWS) {
-            const int vec_ok = (((uintptr_t)gout & 15) == 0) && ((NP * 4) % 16 == 0);
             int cg = CGMAX;
             while (cg > 1 && (cg * acc_row > FIXED_LDS || cg > C))
                 cg /= 2;

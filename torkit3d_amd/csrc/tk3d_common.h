@@ -126,6 +126,22 @@ template <auto Kernel> static inline int tk_allow_dynamic_lds(int bytes)
     return TK3D_OK;
 }
 
+// Compute units of the current device (256 when the query fails), looked up once per device.
+static inline int tk_cu_count()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 256;
+    int n = cached[dev].load(std::memory_order_acquire);
+    if (n > 0)
+        return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    cached[dev].store(n, std::memory_order_release);
+    return n;
+}
+
 // True when a*b*c... of non-negative sizes fits in int64 and is below `limit`.
 static inline bool tk_fits(int64_t limit, int64_t a, int64_t b = 1, int64_t c = 1,
                            int64_t d = 1)
