@@ -189,6 +189,42 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
         }
         if (p0 + (int64_t)NT * V < pe)
             fetch(p0 + (int64_t)NT * V);
+        // Every lane of the wave inside the points and every index inside the row (the
+        // usual case): all LDS reads of a channel are issued together and nothing is
+        // predicated. Otherwise each read sits behind a test of its own.
+        bool plain = p0 + (V - 1) * 64 < pe;
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+#pragma unroll
+            for (int i = 0; i < KK; ++i)
+                plain = plain && src[v][i] >= 0;
+        if (__all(plain)) {
+#pragma unroll 4
+            for (int c = 0; c < nc; ++c) {
+                const T *row = rows + c * n1;
+                T *__restrict__ orow = out + ((int64_t)b * wc_total + wc_off + c0 + c) * np;
+                T x[V][KK];
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+#pragma unroll
+                    for (int i = 0; i < KK; ++i)
+                        x[v][i] = row[src[v][i]];
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    T val = x[v][0];
+                    if (HAS_W) {
+                        // out = 0; out = fma(in, w, out) per neighbour, in slot order
+                        // (interpolate_kernel.cu:31-42 under default contraction).
+                        val = (T)0;
+#pragma unroll
+                        for (int i = 0; i < KK; ++i)
+                            val = tk_fma<T>(x[v][i], wt[v][i], val);
+                    }
+                    __builtin_nontemporal_store(val, &orow[p0 + v * 64]);
+                }
+            }
+            continue;
+        }
 #pragma unroll 4
         for (int c = 0; c < nc; ++c) {
             const T *row = rows + c * n1;
