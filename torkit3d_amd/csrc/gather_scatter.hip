@@ -924,18 +924,28 @@ scatter_fixed_rows_kernel(const float *__restrict__ gout, const int64_t *__restr
                 float *__restrict__ dstrow = gin + ((int64_t)jb.b * c_total + jb.c0 + c) * n1;
                 unsigned long long *__restrict__ row = acc + c * stride;
                 const int kexp = sh.kexp[c];
-                for (int i = threadIdx.x; i < n1; i += NT) {
-                    const unsigned long long q = row[i];
-                    row[i] = 0ull;
-                    // (double)(long long)q in one rounding: high word times 2^32 is exact
-                    const double d = __builtin_fma((double)(int)(unsigned)(q >> 32), 4294967296.0,
-                                                   (double)(unsigned)q);
-                    const float v = (float)__builtin_ldexp(d, -kexp);
-                    if (merge_with_atomics) {
-                        if (v != 0.0f)
-                            unsafeAtomicAdd(&dstrow[i], v);
-                    } else {
-                        dstrow[i] = v;
+                constexpr int U = 4;  // accumulators fetched together
+                for (int i0 = threadIdx.x; i0 < n1; i0 += NT * U) {
+                    unsigned long long q[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        q[u] = i0 + u * NT < n1 ? row[i0 + u * NT] : 0ull;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int i = i0 + u * NT;
+                        if (i >= n1)
+                            break;
+                        row[i] = 0ull;
+                        // (double)(long long)q in one rounding: high word times 2^32 is exact
+                        const double d = __builtin_fma((double)(int)(unsigned)(q[u] >> 32),
+                                                       4294967296.0, (double)(unsigned)q[u]);
+                        const float v = (float)__builtin_ldexp(d, -kexp);
+                        if (merge_with_atomics) {
+                            if (v != 0.0f)
+                                unsafeAtomicAdd(&dstrow[i], v);
+                        } else {
+                            dstrow[i] = v;
+                        }
                     }
                 }
             }
