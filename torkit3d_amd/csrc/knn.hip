@@ -1593,11 +1593,13 @@ __global__ __launch_bounds__(64 * NW) void knn_tree_matrix_kernel_f32(
 // logs the keys it inserts (a superset of what the whole sequence would insert from that
 // slice); then wave 0 replays the logs slice by slice, in key order, against its own
 // structure with the usual strict test. A log that overflows makes wave 0 sweep that
-// slice in full instead. The result is MinK's, slot for slot.
+// slice in full instead. The result is MinK's, slot for slot. A log entry is the key's
+// position within its slice in 16 bits, so a slice has at most 65536 keys.
 template <int KMAX, bool IDX16, int S, int CAP> struct KnnSplitLayout {
     using Tree = KnnTreeLayout<KMAX, IDX16>;
     using Idx = typename Tree::Idx;
-    static constexpr int LOG_BYTES = (int)sizeof(Idx) * CAP * 64;
+    using LogIdx = unsigned short;  // a logged key, counted from the start of its slice
+    static constexpr int LOG_BYTES = (int)sizeof(LogIdx) * CAP * 64;
     static constexpr int LOGS_AT = S * Tree::BYTES;          // S trees, then S - 1 logs
     static constexpr int BYTES = LOGS_AT + (S - 1) * LOG_BYTES;  // (wave 0 keeps none)
 };
@@ -1611,6 +1613,7 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     using Lay = KnnTreeLayout<KMAX, IDX16>;
     using Split = KnnSplitLayout<KMAX, IDX16, S, CAP>;
     using Idx = typename Lay::Idx;
+    using LogIdx = typename Split::LogIdx;
     constexpr int CHUNK = 32;
     constexpr int NT = 64;
     constexpr int HALF = KMAX / 2;
@@ -1628,10 +1631,10 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     unsigned char *const iarg =
         mine + Lay::LEAF_BYTES + Lay::KIDX_BYTES + Lay::IVAL_BYTES + lane;
     auto log_of = [&](int w) {  // w >= 1
-        return reinterpret_cast<Idx *>(knn_split_lds + Split::LOGS_AT +
-                                       (w - 1) * Split::LOG_BYTES) + lane;
+        return reinterpret_cast<LogIdx *>(knn_split_lds + Split::LOGS_AT +
+                                          (w - 1) * Split::LOG_BYTES) + lane;
     };
-    Idx *const log = log_of(wave > 0 ? wave : 1);  // wave 0 never writes one
+    LogIdx *const log = log_of(wave > 0 ? wave : 1);  // wave 0 never writes one
 
     const int b = blockIdx.x / blocks_per_batch;
     const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
@@ -1727,6 +1730,7 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
 
     // Sweep of the keys [k_begin, k_end) in chunks of 32, inserting (and, for the waves
     // other than 0, logging) as the tree kernel does. `skip_below`: keys the fill took.
+    const int log_base = wave * slice_len;  // first key of this wave's slice
     auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
         for (int first = k_begin; first < k_end; first += CHUNK) {
             const int maxbits = __builtin_bit_cast(int, max_key);
@@ -1771,7 +1775,7 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
                     insert(d, first + i);
                     if (write_log) {
                         if (logged < CAP)
-                            log[logged * NT] = (Idx)(first + i);
+                            log[logged * NT] = (LogIdx)(first + i - log_base);
                         ++logged;
                     }
                 }
@@ -1806,14 +1810,14 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
             sweep(w_begin, w_end, 0, false);
             continue;
         }
-        const Idx *__restrict__ wl = log_of(w);
+        const LogIdx *__restrict__ wl = log_of(w);
         int r = 0;
         bool has = r < count;
-        int j = has ? (int)wl[0] : w_begin;
+        int j = w_begin + (has ? (int)wl[0] : 0);
         float ex = K[(int64_t)j * 3 + 0], ey = K[(int64_t)j * 3 + 1], ez = K[(int64_t)j * 3 + 2];
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
             const bool has_next = r + 1 < count;
-            const int j_next = has_next ? (int)wl[(r + 1) * NT] : w_begin;
+            const int j_next = w_begin + (has_next ? (int)wl[(r + 1) * NT] : 0);
             const float nx = K[(int64_t)j_next * 3 + 0], ny = K[(int64_t)j_next * 3 + 1],
                         nz = K[(int64_t)j_next * 3 + 2];
             const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
@@ -1847,8 +1851,6 @@ template <int KMAX, int S, int CAP>
 int knn_tree_split_launch(const float *query, const float *key, float *distance,
                           int64_t *index, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    using Split = KnnSplitLayout<KMAX, true, S, CAP>;
-    static_assert(Split::BYTES + 64 * S * 4 <= 160 * 1024, "LDS of one CU");
     int slice_len = (n2 + S - 1) / S;
     slice_len = (slice_len + 31) / 32 * 32;
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
@@ -1856,15 +1858,27 @@ int knn_tree_split_launch(const float *query, const float *key, float *distance,
     // for k <= 8, 4096 for k <= 16, 8192 for k <= 32, and only while every workgroup has a
     // CU to itself.
     constexpr int MIN_KEYS = KMAX <= 8 ? 2048 : KMAX <= 16 ? 4096 : 8192;
-    if (n2 > 65536 || n2 < MIN_KEYS || slice_len < k || B * bpb > 256)
+    // (a log holds 16-bit positions within its slice)
+    if (n2 < MIN_KEYS || slice_len < k || slice_len > 65536 || B * bpb > 256)
         return TK3D_ERR_UNSUPPORTED;
-    constexpr auto kernel = knn_tree_split_kernel_f32<KMAX, true, S, CAP>;
-    const int allowed = tk_allow_dynamic_lds<kernel>(Split::BYTES);
-    if (allowed != TK3D_OK)
-        return allowed;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(64 * S), Split::BYTES, s, query,
-                       key, distance, index, (int)bpb, n1, n2, k, slice_len);
-    return tk_launch_status();
+    auto launch = [&](auto wide) {
+        // key indices of the slots in LDS: 16 bits up to 65536 keys, else 32 bits and
+        // slightly shorter logs (a slice whose log overflows is swept again by wave 0)
+        constexpr bool IDX16 = !decltype(wide)::value;
+        constexpr int LOG = IDX16 ? CAP : CAP - 16 * S;
+        using Split = KnnSplitLayout<KMAX, IDX16, S, LOG>;
+        static_assert(Split::BYTES + 64 * S * 4 <= 160 * 1024, "LDS of one CU");
+        constexpr auto kernel = knn_tree_split_kernel_f32<KMAX, IDX16, S, LOG>;
+        const int allowed = tk_allow_dynamic_lds<kernel>(Split::BYTES);
+        if (allowed != TK3D_OK)
+            return allowed;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(64 * S), Split::BYTES, s,
+                           query, key, distance, index, (int)bpb, n1, n2, k, slice_len);
+        return tk_launch_status();
+    };
+    if (n2 <= 65536)
+        return launch(std::false_type{});
+    return launch(std::true_type{});
 }
 
 template <int KMAX, bool IDX16, typename T = float>
@@ -2104,7 +2118,8 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
                     insert(d, first + i);
                     if (write_log) {
                         if (logged < CAP)
-                            s_log[wave - 1][logged][lane] = (unsigned short)(first + i);
+                            s_log[wave - 1][logged][lane] =
+                                (unsigned short)(first + i - wave * slice_len);  // within the slice
                         ++logged;
                     }
                 }
@@ -2138,11 +2153,12 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
         }
         int r = 0;
         bool has = r < count;
-        int j = has ? (int)s_log[w - 1][0][lane] : w_begin;
+        int j = w_begin + (has ? (int)s_log[w - 1][0][lane] : 0);
         float d = dist_to(j);
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
             const bool has_next = r + 1 < count;
-            const int j_next = has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : w_begin;
+            const int j_next =
+                w_begin + (has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : 0);
             const float d_next = dist_to(j_next);
             if (has && d < max_key)
                 insert(d, j);
@@ -2185,7 +2201,9 @@ int knn_small_split_launch(const float *query, const float *key, float *distance
     // (timed on an MI355X, 1024 to 65536 keys); with 65536 queries only from 16384 keys on
     // (1.2-1.3 times), slower otherwise.
     const int64_t groups = B * bpb;
-    if (n2 > 65536 || n2 < 1024 || slice_len < k || groups > 1024 || (groups > 512 && n2 < 16384))
+    // (a log holds 16-bit positions within its slice)
+    if (slice_len > 65536 || n2 < 1024 || slice_len < k || groups > 1024 ||
+        (groups > 512 && n2 < 16384))
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((knn_small_split_kernel_f32<SOA, WEIGHTS, CAP>), dim3((unsigned)(B * bpb)),
                        dim3(64 * S), 0, s, query, key, distance, index, weight, eps, (int)bpb, n1,
