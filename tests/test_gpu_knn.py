@@ -209,19 +209,21 @@ def test_shared_key_sweep_for_small_k_on_hard_inputs(cuda, k):
 @pytest.mark.parametrize("b,n1,n2,k", [(1, 100, 262144, 3), (2, 70, 65537, 1), (1, 130, 100000, 16),
                                         (1, 64, 131072, 32), (1, 50, 70000, 20),
                                         (1, 100, 262145, 4), (1, 40, 131073, 17),
-                                        (2, 90, 150001, 8)])
+                                        (2, 90, 150001, 8), (1, 60, 600000, 3),
+                                        (1, 40, 300001, 16), (1, 30, 400000, 32)])
 def test_shared_key_sweep_beyond_65536_keys(cuda, b, n1, n2, k):
     """Few queries against key clouds too long for 16-bit key indices: the slots hold 32-bit
-    indices and the logs positions within a slice (up to 65536 keys per slice: 262144 keys
-    for k <= 16, 131072 for k <= 32; one key more takes another kernel)."""
+    indices and the logs positions within a slice of at most 65536 keys; clouds longer than
+    the waves' slices together (262144 keys for k <= 16, 131072 for k <= 32) are taken in
+    several groups of slices."""
     g = gen(n1 + n2 + k)
     check_raw(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), k, cuda)
 
 
+@pytest.mark.parametrize("n2", [90001, 300000])
 @pytest.mark.parametrize("k", [2, 7, 16, 30])
-def test_shared_key_sweep_beyond_65536_keys_on_hard_inputs(cuda, k):
+def test_shared_key_sweep_beyond_65536_keys_on_hard_inputs(cuda, k, n2):
     g = gen(43)
-    n2 = 90001
     # far-to-near keys: every key is inserted and every log overflows
     q = uniform_cloud(g, 1, 80) * 0.01
     r = torch.linspace(5.0, 0.1, n2)
@@ -229,13 +231,14 @@ def test_shared_key_sweep_beyond_65536_keys_on_hard_inputs(cuda, k):
     check_raw(q, key + 1e-5 * uniform_cloud(g, 1, n2), k, cuda)
     # exact ties, also across slices
     check_raw(lattice_cloud(g, 1, 100, 4), lattice_cloud(g, 1, n2, 4), k, cuda)
-    # NaN in the fill, at the start of the slices (four of 22528 keys, two of 45024), in a
+    # NaN in the fill, at the start of slices (90001 keys: four of 22528, two of 45024;
+    # 300000 keys: two groups of four slices of 37504, three groups of two of 50016), in a
     # run that covers a slice boundary; infinite keys at the end
     q, key = uniform_cloud(g, 1, 100), uniform_cloud(g, 1, n2)
     key[0, 0, 1] = float("nan")
-    key[0, 22528, 2] = float("nan")
-    key[0, 45024, 0] = float("nan")
-    key[0, 45056, 0] = float("nan")
+    for j in (22528, 45024, 45056, 37504, 150016, 100032, 200064):
+        if j < n2:
+            key[0, j, j % 3] = float("nan")
     key[0, 67500:67700] = float("nan")
     key[0, n2 - 2:] = float("inf")
     check_raw(q, key, k, cuda)

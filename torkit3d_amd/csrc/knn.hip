@@ -1594,7 +1594,8 @@ __global__ __launch_bounds__(64 * NW) void knn_tree_matrix_kernel_f32(
 // slice); then wave 0 replays the logs slice by slice, in key order, against its own
 // structure with the usual strict test. A log that overflows makes wave 0 sweep that
 // slice in full instead. The result is MinK's, slot for slot. A log entry is the key's
-// position within its slice in 16 bits, so a slice has at most 65536 keys.
+// position within its slice in 16 bits, so a slice has at most 65536 keys; longer clouds
+// are taken in groups of S slices, wave 0 replaying each group before the next is swept.
 template <int KMAX, bool IDX16, int S, int CAP> struct KnnSplitLayout {
     using Tree = KnnTreeLayout<KMAX, IDX16>;
     using Idx = typename Tree::Idx;
@@ -1659,6 +1660,9 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     // Slots: wave 0 fills them with keys 0..k-1 (mink.cuh:63-72; unused slots hold -inf);
     // the other waves start from k empty slots (+inf), which any real distance displaces.
     bool frozen = false;
+    float max_key = 0.0f;
+    int max_idx = 0;
+    auto start_slots = [&]() {
     for (int s = 0; s < KMAX; ++s) {
         float d = -__builtin_huge_valf();
         if (s < k) {
@@ -1691,8 +1695,10 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
         ival[n * NT] = right ? rv : lv;
         iarg[n * NT] = (unsigned char)(right ? ra : la);
     }
-    float max_key = frozen ? -__builtin_huge_valf() : ival[NT];
-    int max_idx = iarg[NT];
+    max_key = frozen ? -__builtin_huge_valf() : ival[NT];
+    max_idx = iarg[NT];
+    };
+    start_slots();
     int logged = 0;  // entries this lane wrote to its log (may exceed CAP: overflow)
 
     // MinK's insertion of key j at distance d < max_key (see knn_tree_kernel).
@@ -1730,7 +1736,7 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
 
     // Sweep of the keys [k_begin, k_end) in chunks of 32, inserting (and, for the waves
     // other than 0, logging) as the tree kernel does. `skip_below`: keys the fill took.
-    const int log_base = wave * slice_len;  // first key of this wave's slice
+    int log_base = 0;  // first key of the slice this wave is sweeping
     auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
         for (int first = k_begin; first < k_end; first += CHUNK) {
             const int maxbits = __builtin_bit_cast(int, max_key);
@@ -1788,49 +1794,64 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
         }
     };
 
-    const int k_begin = wave * slice_len;
-    const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
-    if (wave == 0)
-        sweep(0, k_end, k, false);
-    else if (k_begin < n2)
-        sweep(k_begin, k_end, 0, true);
-    s_count[wave][lane] = logged;
-    __syncthreads();
+    // The keys are taken in groups of S slices (one group unless the cloud is longer than
+    // S slices of 65536 keys): wave 0 carries its slots from group to group, the others
+    // start every group from empty slots.
+    for (int g0 = 0; g0 < n2; g0 += S * slice_len) {  // uniform over the workgroup
+        const int k_begin = g0 + wave * slice_len;
+        const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
+        log_base = k_begin;
+        if (wave == 0) {
+            sweep(k_begin, k_end, g0 == 0 ? k : 0, false);
+        } else {
+            if (g0 > 0)
+                start_slots();
+            logged = 0;
+            if (k_begin < n2)
+                sweep(k_begin, k_end, 0, true);
+        }
+        s_count[wave][lane] = logged;
+        __syncthreads();
+        if (wave == 0) {
+            // ---- wave 0 replays the other slices of the group in key order ----
+            for (int w = 1; w < S; ++w) {
+                const int w_begin = g0 + w * slice_len;
+                if (w_begin >= n2)
+                    break;
+                const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
+                const int count = s_count[w][lane];
+                if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
+                    sweep(w_begin, w_end, 0, false);
+                    continue;
+                }
+                const LogIdx *__restrict__ wl = log_of(w);
+                int r = 0;
+                bool has = r < count;
+                int j = w_begin + (has ? (int)wl[0] : 0);
+                float ex = K[(int64_t)j * 3 + 0], ey = K[(int64_t)j * 3 + 1],
+                      ez = K[(int64_t)j * 3 + 2];
+                while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+                    const bool has_next = r + 1 < count;
+                    const int j_next = w_begin + (has_next ? (int)wl[(r + 1) * NT] : 0);
+                    const float nx = K[(int64_t)j_next * 3 + 0], ny = K[(int64_t)j_next * 3 + 1],
+                                nz = K[(int64_t)j_next * 3 + 2];
+                    const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
+                    if (has && d < max_key)
+                        insert(d, j);
+                    ++r;
+                    has = has_next;
+                    j = j_next;
+                    ex = nx;
+                    ey = ny;
+                    ez = nz;
+                }
+            }
+        }
+        if (g0 + S * slice_len < n2)  // uniform
+            __syncthreads();  // the logs are free for the next group
+    }
     if (wave != 0)
         return;
-
-    // ---- wave 0 replays the other slices in key order ----
-    for (int w = 1; w < S; ++w) {
-        const int w_begin = w * slice_len;
-        if (w_begin >= n2)
-            break;
-        const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
-        const int count = s_count[w][lane];
-        if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
-            sweep(w_begin, w_end, 0, false);
-            continue;
-        }
-        const LogIdx *__restrict__ wl = log_of(w);
-        int r = 0;
-        bool has = r < count;
-        int j = w_begin + (has ? (int)wl[0] : 0);
-        float ex = K[(int64_t)j * 3 + 0], ey = K[(int64_t)j * 3 + 1], ez = K[(int64_t)j * 3 + 2];
-        while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-            const bool has_next = r + 1 < count;
-            const int j_next = w_begin + (has_next ? (int)wl[(r + 1) * NT] : 0);
-            const float nx = K[(int64_t)j_next * 3 + 0], ny = K[(int64_t)j_next * 3 + 1],
-                        nz = K[(int64_t)j_next * 3 + 2];
-            const float d = tk_dist2<float>(ex, ey, ez, qx, qy, qz);
-            if (has && d < max_key)
-                insert(d, j);
-            ++r;
-            has = has_next;
-            j = j_next;
-            ex = nx;
-            ey = ny;
-            ez = nz;
-        }
-    }
 
     if (active) {
         float *od = distance + ((int64_t)b * n1 + qi) * k;
@@ -1851,15 +1872,17 @@ template <int KMAX, int S, int CAP>
 int knn_tree_split_launch(const float *query, const float *key, float *distance,
                           int64_t *index, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    int slice_len = (n2 + S - 1) / S;
+    // a log holds 16-bit positions within its slice: slices of at most 65536 keys, in as
+    // many groups of S slices as that takes
+    const int groups = (int)(((int64_t)n2 + (int64_t)S * 65536 - 1) / ((int64_t)S * 65536));
+    int slice_len = (int)(((int64_t)n2 + (int64_t)S * groups - 1) / ((int64_t)S * groups));
     slice_len = (slice_len + 31) / 32 * 32;
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     // Worth it when sweeping dominates the insertions (timed on an MI355X): from 2048 keys
     // for k <= 8, 4096 for k <= 16, 8192 for k <= 32, and only while every workgroup has a
     // CU to itself.
     constexpr int MIN_KEYS = KMAX <= 8 ? 2048 : KMAX <= 16 ? 4096 : 8192;
-    // (a log holds 16-bit positions within its slice)
-    if (n2 < MIN_KEYS || slice_len < k || slice_len > 65536 || B * bpb > 256)
+    if (n2 < MIN_KEYS || slice_len < k || B * bpb > 256)
         return TK3D_ERR_UNSUPPORTED;
     auto launch = [&](auto wide) {
         // key indices of the slots in LDS: 16 bits up to 65536 keys, else 32 bits and
@@ -2046,20 +2069,23 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
     int ki[KMAX];
     float max_key = 0.0f;
     int max_idx = 0;
+    auto start_slots = [&]() {
 #pragma unroll
-    for (int s = 0; s < KMAX; ++s) {
-        kd[s] = -__builtin_huge_valf();
-        ki[s] = 0;
-        if (s < k) {  // uniform
-            const float d = wave == 0 ? dist_to(s) : __builtin_huge_valf();
-            kd[s] = d;
-            ki[s] = s;
-            if (s == 0 || d > max_key) {
-                max_key = d;
-                max_idx = s;
+        for (int s = 0; s < KMAX; ++s) {
+            kd[s] = -__builtin_huge_valf();
+            ki[s] = 0;
+            if (s < k) {  // uniform
+                const float d = wave == 0 ? dist_to(s) : __builtin_huge_valf();
+                kd[s] = d;
+                ki[s] = s;
+                if (s == 0 || d > max_key) {
+                    max_key = d;
+                    max_idx = s;
+                }
             }
         }
-    }
+    };
+    start_slots();
     int logged = 0;
     // MinK's insertion (mink.cuh:74-87): overwrite the maximum's slot, then rescan from the
     // inserted key over ascending slots with strict '>'.
@@ -2078,6 +2104,7 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
             max_idx = up ? s : max_idx;
         }
     };
+    int log_base = 0;  // first key of the slice this wave is sweeping
     auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
         for (int first = k_begin; first < k_end; first += CHUNK) {
             const int maxbits = __builtin_bit_cast(int, max_key);
@@ -2119,7 +2146,7 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
                     if (write_log) {
                         if (logged < CAP)
                             s_log[wave - 1][logged][lane] =
-                                (unsigned short)(first + i - wave * slice_len);  // within the slice
+                                (unsigned short)(first + i - log_base);  // within the slice
                         ++logged;
                     }
                 }
@@ -2130,44 +2157,58 @@ __global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
         }
     };
 
-    const int k_begin = wave * slice_len;
-    const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
-    if (wave == 0)
-        sweep(0, k_end, k, false);
-    else if (k_begin < n2)
-        sweep(k_begin, k_end, 0, true);
-    s_count[wave][lane] = logged;
-    __syncthreads();
+    // The keys are taken in groups of S slices (one group unless the cloud is longer than
+    // S slices of 65536 keys): wave 0 carries its slots from group to group, the others
+    // start every group from empty slots.
+    for (int g0 = 0; g0 < n2; g0 += S * slice_len) {  // uniform over the workgroup
+        const int k_begin = g0 + wave * slice_len;
+        const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
+        log_base = k_begin;
+        if (wave == 0) {
+            sweep(k_begin, k_end, g0 == 0 ? k : 0, false);
+        } else {
+            if (g0 > 0)
+                start_slots();
+            logged = 0;
+            if (k_begin < n2)
+                sweep(k_begin, k_end, 0, true);
+        }
+        s_count[wave][lane] = logged;
+        __syncthreads();
+        if (wave == 0) {
+            for (int w = 1; w < S; ++w) {
+                const int w_begin = g0 + w * slice_len;
+                if (w_begin >= n2)
+                    break;
+                const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
+                const int count = s_count[w][lane];
+                if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
+                    sweep(w_begin, w_end, 0, false);
+                    continue;
+                }
+                int r = 0;
+                bool has = r < count;
+                int j = w_begin + (has ? (int)s_log[w - 1][0][lane] : 0);
+                float d = dist_to(j);
+                while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
+                    const bool has_next = r + 1 < count;
+                    const int j_next =
+                        w_begin + (has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : 0);
+                    const float d_next = dist_to(j_next);
+                    if (has && d < max_key)
+                        insert(d, j);
+                    ++r;
+                    has = has_next;
+                    j = j_next;
+                    d = d_next;
+                }
+            }
+        }
+        if (g0 + S * slice_len < n2)  // uniform
+            __syncthreads();  // the logs are free for the next group
+    }
     if (wave != 0)
         return;
-
-    for (int w = 1; w < S; ++w) {
-        const int w_begin = w * slice_len;
-        if (w_begin >= n2)
-            break;
-        const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
-        const int count = s_count[w][lane];
-        if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
-            sweep(w_begin, w_end, 0, false);
-            continue;
-        }
-        int r = 0;
-        bool has = r < count;
-        int j = w_begin + (has ? (int)s_log[w - 1][0][lane] : 0);
-        float d = dist_to(j);
-        while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-            const bool has_next = r + 1 < count;
-            const int j_next =
-                w_begin + (has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : 0);
-            const float d_next = dist_to(j_next);
-            if (has && d < max_key)
-                insert(d, j);
-            ++r;
-            has = has_next;
-            j = j_next;
-            d = d_next;
-        }
-    }
 
     if (active) {
         float *od = distance + ((int64_t)b * n1 + qi) * k;
@@ -2194,16 +2235,18 @@ int knn_small_split_launch(const float *query, const float *key, float *distance
                            int k, hipStream_t s)
 {
     constexpr int S = 4, CAP = 96;
-    int slice_len = (n2 + S - 1) / S;
+    // a log holds 16-bit positions within its slice: slices of at most 65536 keys, in as
+    // many groups of S slices as that takes
+    const int key_groups = (int)(((int64_t)n2 + (int64_t)S * 65536 - 1) / ((int64_t)S * 65536));
+    int slice_len =
+        (int)(((int64_t)n2 + (int64_t)S * key_groups - 1) / ((int64_t)S * key_groups));
     slice_len = (slice_len + 31) / 32 * 32;
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     // 1.2-2.8 times faster than one wave per 64 queries up to 32768 queries in the launch
     // (timed on an MI355X, 1024 to 65536 keys); with 65536 queries only from 16384 keys on
     // (1.2-1.3 times), slower otherwise.
     const int64_t groups = B * bpb;
-    // (a log holds 16-bit positions within its slice)
-    if (slice_len > 65536 || n2 < 1024 || slice_len < k || groups > 1024 ||
-        (groups > 512 && n2 < 16384))
+    if (n2 < 1024 || slice_len < k || groups > 1024 || (groups > 512 && n2 < 16384))
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((knn_small_split_kernel_f32<SOA, WEIGHTS, CAP>), dim3((unsigned)(B * bpb)),
                        dim3(64 * S), 0, s, query, key, distance, index, weight, eps, (int)bpb, n1,
