@@ -1738,15 +1738,42 @@ __global__ __launch_bounds__(64 * S) void knn_tree_split_kernel_f32(
     // other than 0, logging) as the tree kernel does. `skip_below`: keys the fill took.
     int log_base = 0;  // first key of the slice this wave is sweeping
     auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
+        // With one wave per SIMD nothing hides the latency of the key loads, so they run
+        // ahead: lane l holds key `held + l` (two chunks per load, the next 64 keys
+        // requested before the current ones are used) and a chunk takes its keys out of
+        // those registers lane by lane.
+        float hx = 0, hy = 0, hz = 0, nx2 = 0, ny2 = 0, nz2 = 0;
+        auto request = [&](int base) {
+            int j = base + lane;
+            j = j < k_end ? j : k_end - 1;
+            j = j < 0 ? 0 : j;
+            nx2 = K[(int64_t)j * 3 + 0];
+            ny2 = K[(int64_t)j * 3 + 1];
+            nz2 = K[(int64_t)j * 3 + 2];
+        };
+        if (k_begin < k_end)
+            request(k_begin);
         for (int first = k_begin; first < k_end; first += CHUNK) {
+            const int within = (first - k_begin) & 63;  // 0 or 32: uniform
+            if (within == 0) {
+                hx = nx2;
+                hy = ny2;
+                hz = nz2;
+                if (first + 64 < k_end)
+                    request(first + 64);
+            }
             const int maxbits = __builtin_bit_cast(int, max_key);
             unsigned mask = 0u;
             if (first + CHUNK <= k_end) {
-                const float *__restrict__ g = K + (int64_t)first * 3;
 #pragma unroll
                 for (int i = 0; i < CHUNK; ++i) {
-                    const float d = tk_dist2<float>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
-                                                    qy, qz);
+                    const float kx = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, hx), within + i));
+                    const float ky = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, hy), within + i));
+                    const float kz = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, hz), within + i));
+                    const float d = tk_dist2<float>(kx, ky, kz, qx, qy, qz);
                     const unsigned diff = (unsigned)(__builtin_bit_cast(int, d) - maxbits);
                     mask = __builtin_amdgcn_alignbit(mask, diff, 31);
                 }
