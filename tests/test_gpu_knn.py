@@ -412,8 +412,8 @@ def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("b,n1,n2,k", [(2, 700, 900, 3), (8, 8192 + 1, 2048 + 3, 4),   # pre-filtered
                                         (2, 300, 1000, 7), (16, 8192, 2048, 16),        # pre-filtered
-                                        (2, 300, 1000, 16), (1, 100, 500, 33), (1, 64, 300, 64),
-                                        (1, 40, 200, 65)])                               # copies
+                                        (2, 300, 1000, 16), (1, 100, 9000, 6),           # copies
+                                        (1, 100, 500, 33), (1, 64, 300, 64), (1, 40, 200, 65)])
 def test_channels_first_clouds_are_read_in_place_or_copied(cuda, b, n1, n2, k, dtype):
     # knn_points(transpose=True) on [B,3,N] clouds: same rows as on the [B,N,3] clouds
     from torkit3d_amd import _fused
@@ -429,11 +429,14 @@ def test_channels_first_clouds_are_read_in_place_or_copied(cuda, b, n1, n2, k, d
     np.testing.assert_array_equal(i.cpu().numpy(), oi)
     raw = _fused.knn_distance_bcn(qt, kt, k, 1)
     # fp32: the library declines where its faster kernels only read [B,N,3] (k > 16, and
-    # k = 5..16 on launches too small for the pre-filtered sweep); fp64: k > 64 only
+    # k = 5..16 where the pre-filtered sweep does not pay: short key clouds, or few queries
+    # against a very long one); fp64: k > 64 only
     if dtype == torch.float64:
         declined = k > 64
     else:
-        declined = k > 16 or (k > 4 and not (b * n1 >= 131072 and n2 >= 2048))
+        few_long = b * n1 < 32768 and n2 > (8192 if k <= 8 else 32768)
+        long_enough = n2 >= (512 if k <= 8 else 1024) or (n2 >= 512 and b * n1 >= 131072)
+        declined = k > 16 or (k > 4 and (few_long or not long_enough))
     assert (raw is None) == declined
     if raw is not None:
         assert torch.equal(raw[0], d) and torch.equal(raw[1], i)

@@ -423,11 +423,13 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 //     query : Xh Xl Xh  Yh Yl Yh  T0 T1 | Zh Zl Zh  1  1  0  T0 T1        (X = -2 q'x)
 // In the 32 x 32 result lane l holds rows (keys) 16 h .. 16 h + 15, h = l / 32, of column
 // (query) l % 32; the keys of a tile are stored in that row order, so the sign bits of a
-// lane are 16 consecutive bits of the chunk mask. The wave's 128 queries are four blocks
-// of 32; lane l owns the queries of column l % 32 in blocks h and 2 + h, computes their
-// thr and writes -thr into the T terms of its own half only (the other half holds zeros
-// there), so no thr crosses lanes; the two halves of a mask meet through one exchange
-// between lanes l and l ^ 32 per chunk. Error budget in the rescaled units, on top of the
+// lane are 16 consecutive bits of the chunk mask. The wave's 64 QPL queries are 2 QPL
+// blocks of 32; lane l owns the queries of column l % 32 in blocks h, 2 + h, ..., computes
+// their thr and writes -thr into the T terms of its own half only (the other half holds
+// zeros there), so no thr crosses lanes; the two halves of a mask meet through one exchange
+// between lanes l and l ^ 32 per chunk. The library runs it with one query per lane in
+// workgroups of 512 lanes (LANES): 120 registers, four waves per SIMD, where two queries
+// per lane need 238 and leave two. Error budget in the rescaled units, on top of the
 // one above (products of the second pieces are left out, thr is rounded to two pieces):
 //     pieces dropped from 2 q'.k', subnormal pieces                       5 u R
 //     |k'|^2 and thr in two pieces                           4 u R + 4 u (M + R)
@@ -437,13 +439,13 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 //     canonical d2, |k'|^2 as staged, thr itself             10 u R + 3 u (M + R)
 // below 58 u R + 39 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
 // from the centre (rescaled; thr would leave fp16's range) take every key as a candidate.
-template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX>
-__global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
+template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK>
+__global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
     float eps, int blocks_per_batch, int n1, int n2, int k)
 {
-    constexpr int BLOCK = KNN_BLOCK;
+    constexpr int BLOCK = LANES;
     constexpr int NW = BLOCK / TK_WAVE;
     constexpr int STAGE = 512;
     constexpr int CHUNK = 32;
@@ -456,10 +458,11 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
     // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
     // the sweep runs into), then two of raw keys (x, y, z, 0) for the service steps.
     // (MATRIX: two stage buffers of key terms, [tile][half][row] x 16 bytes, instead.)
-    static_assert(!MATRIX || QPL == 2, "four blocks of 32 queries per wave");
+    static_assert(!MATRIX || QPL == 1 || QPL == 2, "two or four blocks of 32 queries per wave");
     constexpr int SCORE_FLOATS = MATRIX ? 2 * STAGE * 8 : 2 * STAGE * 4 + 32;
     constexpr int STAGING_FLOATS = SCORE_FLOATS + 2 * STAGE * 4;
-    constexpr int TRANSPOSE_FLOATS = NW * 2 * TK_WAVE * (KMAX + 1);  // see the end of the kernel
+    constexpr int TWAVES = NW < 4 ? NW : 4;  // waves that transpose their results together
+    constexpr int TRANSPOSE_FLOATS = TWAVES * 2 * TK_WAVE * (KMAX + 1);  // see the end of the kernel
     __shared__ __align__(16) float
         skey[STAGING_FLOATS > TRANSPOSE_FLOATS ? STAGING_FLOATS : TRANSPOSE_FLOATS];
     float4 *const sraw = reinterpret_cast<float4 *>(skey + SCORE_FLOATS);
@@ -628,7 +631,7 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
         pending[i] = 0;
     }
 
-    // MATRIX: the query side of the 16 terms for the wave's four blocks of 32 queries.
+    // MATRIX: the query side of the 16 terms for the wave's 2 QPL blocks of 32 queries.
     // Block 2 i + h' holds query i of the lanes of half h'; this lane supplies terms
     // 8 h .. 8 h + 7 of column lane % 32 in every block, from its own coordinates or, for
     // the other half's blocks, its partner's. The T terms (.w) are written per chunk.
@@ -847,12 +850,20 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
                 }
                 // rows of this half: keys 16 h .. 16 h + 15 of the chunk, first key in the
                 // highest bit; the other half's rows of this lane's blocks come from lane ^ 32
-                const unsigned send = half == 0 ? (m16[1] | (m16[3] << 16)) : (m16[0] | (m16[2] << 16));
-                const unsigned recv = __shfl_xor(send, 32);
-                const unsigned own0 = half == 0 ? m16[0] : m16[1], own1 = half == 0 ? m16[2] : m16[3];
-                const unsigned oth0 = recv & 0xffffu, oth1 = recv >> 16;
-                mask[0] = half == 0 ? ((own0 << 16) | oth0) : ((oth0 << 16) | own0);
-                mask[1] = half == 0 ? ((own1 << 16) | oth1) : ((oth1 << 16) | own1);
+                if constexpr (QPL == 2) {
+                    const unsigned send =
+                        half == 0 ? (m16[1] | (m16[3] << 16)) : (m16[0] | (m16[2] << 16));
+                    const unsigned recv = __shfl_xor(send, 32);
+                    const unsigned own0 = half == 0 ? m16[0] : m16[1],
+                                   own1 = half == 0 ? m16[2] : m16[3];
+                    const unsigned oth0 = recv & 0xffffu, oth1 = recv >> 16;
+                    mask[0] = half == 0 ? ((own0 << 16) | oth0) : ((oth0 << 16) | own0);
+                    mask[1] = half == 0 ? ((own1 << 16) | oth1) : ((oth1 << 16) | own1);
+                } else {
+                    const unsigned recv = __shfl_xor(half == 0 ? m16[1] : m16[0], 32);
+                    const unsigned own = half == 0 ? m16[0] : m16[1];
+                    mask[0] = half == 0 ? ((own << 16) | recv) : ((recv << 16) | own);
+                }
             } else {
             const float4 *ck = sbuf + c0k;
             // Groups of G keys: the next group is read from LDS before the current one is
@@ -959,9 +970,10 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
     // stores are runs of consecutive elements instead of one element per k ----
     __syncthreads();
     constexpr int ROW = KMAX + 1;
-    float *const tbuf = skey + wave * (2 * TK_WAVE * ROW);  // values, then indices
+    float *const tbuf = skey + (wave % TWAVES) * (2 * TK_WAVE * ROW);  // values, then indices
     int *const ibuf = reinterpret_cast<int *>(tbuf + TK_WAVE * ROW);
-    static_assert(NW * 2 * TK_WAVE * ROW == TRANSPOSE_FLOATS, "LDS for the transpose");
+    static_assert(TWAVES * 2 * TK_WAVE * ROW == TRANSPOSE_FLOATS, "LDS for the transpose");
+    auto emit = [&]() {
 #pragma unroll
     for (int i = 0; i < QPL; ++i) {
         const int q0 = (qblock * QPL + i) * BLOCK + wave * TK_WAVE;  // first query of the wave
@@ -996,6 +1008,18 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_filter_kernel_f32(
                                      __builtin_bit_cast(float, kd[i][2])};
                 knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + q0 + lane) * 3);
             }
+        }
+    }
+    };
+    if constexpr (NW == TWAVES) {
+        emit();
+    } else {
+#pragma unroll 1
+        for (int pass = 0; pass < NW / TWAVES; ++pass) {
+            if (pass > 0)
+                __syncthreads();  // the waves of the previous pass are done with the buffers
+            if (wave / TWAVES == pass)
+                emit();
         }
     }
 }
@@ -2058,229 +2082,6 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_global_kernel(
     }
 }
 
-// k <= 4 with few queries: the shared-key sweep of knn_tree_split_kernel_f32 with the
-// slots in registers. Four waves serve the same 64 queries; wave 0 runs MinK on the first
-// slice of the keys, the others run a MinK of their own on their slices from k empty
-// slots and log the keys they insert; wave 0 then replays the logs in key order (an
-// overflowing log makes it sweep that slice in full).
-template <bool SOA, bool WEIGHTS, int CAP>
-__global__ __launch_bounds__(256) void knn_small_split_kernel_f32(
-    const float *__restrict__ query, const float *__restrict__ key,
-    float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
-    float eps, int blocks_per_batch, int n1, int n2, int k, int slice_len)
-{
-    constexpr int KMAX = 4, CHUNK = 32, NT = 64, S = 4;
-    __shared__ unsigned short s_log[S - 1][CAP][NT];  // wave 0 keeps none
-    __shared__ int s_count[S][NT];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.x / blocks_per_batch;
-    const int qi = (blockIdx.x - b * blocks_per_batch) * NT + lane;
-    const bool active = qi < n1;
-    const float *__restrict__ K = key + (int64_t)b * n2 * 3;
-    float qx = 0, qy = 0, qz = 0;
-    if (active) {
-        const float *__restrict__ Q = query + (int64_t)b * n1 * 3;
-        qx = knn_coord<SOA>(Q, n1, qi, 0);
-        qy = knn_coord<SOA>(Q, n1, qi, 1);
-        qz = knn_coord<SOA>(Q, n1, qi, 2);
-    }
-    auto dist_to = [&](int j) {
-        return tk_dist2<float>(knn_coord<SOA>(K, n2, j, 0), knn_coord<SOA>(K, n2, j, 1),
-                               knn_coord<SOA>(K, n2, j, 2), qx, qy, qz);
-    };
-
-    // Slots: wave 0 fills them with keys 0..k-1 (mink.cuh:63-72); the other waves start
-    // from k empty slots (+inf). Unused slots stay at -inf and are never the maximum.
-    float kd[KMAX];
-    int ki[KMAX];
-    float max_key = 0.0f;
-    int max_idx = 0;
-    auto start_slots = [&]() {
-#pragma unroll
-        for (int s = 0; s < KMAX; ++s) {
-            kd[s] = -__builtin_huge_valf();
-            ki[s] = 0;
-            if (s < k) {  // uniform
-                const float d = wave == 0 ? dist_to(s) : __builtin_huge_valf();
-                kd[s] = d;
-                ki[s] = s;
-                if (s == 0 || d > max_key) {
-                    max_key = d;
-                    max_idx = s;
-                }
-            }
-        }
-    };
-    start_slots();
-    int logged = 0;
-    // MinK's insertion (mink.cuh:74-87): overwrite the maximum's slot, then rescan from the
-    // inserted key over ascending slots with strict '>'.
-    auto insert = [&](float d, int j) {
-#pragma unroll
-        for (int s = 0; s < KMAX; ++s) {
-            const bool here = (s == max_idx);
-            kd[s] = here ? d : kd[s];
-            ki[s] = here ? j : ki[s];
-        }
-        max_key = d;
-#pragma unroll
-        for (int s = 0; s < KMAX; ++s) {
-            const bool up = kd[s] > max_key;
-            max_key = up ? kd[s] : max_key;
-            max_idx = up ? s : max_idx;
-        }
-    };
-    int log_base = 0;  // first key of the slice this wave is sweeping
-    auto sweep = [&](int k_begin, int k_end, int skip_below, bool write_log) {
-        for (int first = k_begin; first < k_end; first += CHUNK) {
-            const int maxbits = __builtin_bit_cast(int, max_key);
-            unsigned mask = 0u;
-            if (first + CHUNK <= k_end) {
-#pragma unroll
-                for (int i = 0; i < CHUNK; ++i) {  // uniform addresses: scalar loads
-                    const unsigned diff =
-                        (unsigned)(__builtin_bit_cast(int, dist_to(first + i)) - maxbits);
-                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);  // (mask << 1) | sign
-                }
-            } else {
-                for (int i = 0; i < CHUNK; ++i) {
-                    const int j = first + i < k_end ? first + i : k_end - 1;  // masked below
-                    const unsigned diff = (unsigned)(__builtin_bit_cast(int, dist_to(j)) - maxbits);
-                    mask = __builtin_amdgcn_alignbit(mask, diff, 31);
-                }
-            }
-            // The sign trick orders bit patterns; a NaN maximum (a NaN in slot 0 of the
-            // fill, which MinK never replaces) admits nothing, as the strict test below
-            // confirms for every candidate anyway.
-            int lo = skip_below - first;
-            lo = lo < 0 ? 0 : (lo > CHUNK ? CHUNK : lo);
-            int hi = k_end - first;
-            hi = hi > CHUNK ? CHUNK : hi;
-            unsigned valid = (lo >= CHUNK) ? 0u : (0xffffffffu >> lo);
-            valid &= (hi >= CHUNK) ? 0xffffffffu : ~(0xffffffffu >> hi);
-            mask &= valid;
-            bool has = mask != 0u;
-            int i = has ? __builtin_clz(mask) : 0;
-            float d = dist_to(first + i < k_end ? first + i : k_end - 1);
-            while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-                mask &= ~(0x80000000u >> i);
-                const bool has_next = mask != 0u;
-                const int i_next = has_next ? __builtin_clz(mask) : 0;
-                const float d_next = dist_to(first + i_next < k_end ? first + i_next : k_end - 1);
-                if (has && d < max_key) {
-                    insert(d, first + i);
-                    if (write_log) {
-                        if (logged < CAP)
-                            s_log[wave - 1][logged][lane] =
-                                (unsigned short)(first + i - log_base);  // within the slice
-                        ++logged;
-                    }
-                }
-                has = has_next;
-                i = i_next;
-                d = d_next;
-            }
-        }
-    };
-
-    // The keys are taken in groups of S slices (one group unless the cloud is longer than
-    // S slices of 65536 keys): wave 0 carries its slots from group to group, the others
-    // start every group from empty slots.
-    for (int g0 = 0; g0 < n2; g0 += S * slice_len) {  // uniform over the workgroup
-        const int k_begin = g0 + wave * slice_len;
-        const int k_end = (k_begin + slice_len < n2) ? k_begin + slice_len : n2;
-        log_base = k_begin;
-        if (wave == 0) {
-            sweep(k_begin, k_end, g0 == 0 ? k : 0, false);
-        } else {
-            if (g0 > 0)
-                start_slots();
-            logged = 0;
-            if (k_begin < n2)
-                sweep(k_begin, k_end, 0, true);
-        }
-        s_count[wave][lane] = logged;
-        __syncthreads();
-        if (wave == 0) {
-            for (int w = 1; w < S; ++w) {
-                const int w_begin = g0 + w * slice_len;
-                if (w_begin >= n2)
-                    break;
-                const int w_end = (w_begin + slice_len < n2) ? w_begin + slice_len : n2;
-                const int count = s_count[w][lane];
-                if (__builtin_amdgcn_ballot_w64(count > CAP)) {  // uniform: a log overflowed
-                    sweep(w_begin, w_end, 0, false);
-                    continue;
-                }
-                int r = 0;
-                bool has = r < count;
-                int j = w_begin + (has ? (int)s_log[w - 1][0][lane] : 0);
-                float d = dist_to(j);
-                while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
-                    const bool has_next = r + 1 < count;
-                    const int j_next =
-                        w_begin + (has_next ? (int)s_log[w - 1][r + 1 < CAP ? r + 1 : 0][lane] : 0);
-                    const float d_next = dist_to(j_next);
-                    if (has && d < max_key)
-                        insert(d, j);
-                    ++r;
-                    has = has_next;
-                    j = j_next;
-                    d = d_next;
-                }
-            }
-        }
-        if (g0 + S * slice_len < n2)  // uniform
-            __syncthreads();  // the logs are free for the next group
-    }
-    if (wave != 0)
-        return;
-
-    if (active) {
-        float *od = distance + ((int64_t)b * n1 + qi) * k;
-        int64_t *oi = index + ((int64_t)b * n1 + qi) * k;
-#pragma unroll
-        for (int s = 0; s < KMAX; ++s) {
-            if (s < k) {
-                od[s] = kd[s];
-                oi[s] = (int64_t)ki[s];
-            }
-        }
-        if constexpr (WEIGHTS) {  // k == 3
-            const float d3[3] = {kd[0], kd[1], kd[2]};
-            knn_three_weights<float>(d3, eps, weight + ((int64_t)b * n1 + qi) * 3);
-        }
-    }
-}
-
-// Applies when the plain launch (one wave per 64 queries) would leave SIMDs idle and the
-// key cloud is long enough; TK3D_ERR_UNSUPPORTED otherwise.
-template <bool SOA, bool WEIGHTS>
-int knn_small_split_launch(const float *query, const float *key, float *distance,
-                           int64_t *index, float *weight, float eps, int64_t B, int n1, int n2,
-                           int k, hipStream_t s)
-{
-    constexpr int S = 4, CAP = 96;
-    // a log holds 16-bit positions within its slice: slices of at most 65536 keys, in as
-    // many groups of S slices as that takes
-    const int key_groups = (int)(((int64_t)n2 + (int64_t)S * 65536 - 1) / ((int64_t)S * 65536));
-    int slice_len =
-        (int)(((int64_t)n2 + (int64_t)S * key_groups - 1) / ((int64_t)S * key_groups));
-    slice_len = (slice_len + 31) / 32 * 32;
-    const int64_t bpb = ((int64_t)n1 + 63) / 64;
-    // 1.2-2.8 times faster than one wave per 64 queries up to 32768 queries in the launch
-    // (timed on an MI355X, 1024 to 65536 keys); with 65536 queries only from 16384 keys on
-    // (1.2-1.3 times), slower otherwise.
-    const int64_t groups = B * bpb;
-    if (n2 < 1024 || slice_len < k || groups > 1024 || (groups > 512 && n2 < 16384))
-        return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_small_split_kernel_f32<SOA, WEIGHTS, CAP>), dim3((unsigned)(B * bpb)),
-                       dim3(64 * S), 0, s, query, key, distance, index, weight, eps, (int)bpb, n1,
-                       n2, k, slice_len);
-    return tk_launch_status();
-}
-
 template <typename T, int KMAX, bool SOA = false, bool WEIGHTS = false>
 void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64_t B,
                 int bpb, int n1, int n2, int k, hipStream_t s, T *weight = nullptr,
@@ -2296,31 +2097,34 @@ void knn_launch(const T *query, const T *key, T *distance, int64_t *index, int64
                            index, weight, eps, bpb, n1, n2, k);
 }
 
-// The pre-filtered kernel pays when the launch fills the chip with two queries per lane
-// and the key cloud is long enough to amortise its prologue (two passes over the keys per
-// workgroup); TK3D_ERR_UNSUPPORTED otherwise. Thresholds from timing it against the
-// kernels above on an MI355X for k = 1..16, 16384 to 524288 queries, 256 to 8192 keys:
-// 1.05-1.5 times faster inside them, 0.6-1.0 outside.
+// Where the pre-filtered kernel is the fastest route for k <= 16, from timing it against
+// every other kernel here on an MI355X (k = 1..16, 128 to 524288 queries, 128 to 65536
+// keys, 1100 shapes): 1.1-2.0 times faster inside these bounds, 0.7-1.0 outside. Short key
+// clouds do not amortise its prologue (two passes over the keys per workgroup); with few
+// queries and very long clouds the kernels that share the keys of 64 queries among several
+// waves win, from k = 5 on.
 inline bool knn_filter_pays(int64_t queries, int n2, int k)
 {
-    if (n2 >= 2048)
-        return queries >= 32768;
-    if (n2 >= 1024)
-        return queries >= 262144;
-    return n2 >= 512 && queries >= (k <= 4 ? 131072 : k <= 8 ? 262144 : 524288);
+    if (k <= 4)
+        return n2 >= 512 || (n2 >= 256 && queries >= 4096);
+    if (queries < 32768 && n2 > (k <= 8 ? 8192 : 32768))
+        return false;
+    return n2 >= (k <= 8 ? 512 : 1024) || (n2 >= 512 && queries >= 131072);
 }
 
-template <int KMAX, bool SOA, bool WEIGHTS, bool MATRIX = true>
+template <int KMAX, bool SOA, bool WEIGHTS>
 int knn_filter_launch(const float *query, const float *key, float *distance, int64_t *index,
                       float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
-    constexpr int QPL = 2;
-    const int64_t bpb = ((int64_t)n1 + QPL * KNN_BLOCK - 1) / (QPL * KNN_BLOCK);
+    // One query per lane, 512 lanes: two workgroups (16 waves) per CU. Two queries per lane
+    // in 256 lanes need twice the registers, which leaves two waves per SIMD, and were 1.1
+    // to 1.4 times slower on every shape (k = 16 at B=32, 8192 x 2048: 222 -> 191 us).
+    const int64_t bpb = ((int64_t)n1 + 511) / 512;
     if (!knn_filter_pays(B * n1, n2, k) || B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, QPL, SOA, WEIGHTS, MATRIX>), dim3((unsigned)(B * bpb)),
-                       dim3(KNN_BLOCK), 0, s, query, key, distance, index, weight, eps, (int)bpb,
-                       n1, n2, k);
+    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512>),
+                       dim3((unsigned)(B * bpb)), dim3(512), 0, s, query, key, distance, index,
+                       weight, eps, (int)bpb, n1, n2, k);
     return tk_launch_status();
 }
 
@@ -2347,12 +2151,7 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
     hipStream_t s = (hipStream_t)stream;
     const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
     if (k <= 4) {
-        if constexpr (sizeof(T) == 4) {
-            const int rc = knn_small_split_launch<false, false>(query, key, distance, index,
-                                                                nullptr, 0.0f, B, n1, n2, kk, s);
-            if (rc != TK3D_ERR_UNSUPPORTED)
-                return rc;
-        }
+        // the pre-filtered kernel wherever it pays (512 keys or more), else the batched kernel
         if constexpr (sizeof(T) == 4) {
             const int rc = knn_filter_launch<4, false, false>(query, key, distance, index, nullptr,
                                                               0.0f, B, n1, n2, kk, s);
@@ -2364,6 +2163,16 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
         // 0.30 ms against 0.41 ms with the slots in registers). Small launches with k <= 8
         // are a little faster in registers.
+        if (k <= 16) {
+            // pre-filtered sweep on the matrix cores, slots in registers: wherever it pays
+            const int rc =
+                k <= 8 ? knn_filter_launch<8, false, false>(query, key, distance, index, nullptr,
+                                                            0.0f, B, n1, n2, kk, s)
+                       : knn_filter_launch<16, false, false>(query, key, distance, index, nullptr,
+                                                             0.0f, B, n1, n2, kk, s);
+            if (rc != TK3D_ERR_UNSUPPORTED)
+                return rc;
+        }
         if (k <= 16) {
             // few queries: four waves share the keys of every 64 queries (1.2-3.3 times
             // faster from 2048 / 4096 keys on)
@@ -2386,16 +2195,6 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
             // a chip's worth of queries on long key clouds: matrix-core sweep into the tree
             const int rc = knn_tree_matrix_launch<32, 2>(query, key, distance, index, B, n1, n2,
                                                          kk, s);
-            if (rc != TK3D_ERR_UNSUPPORTED)
-                return rc;
-        }
-        if (k <= 16) {
-            // many queries: pre-filtered sweep, slots in registers
-            const int rc =
-                k <= 8 ? knn_filter_launch<8, false, false>(query, key, distance, index, nullptr,
-                                                            0.0f, B, n1, n2, kk, s)
-                       : knn_filter_launch<16, false, false>(query, key, distance, index, nullptr,
-                                                             0.0f, B, n1, n2, kk, s);
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
@@ -2473,11 +2272,8 @@ int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int
     if constexpr (sizeof(T) == 4) {
         int rc = TK3D_ERR_UNSUPPORTED;
         if (k <= 4) {
-            rc = knn_small_split_launch<true, false>(query, key, distance, index, nullptr, 0.0f, B,
-                                                     n1, n2, kk, s);
-            if (rc == TK3D_ERR_UNSUPPORTED)
-                rc = knn_filter_launch<4, true, false>(query, key, distance, index, nullptr, 0.0f,
-                                                       B, n1, n2, kk, s);
+            rc = knn_filter_launch<4, true, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                   n1, n2, kk, s);
             if (rc == TK3D_ERR_UNSUPPORTED) {
                 knn_launch<T, 4, true>(query, key, distance, index, B, (int)bpb, n1, n2, kk, s);
                 rc = tk_launch_status();
@@ -2526,15 +2322,6 @@ int three_nn(const T *query, const T *key, bool channels_first, int64_t B, int64
         return TK3D_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if constexpr (sizeof(T) == 4) {
-        const int rc = channels_first
-                           ? knn_small_split_launch<true, true>(query, key, distance, index, weight,
-                                                                (float)eps, B, (int)N1, (int)N2,
-                                                                3, s)
-                           : knn_small_split_launch<false, true>(query, key, distance, index,
-                                                                 weight, (float)eps, B, (int)N1,
-                                                                 (int)N2, 3, s);
-        if (rc != TK3D_ERR_UNSUPPORTED)
-            return rc;
         const int rf = channels_first
                            ? knn_filter_launch<4, true, true>(query, key, distance, index, weight,
                                                               (float)eps, B, (int)N1, (int)N2, 3, s)
