@@ -331,10 +331,12 @@ def test_matrix_prefilter_with_a_short_cloud_on_hard_inputs(cuda, kind):
     check_forward(a.contiguous(), c.contiguous(), cuda)
 
 
+@pytest.mark.parametrize("b", [48, 72])  # two and four query blocks per wave
 @pytest.mark.parametrize("kind", HARD_KINDS)
-def test_matrix_prefilter_is_exact_on_hard_inputs(cuda, kind):
-    b, n1, n2 = 48, 2500, 3001
+def test_matrix_prefilter_is_exact_on_hard_inputs(cuda, kind, b):
+    n1, n2 = 2500, 3001
     assert min(n1 - 400, n2) >= 2048 and b * ((n1 - 400 + 511) // 512 + (n2 + 511) // 512) >= 512
+    assert (b * ((n1 + 511) // 512 + (n2 + 511) // 512) <= 640) == (b == 48)
     a, c = _clouds(kind, gen(sum(map(ord, kind)) + 1), b, n1, n2)
     check_forward(a.contiguous(), c.contiguous(), cuda)
 

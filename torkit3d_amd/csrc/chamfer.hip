@@ -1679,6 +1679,17 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
                 int64_t slice_len;
                 blocks += qb[w] * chamfer_slices(nk[w], want[w], 128, slice_len);
             }
+            // Launches of up to one and a half workgroups per CU (two and a half on key
+            // clouds of up to 4096 points) run with two query blocks per wave instead of
+            // four: twice the workgroups of half the queries, so the chip holds them all at
+            // once with work for every SIMD (B=16, 4096 x 4096: 43 -> 37 us; B=24,
+            // 2048 x 2048: 42 -> 32 us; B=48, 2500 x 3001: 107 -> 84 us). Larger launches
+            // lose to the key terms every workgroup stages for itself (B=32, 16384 x 16384:
+            // 0.59 -> 0.64 ms).
+            const int64_t nkmax = N1 > N2 ? N1 : N2;
+            if (blocks >= 96 && (blocks <= 384 || (blocks <= 640 && nkmax <= 4096)))
+                return chamfer_forward_mfma_launch<2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+                                                      idx2, s, want[0], want[1]);
             if (blocks >= 96)
                 return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                                       idx2, s, want[0], want[1]);
