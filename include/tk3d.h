@@ -69,6 +69,22 @@ int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2,
                                       double *dist1, int64_t *idx1, double *dist2,
                                       int64_t *idx2, void *stream);
 
+/* The same operation (chamfer_distance_kernel.cu:91-151) for callers that can lend
+ * scratch memory: with `workspace` (256-byte aligned device memory of at least
+ * tk3d_chamfer_distance_forward_workspace_bytes(B, N1, N2) bytes, contents irrelevant
+ * before and after) both clouds are first sorted along a space-filling curve, and a wave
+ * then sweeps only the key tiles that can hold a nearest neighbour of its queries.
+ * Results are bit-identical to tk3d_chamfer_distance_forward_f32 for every input. The
+ * size function returns 0 for shapes this path does not serve (clouds under 2048 or over
+ * 65536 points); with a null or short workspace the call is
+ * tk3d_chamfer_distance_forward_f32. */
+size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2);
+int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2,
+                                         int64_t B, int64_t N1, int64_t N2,
+                                         float *dist1, int64_t *idx1, float *dist2,
+                                         int64_t *idx2, void *workspace,
+                                         size_t workspace_bytes, void *stream);
+
 /* Replaces chamfer_distance_backward_cuda
  * (chamfer_distance.h:10-16, chamfer_distance_kernel.cu:200-274).
  * grad_xyz1[b,i] = 2*gd1[b,i]*(x1[b,i]-x2[b,idx1[b,i]])

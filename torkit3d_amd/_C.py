@@ -235,8 +235,21 @@ def chamfer_distance_forward_cuda(xyz1, xyz2):
         idx1 = torch.empty((b, n1), dtype=torch.int64, device=dev)
         dist2 = torch.empty((b, n2), dtype=xyz1.dtype, device=dev)
         idx2 = torch.empty((b, n2), dtype=torch.int64, device=dev)
-        _lib.call("tk3d_chamfer_distance_forward", xyz1, ptr(xyz1), ptr(xyz2), i64(b), i64(n1),
-                  i64(n2), ptr(dist1), ptr(idx1), ptr(dist2), ptr(idx2), stream_of(xyz1))
+        ws_bytes = _lib.chamfer_workspace_bytes(b, n1, n2) if xyz1.dtype == torch.float32 else 0
+        if ws_bytes:
+            # clouds of a few thousand points and more: sorted along a space-filling curve
+            # in a scratch buffer, and only key tiles near a wave's queries are swept
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+            fn = _lib.lib().tk3d_chamfer_distance_forward_ws_f32
+            fn.restype = ctypes.c_int
+            _lib.check(fn(ptr(xyz1), ptr(xyz2), i64(b), i64(n1), i64(n2), ptr(dist1), ptr(idx1),
+                          ptr(dist2), ptr(idx2), ctypes.c_void_p(ws.data_ptr()),
+                          ctypes.c_size_t(ws_bytes), stream_of(xyz1)),
+                       "tk3d_chamfer_distance_forward_ws_f32")
+        else:
+            _lib.call("tk3d_chamfer_distance_forward", xyz1, ptr(xyz1), ptr(xyz2), i64(b),
+                      i64(n1), i64(n2), ptr(dist1), ptr(idx1), ptr(dist2), ptr(idx2),
+                      stream_of(xyz1))
     return [dist1, idx1, dist2, idx2]
 
 

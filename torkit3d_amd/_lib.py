@@ -75,6 +75,19 @@ def fps_workspace_bytes(b, n, element_size):
     return int(_fps_workspace_fn(i64(b), i64(n), ctypes.c_size_t(element_size)))
 
 
+_chamfer_workspace_fn = None
+
+
+def chamfer_workspace_bytes(b, n1, n2):
+    """Scratch bytes ``tk3d_chamfer_distance_forward_ws_f32`` wants for this shape (0: none)."""
+    global _chamfer_workspace_fn
+    if _chamfer_workspace_fn is None:
+        fn = lib().tk3d_chamfer_distance_forward_workspace_bytes
+        fn.restype = ctypes.c_size_t
+        _chamfer_workspace_fn = fn
+    return int(_chamfer_workspace_fn(i64(b), i64(n1), i64(n2)))
+
+
 ERR_UNSUPPORTED = -6  # TK3D_ERR_UNSUPPORTED
 
 

@@ -39,6 +39,10 @@ template <typename T> struct ChamferDir {
 template <typename T> struct ChamferFwdArgs {
     ChamferDir<T> dir[2];
     int nblocks0;  // workgroups of direction 0; the rest belong to direction 1
+    // When set: [2, nbatch] flags, and a workgroup of direction w and batch element b
+    // works only if only_if[w * nbatch + b] is non-zero (vector pre-filter kernel only).
+    const int *only_if;
+    int nbatch;
 };
 
 template <typename T> __device__ __forceinline__ T chamfer_init_min();
@@ -316,7 +320,7 @@ __device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict
     out_j = gj == 0x7fffffff ? -1 : gj;
 }
 
-template <int QPL, int BLOCK, int TILE, int STAGE>
+template <int QPL, int BLOCK, int TILE, int STAGE, bool GATED = false>
 __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFwdArgs<float> args)
 {
     static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
@@ -335,6 +339,10 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     const int wave = tid / TK_WAVE;
     int b, qblock, slice;
     const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
+    if constexpr (GATED) {
+        if (args.only_if[(int)(&d - args.dir) * args.nbatch + b] == 0)
+            return;  // uniform over the workgroup
+    }
     const int nq = d.nq;
     // This workgroup sweeps keys [k0, k0 + nk); to the filter that slice is the key cloud.
     const int k0 = slice * d.slice_len;
@@ -1515,6 +1523,8 @@ int chamfer_fill_args(ChamferFwdArgs<T> &a, const T *xyz1, const T *xyz2, int64_
     if (nblocks > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
     a.nblocks0 = (int)nb[0];
+    a.only_if = nullptr;
+    a.nbatch = (int)B;
     return TK3D_OK;
 }
 
@@ -1564,7 +1574,8 @@ int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
 template <int QPL, int BLOCK = 256, int TILE = 64, int STAGE = 1024>
 int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                                   int64_t N2, float *dist1, int64_t *idx1, float *dist2,
-                                  int64_t *idx2, hipStream_t stream, int slices = 1)
+                                  int64_t *idx2, hipStream_t stream, int slices = 1,
+                                  const int *only_if = nullptr)
 {
     ChamferFwdArgs<float> a;
     int64_t nblocks;
@@ -1572,6 +1583,11 @@ int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t 
         a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, slices, nblocks);
     if (rc != TK3D_OK)
         return rc;
+    a.only_if = only_if;
+    if (only_if != nullptr)
+        return chamfer_forward_run<float>(
+            chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE, true>, BLOCK, a, nblocks, B,
+            stream);
     return chamfer_forward_run<float>(chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE>,
                                       BLOCK, a, nblocks, B, stream);
 }
@@ -1721,6 +1737,823 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
                                                  idx2, s);
 }
 
+// ---- fp32 forward on clouds sorted along a space-filling curve ---------------------
+//
+// The sweeps above evaluate every (query, key) pair. Points that are far apart cannot be
+// nearest neighbours, and once both clouds are ordered along a space-filling curve that
+// can be decided for 32 keys and a wave's queries at a time:
+//
+//   chamfer_sort_kernel (one workgroup per cloud): bounding box, centre and scale as in
+//     the matrix pre-filter, a counting sort of the points by the 15-bit Morton code of
+//     their cell in a 32^3 grid over the box, then, per tile of 32 sorted points, the 16
+//     fp16 terms of every key (the layout the matrix kernel stages in LDS) and the tile's
+//     bounding box in centred, scaled coordinates. The sorted points carry their original
+//     index.
+//   chamfer_pruned_kernel (waves work alone, no LDS): a wave takes NQB x 32 consecutive
+//     sorted queries - a compact patch - and sweeps a key tile only if the squared gap
+//     between the patch's box and the tile's box does not exceed T, an upper bound of
+//     every query's distance to the nearest key met so far: first the tiles that overlap
+//     the patch, then in passes at T/16, T/4 and T with T taken anew each time. The
+//     sweep, the three smallest tile minima per lane and the exact re-evaluation of the
+//     candidate tiles are those of the matrix kernel; ties between equal distances go to
+//     the lower original index, compared explicitly because sorted order is not index
+//     order. Queries with three or more candidate tiles are scanned exactly over the
+//     swept tiles only.
+//
+// Why a skipped tile cannot matter. With the notation of the matrix kernel (k', q' the
+// centred, scaled points as rounded, u = 2^-24, R = (max|k'| + |q'|)^2): the score of a
+// swept key satisfies |s + |q'|^2 - d2| <= 45.3 u R for its canonical distance d2 (in
+// scaled units), so ub = min s + |q'|^2 + 128 u R (the sum in fp32: 4 u R more) is at
+// least the canonical distance of some swept key. For a key of a skipped tile,
+// d2 >= |q' - k'|^2 - 7.1 u R >= gap^2 - 7.1 u R, where gap^2, evaluated in fp32 from box
+// corners that are themselves coordinates of rounded points, is within a factor 1 - 8u of
+// the exact squared gap. A tile is skipped only if gap^2 > (T + 128 u R) * 1.001 with
+// T >= ub of every query of the wave, so each of its keys is strictly farther from every
+// query than a key already met: it can neither be the minimum nor tie with it. T only
+// shrinks as tiles are swept, so a tile skipped under an earlier T stays skipped rightly.
+//
+// Input the bound does not cover (non-finite coordinates, extents outside 2^+-40, queries
+// further than 8000 extents from the key cloud) and waves whose exact scans would take
+// long (heavy ties on many swept tiles) raise a flag for their cloud and direction; the
+// vector pre-filter kernel runs behind this one and serves exactly the flagged ones.
+struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
+    float c[3];            // centre of the bounding box
+    float scale;           // 2^-(exponent of the largest half extent)
+    int kmax2_bits;        // largest |k'|^2 (bit pattern of the float)
+    int unsafe;            // the bound does not cover this cloud
+    float lo[3], hi[3];    // bounding box, caller's units
+    int pad[4];
+};
+
+struct ChamferSortArgs {
+    const float *xyz[2];
+    float4 *sorted[2];  // [B, npad]: x, y, z, original index (bits); padding: NaN, -1
+    uint4 *terms[2];    // [B, npad / 32][2][32]
+    float4 *boxes[2];   // [B, npad / 32][2]: lo, hi in centred, scaled coordinates
+    ChamferSortedHdr *hdr;  // [2, B]
+    int *flags;             // [2, B]
+    int n[2], npad[2];
+    int B;
+};
+
+__device__ __forceinline__ int chamfer_morton5(int v)
+{
+    v &= 0x1f;
+    v = (v | (v << 8)) & 0x100f;
+    v = (v | (v << 4)) & 0x10c3;
+    v = (v | (v << 2)) & 0x1249;
+    return v;
+}
+
+// Position of cell (x, y, z), each below 32, along the 3-D Hilbert curve of order 5
+// (Skilling's transposed form, then the bits interleaved): consecutive positions are
+// neighbouring cells, so a run of consecutive sorted points is a compact patch, which a
+// run along the Morton curve, with its jumps, often is not.
+__device__ __forceinline__ int chamfer_hilbert15(unsigned x, unsigned y, unsigned z)
+{
+    unsigned X[3] = {x, y, z};
+#pragma unroll
+    for (unsigned Q = 16; Q > 1; Q >>= 1) {
+        const unsigned P = Q - 1;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const bool set = (X[i] & Q) != 0;
+            const unsigned t = (X[0] ^ X[i]) & P;
+            X[0] ^= set ? P : t;
+            if (i != 0)
+                X[i] ^= set ? 0u : t;
+        }
+    }
+    X[1] ^= X[0];
+    X[2] ^= X[1];
+    unsigned t = 0;
+#pragma unroll
+    for (unsigned Q = 16; Q > 1; Q >>= 1)
+        t ^= (X[2] & Q) ? Q - 1 : 0u;
+    X[0] ^= t;
+    X[1] ^= t;
+    X[2] ^= t;
+    return (chamfer_morton5((int)X[0]) << 2) | (chamfer_morton5((int)X[1]) << 1) |
+           chamfer_morton5((int)X[2]);
+}
+
+constexpr int CHAMFER_SORT_CELLS = 32768;
+
+// Bounding box of a cloud and the cell of every point. CHAMFER_CELL_PARTS workgroups per
+// cloud: each finds the bounding box of the whole cloud for itself (a pass over memory)
+// and then computes the cells of its share of the points (the arithmetic of the launch),
+// kept where the key terms will go. Points are loaded U at a time per lane so that a pass
+// over the cloud is a few round trips to memory.
+constexpr int CHAMFER_CELL_PARTS = 4;
+
+__global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
+{
+    constexpr int NT = 1024, NW = NT / TK_WAVE, U = 8, PARTS = CHAMFER_CELL_PARTS;
+    __shared__ float sred[NW][8];
+    __shared__ int sbad;
+    const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
+    const int cloud = (int)blockIdx.x / PARTS, part = (int)blockIdx.x - cloud * PARTS;
+    const int which = cloud >= a.B;
+    const int b = cloud - which * a.B;
+    const int n = a.n[which], npad = a.npad[which];
+    const float *__restrict__ P = a.xyz[which] + (int64_t)b * n * 3;
+    unsigned short *__restrict__ cells =
+        reinterpret_cast<unsigned short *>(a.terms[which] + (int64_t)b * npad * 2);
+    ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
+    const float INF = __builtin_huge_valf();
+
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    bool bad = false;
+    for (int base = 0; base < n; base += NT * U) {
+        TkPoint3<float> p[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * NT + tid;
+            p[u] = tk_load3<float>(P + (int64_t)(j < n ? j : n - 1) * 3);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float v[3] = {p[u].x, p[u].y, p[u].z};
+#pragma unroll
+            for (int ax = 0; ax < 3; ++ax) {
+                bad |= !(v[ax] - v[ax] == 0.0f);
+                lo[ax] = __builtin_fminf(lo[ax], v[ax]);
+                hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
+            }
+        }
+    }
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        lo[ax] = wave_reduce_min(lo[ax]);
+        hi[ax] = wave_reduce_max(hi[ax]);
+    }
+    if (tid == 0)
+        sbad = 0;
+    __syncthreads();
+    if (lane == 0) {
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            sred[wave][ax] = lo[ax];
+            sred[wave][3 + ax] = hi[ax];
+        }
+    }
+    if (bad)
+        sbad = 1;
+    __syncthreads();
+    float cc[3], ext = 0.0f;
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        float l = sred[0][ax], h = sred[0][3 + ax];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][ax]);
+            h = __builtin_fmaxf(h, sred[w][3 + ax]);
+        }
+        lo[ax] = l;
+        hi[ax] = h;
+        cc[ax] = 0.5f * l + 0.5f * h;
+        ext = __builtin_fmaxf(ext, 0.5f * h - 0.5f * l);
+    }
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
+    const bool safe = n > 0 && sbad == 0 && (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) &&
+                      (c2 - c2 == 0.0f) && (ext - ext == 0.0f) &&
+                      (ext == 0.0f || (ebits >= -40 && ebits <= 40));
+    if (tid == 0 && part == 0) {
+        a.flags[which * a.B + b] = 0;
+        hdr->c[0] = c0;
+        hdr->c[1] = c1;
+        hdr->c[2] = c2;
+        hdr->scale =
+            ext == 0.0f ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
+        hdr->kmax2_bits = 0;
+        hdr->unsafe = safe ? 0 : 1;
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            hdr->lo[ax] = lo[ax];
+            hdr->hi[ax] = hi[ax];
+        }
+    }
+    if (!safe)  // uniform over the workgroup
+        return;
+    // cells: 32 per axis over the largest extent (a point on the upper face: cell 31)
+    const float inv = ext > 0.0f ? (16.0f / ext) * 0.99999f : 0.0f;
+    const int share = (n + PARTS - 1) / PARTS;
+    const int first = part * share, last = first + share < n ? first + share : n;
+    for (int j = first + tid; j < last; j += NT) {
+        const TkPoint3<float> p = tk_load3<float>(P + (int64_t)j * 3);
+        int ix = (int)((p.x - lo[0]) * inv), iy = (int)((p.y - lo[1]) * inv);
+        int iz = (int)((p.z - lo[2]) * inv);
+        ix = ix > 31 ? 31 : ix;
+        iy = iy > 31 ? 31 : iy;
+        iz = iz > 31 ? 31 : iz;
+        cells[j] = (unsigned short)chamfer_hilbert15((unsigned)ix, (unsigned)iy, (unsigned)iz);
+    }
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ int wave_inclusive_sum(int v)
+{
+    // within rows of 16 lanes, then row 0 -> 1, 2 -> 3 and rows 0..1 -> 2..3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31
+    return v;
+}
+
+// One workgroup per cloud: counting sort of the points by cell.
+__global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
+{
+    constexpr int NT = 1024, NW = NT / TK_WAVE, CELLS = CHAMFER_SORT_CELLS, U = 8;
+    extern __shared__ int hist[];  // CELLS counters
+    __shared__ int swave[NW];
+    const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
+    const int which = (int)blockIdx.x >= a.B;
+    const int b = (int)blockIdx.x - which * a.B;
+    const int n = a.n[which], npad = a.npad[which];
+    if (a.hdr[which * a.B + b].unsafe != 0)  // uniform over the workgroup
+        return;
+    const float *__restrict__ P = a.xyz[which] + (int64_t)b * n * 3;
+    float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
+    const unsigned short *__restrict__ cells =
+        reinterpret_cast<const unsigned short *>(a.terms[which] + (int64_t)b * npad * 2);
+    for (int i = tid; i < CELLS; i += NT)
+        hist[i] = 0;
+    __syncthreads();
+    for (int base = 0; base < n; base += NT * U) {
+        int cell[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * NT + tid;
+            cell[u] = cells[j < n ? j : n - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (base + u * NT + tid < n)
+                atomicAdd(&hist[cell[u]], 1);
+        }
+    }
+    __syncthreads();
+    // Every wave turns its 2048 counters into starting positions within its range, 64
+    // at a time; the ranges' own starts are added when a position is taken.
+    {
+        constexpr int PER_WAVE = CELLS / NW;
+        int carry = 0;
+        for (int i = 0; i < PER_WAVE; i += TK_WAVE) {
+            const int at = wave * PER_WAVE + i + lane;
+            const int count = hist[at];
+            const int incl = wave_inclusive_sum(count);
+            hist[at] = carry + incl - count;
+            carry += __builtin_amdgcn_readlane(incl, TK_WAVE - 1);
+        }
+        if (lane == 0)
+            swave[wave] = carry;
+    }
+    __syncthreads();
+    int wave_start[NW];
+    {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            wave_start[w] = run;
+            run += swave[w];
+        }
+    }
+    for (int base = 0; base < n; base += NT * U) {
+        TkPoint3<float> p[U];
+        int cell[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * NT + tid;
+            const int jj = j < n ? j : n - 1;
+            p[u] = tk_load3<float>(P + (int64_t)jj * 3);
+            cell[u] = cells[jj];
+        }
+        int pos[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * NT + tid;
+            pos[u] = j < n ? atomicAdd(&hist[cell[u]], 1) : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * NT + tid;
+            int start = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                start = (cell[u] >> 11) == w ? wave_start[w] : start;
+            if (j < n)
+                sorted[pos[u] + start] =
+                    make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, j));
+        }
+    }
+}
+
+// Key terms and bounding boxes of the sorted tiles, one lane per point; the padding up to
+// a whole number of 128 points is written here too.
+__global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, int blocks0)
+{
+    const int tid = threadIdx.x;
+    const int which = (int)blockIdx.x >= blocks0;
+    const int lb = (int)blockIdx.x - which * blocks0;
+    const int n = a.n[which], npad = a.npad[which];
+    // (npad is a multiple of 128: a cloud's last block may be half empty)
+    const int bpc = (npad + 255) / 256;
+    const int b = lb / bpc;
+    const int i = (lb - b * bpc) * 256 + tid;
+    ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
+    if (hdr->unsafe != 0 || i >= npad)  // (uniform over each half wave: npad % 32 == 0)
+        return;
+    float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
+    uint4 *__restrict__ terms = a.terms[which] + (int64_t)b * npad * 2;
+    float4 *__restrict__ boxes = a.boxes[which] + (int64_t)b * (npad / 32) * 2;
+    const float INF = __builtin_huge_valf();
+    const float c0 = hdr->c[0], c1 = hdr->c[1], c2 = hdr->c[2], scale = hdr->scale;
+    const bool exists = i < n;
+    const float qnan = __builtin_nanf("");
+    float4 s = make_float4(qnan, qnan, qnan, __builtin_bit_cast(float, -1));
+    if (exists)
+        s = sorted[i];
+    else
+        sorted[i] = s;
+    const float x = ((exists ? s.x : c0) - c0) * scale;
+    const float y = ((exists ? s.y : c1) - c1) * scale;
+    const float z = ((exists ? s.z : c2) - c2) * scale;
+    const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+    uint4 h0, h1;
+    chamfer_key_terms(x, y, z, nn, exists, h0, h1);
+    uint4 *tile = terms + (i >> 5) * 64 + (i & 31);
+    tile[0] = h0;
+    tile[32] = h1;
+    float bl[3] = {exists ? x : INF, exists ? y : INF, exists ? z : INF};
+    float bh[3] = {exists ? x : -INF, exists ? y : -INF, exists ? z : -INF};
+    float kmax2 = nn;  // (0 for padding)
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            bl[ax] = __builtin_fminf(bl[ax], __shfl_xor(bl[ax], o));
+            bh[ax] = __builtin_fmaxf(bh[ax], __shfl_xor(bh[ax], o));
+        }
+        kmax2 = __builtin_fmaxf(kmax2, __shfl_xor(kmax2, o));
+    }
+    if ((i & 31) == 0) {
+        boxes[(i >> 5) * 2 + 0] = make_float4(bl[0], bl[1], bl[2], 0.0f);
+        boxes[(i >> 5) * 2 + 1] = make_float4(bh[0], bh[1], bh[2], 0.0f);
+        // non-negative floats order as their bit patterns
+        atomicMax(&hdr->kmax2_bits, __builtin_bit_cast(int, kmax2));
+    }
+}
+
+struct ChamferPrunedArgs {
+    const float4 *sorted[2];
+    const uint4 *terms[2];
+    const float4 *boxes[2];
+    const ChamferSortedHdr *hdr;
+    int *flags;
+    float *dist[2];
+    int64_t *idx[2];
+    int n[2], npad[2];
+    int B;
+    int waves_per_cloud[2];
+    int waves0;  // waves of direction 0 (queries: cloud 0); the rest belong to direction 1
+};
+
+__device__ __forceinline__ int wave_reduce_min_int(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int other = __shfl_xor(v, o);
+        v = other < v ? other : v;
+    }
+    return v;
+}
+
+template <int NQB, int RMAX>
+__global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & (TK_WAVE - 1);
+    const int col = lane & 31, half = lane >> 5;
+    const float INF = __builtin_huge_valf();
+    // the workgroups of a cloud on one XCD, as in chamfer_decode_block
+    int lb = blockIdx.x;
+    {
+        const int nb = gridDim.x, per = nb >> 3, full = per << 3;
+        if (lb < full)
+            lb = (lb & 7) * per + (lb >> 3);
+    }
+    int wid = __builtin_amdgcn_readfirstlane(lb * 4 + tid / TK_WAVE);
+    const int which = wid >= a.waves0;
+    if (which)
+        wid -= a.waves0;
+    const int wpc = a.waves_per_cloud[which];
+    if (wid >= a.B * wpc)
+        return;
+    const int b = wid / wpc, qw = wid - b * wpc;
+    const int nq = a.n[which], npq = a.npad[which], npk = a.npad[1 - which];
+    const ChamferSortedHdr *hq = a.hdr + which * a.B + b;
+    const ChamferSortedHdr *hk = a.hdr + (1 - which) * a.B + b;
+    int *flag = a.flags + which * a.B + b;
+    const float c0 = hk->c[0], c1 = hk->c[1], c2 = hk->c[2], scale = hk->scale;
+    // the query cloud's farthest corner from the key cloud's centre, in key extents
+    float far2 = 0.0f;
+    {
+        const float cc[3] = {c0, c1, c2};
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            const float m = __builtin_fmaxf(__builtin_fabsf(hq->lo[ax] - cc[ax]),
+                                            __builtin_fabsf(hq->hi[ax] - cc[ax])) * scale;
+            far2 = __builtin_fmaf(m, m, far2);
+        }
+    }
+    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f)) {  // uniform over the wave
+        if (lane == 0)
+            atomicOr(flag, 1);
+        return;
+    }
+    if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+        return;  // the cloud goes to the other kernel anyway
+    const float4 *__restrict__ SQ = a.sorted[which] + (int64_t)b * npq;
+    const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
+    const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
+    const float4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32) * 2;
+    const int ntiles = npk / 32;
+    const int rounds = (ntiles + TK_WAVE - 1) / TK_WAVE;  // <= RMAX
+    const float kmax =
+        __builtin_sqrtf(__builtin_bit_cast(float, hk->kmax2_bits)) * 1.000001f;
+    const float guard = 1e-36f * scale * scale;
+
+    // ---- queries ----
+    tk_f16x8 qterm[NQB];
+    float qnorm[NQB], qn2[NQB], rx[NQB], ry[NQB], rz[NQB];
+    int qid[NQB];
+    float v0[NQB], v1[NQB], v2[NQB];
+    int id0[NQB], id1[NQB];
+    float blo[3] = {INF, INF, INF}, bhi[3] = {-INF, -INF, -INF};
+    float qnmax = 0.0f;
+#pragma unroll
+    for (int g = 0; g < NQB; ++g) {
+        const float4 s = SQ[(qw * NQB + g) * 32 + col];
+        qid[g] = __builtin_bit_cast(int, s.w);
+        const bool ok = qid[g] >= 0;
+        rx[g] = s.x;
+        ry[g] = s.y;
+        rz[g] = s.z;
+        const float px = ((ok ? s.x : c0) - c0) * scale;
+        const float py = ((ok ? s.y : c1) - c1) * scale;
+        const float pz = ((ok ? s.z : c2) - c2) * scale;
+        qn2[g] = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px));
+        qnorm[g] = 1.000001f * __builtin_sqrtf(qn2[g]);
+        qterm[g] = __builtin_bit_cast(tk_f16x8, chamfer_query_terms(px, py, pz, half));
+        v0[g] = v1[g] = v2[g] = INF;
+        id0[g] = id1[g] = -1;
+        if (ok) {
+            blo[0] = __builtin_fminf(blo[0], px);
+            blo[1] = __builtin_fminf(blo[1], py);
+            blo[2] = __builtin_fminf(blo[2], pz);
+            bhi[0] = __builtin_fmaxf(bhi[0], px);
+            bhi[1] = __builtin_fmaxf(bhi[1], py);
+            bhi[2] = __builtin_fmaxf(bhi[2], pz);
+            qnmax = __builtin_fmaxf(qnmax, qnorm[g]);
+        }
+    }
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        blo[ax] = wave_reduce_min(blo[ax]);
+        bhi[ax] = wave_reduce_max(bhi[ax]);
+    }
+    if (!(blo[0] <= bhi[0]))  // a wave of padding only (uniform over the wave)
+        return;
+    qnmax = wave_reduce_max(qnmax);
+    const float rw = kmax + qnmax;
+    const float slackw = rw * rw * 7.6293945e-06f + guard;  // 2^-17 R of the wave
+
+    // squared gap between the wave's patch and the box of each of this lane's tiles (tile
+    // r * 64 + lane in g2[r]; an empty box or no tile: +inf)
+    float g2[RMAX];
+#pragma unroll
+    for (int r0 = 0; r0 < RMAX; r0 += 8) {  // eight boxes in flight at a time
+        float4 bl[8], bh[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int t = (r0 + r) * TK_WAVE + lane;
+            const int tt = t < ntiles ? t : 0;
+            bl[r] = BX[tt * 2];
+            bh[r] = BX[tt * 2 + 1];
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const float4 l = bl[r], h = bh[r];
+            const float gx = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.x - bhi[0], blo[0] - h.x));
+            const float gy = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.y - bhi[1], blo[1] - h.y));
+            const float gz = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.z - bhi[2], blo[2] - h.z));
+            g2[r0 + r] = (r0 + r) * TK_WAVE + lane < ntiles
+                             ? __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx))
+                             : INF;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const tk_f32x16 zero = {};
+    auto sweep_tile = [&](const tk_f16x8 &ka, int t) {
+#pragma unroll
+        for (int g = 0; g < NQB; ++g) {
+            const tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qterm[g], zero, 0, 0, 0);
+            const float x = chamfer_fold16(INF, acc);
+            const bool lt0 = x < v0[g];
+            const bool lt1 = x < v1[g];
+            id1[g] = lt1 ? t : id1[g];
+            id1[g] = lt0 ? id0[g] : id1[g];
+            id0[g] = lt0 ? t : id0[g];
+            v2[g] = __builtin_amdgcn_fmed3f(v1[g], v2[g], x);
+            v1[g] = __builtin_amdgcn_fmed3f(v0[g], v1[g], x);
+            v0[g] = __builtin_amdgcn_fmed3f(-INF, v0[g], x);
+        }
+    };
+    unsigned swept = 0;  // bit r: tile r * 64 + lane has been swept
+    int nswept = 0;
+    auto run_phase = [&](float thr) {
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+            if (r >= rounds)
+                break;
+            const int mine = r * TK_WAVE + lane;
+            const bool take = mine < ntiles && !((swept >> r) & 1u) && g2[r] <= thr;
+            unsigned long long m = __builtin_amdgcn_ballot_w64(take);
+            if (take)
+                swept |= 1u << r;
+            if (m == 0)
+                continue;
+            while (m != 0) {  // four tiles in flight at a time
+                int t[4];
+                uint4 ka[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    t[u] = -1;
+                    if (m != 0) {
+                        t[u] = r * TK_WAVE + (int)__builtin_ctzll(m);
+                        m &= m - 1;
+                        ka[u] = TK[(int64_t)t[u] * 64 + lane];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (t[u] >= 0) {
+                        sweep_tile(__builtin_bit_cast(tk_f16x8, ka[u]), t[u]);
+                        ++nswept;
+                    }
+                }
+            }
+        }
+    };
+    // an upper bound of every query's squared distance to its nearest key so far
+    auto bound = [&]() {
+        float ub = -INF;
+#pragma unroll
+        for (int g = 0; g < NQB; ++g) {
+            const float best = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
+            ub = qid[g] >= 0 ? __builtin_fmaxf(ub, best + qn2[g]) : ub;
+        }
+        return wave_reduce_max(ub);
+    };
+
+    // ---- tiles that overlap the patch; without any, the nearest tile ----
+    run_phase(0.0f);
+    if (nswept == 0) {
+        float best = INF;
+        int at = -1;
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+            if (g2[r] < best) {
+                best = g2[r];
+                at = r * TK_WAVE + lane;
+            }
+        }
+        const float least = wave_reduce_min(best);
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(best == least && at >= 0);
+        if (m == 0) {  // no key tile holds a point (cannot happen with nk >= 1): hand over
+            if (lane == 0)
+                atomicOr(flag, 1);
+            return;
+        }
+        const int t = __builtin_amdgcn_readlane(at, (int)__builtin_ctzll(m));
+        if (lane == (t & (TK_WAVE - 1)))
+            swept |= 1u << (t / TK_WAVE);
+        sweep_tile(__builtin_bit_cast(tk_f16x8, TK[(int64_t)t * 64 + lane]), t);
+        ++nswept;
+    }
+    // ---- everything within reach, nearest first in three passes ----
+    run_phase((bound() + slackw) * 0.0625f);
+    run_phase((bound() + slackw) * 0.25f);
+    run_phase((bound() + slackw) * 1.001f);
+
+    // ---- exact evaluation of each half's candidate tiles, then the merge ----
+    unsigned over_mask[NQB];
+    int nover = 0;
+#pragma unroll
+    for (int g = 0; g < NQB; ++g) {
+        const bool ok = qid[g] >= 0;
+        const float best_score = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
+        const float r = kmax + qnorm[g];
+        const float thr = best_score + (r * r * 7.6293945e-06f + guard);  // 2^-17 R
+        const bool crowded = v2[g] <= thr;  // three or more candidate tiles in this half
+        const bool over =
+            ok && ((__builtin_amdgcn_ballot_w64(crowded) >> col & 0x100000001ull) != 0);
+        float bestd = INF;
+        int bestj = -1;
+        if (ok && !over) {
+            const int ta = v0[g] <= thr ? id0[g] : -1, tb = v1[g] <= thr ? id1[g] : -1;
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                const int tile = pass == 0 ? ta : tb;
+                if (tile < 0)
+                    continue;
+                // this half's keys of the tile: runs of 4 keys, 8 keys apart
+                const float4 *p = SK + (int64_t)tile * 32 + half * 4;
+                float4 f[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    f[e] = p[(e >> 2) * 8 + (e & 3)];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float dd = tk_dist2<float>(f[e].x, f[e].y, f[e].z, rx[g], ry[g], rz[g]);
+                    const int oj = __builtin_bit_cast(int, f[e].w);
+                    if (dd < bestd || (dd == bestd && oj < bestj)) {
+                        bestd = dd;
+                        bestj = oj;
+                    }
+                }
+            }
+        }
+        // the other half's result: smaller distance, then lower key index
+        const float od = __shfl_xor(bestd, 32);
+        const int oj = __shfl_xor(bestj, 32);
+        if (oj >= 0 && (bestj < 0 || od < bestd || (od == bestd && oj < bestj))) {
+            bestd = od;
+            bestj = oj;
+        }
+        if (half == 0 && ok && !over) {
+            const int64_t o = (int64_t)b * nq + qid[g];
+            a.dist[which][o] = bestd;
+            a.idx[which][o] = (int64_t)bestj;
+        }
+        over_mask[g] = (unsigned)__builtin_amdgcn_ballot_w64(over && half == 0);
+        nover += __builtin_popcount(over_mask[g]);
+    }
+    if (nover == 0)
+        return;
+    // Exact scans cost a pass over the swept tiles each: beyond a budget the cloud is
+    // handed to the other kernel (heavy ties: quantised or duplicated points).
+    if ((int64_t)nover * nswept > 16384) {
+        if (lane == 0)
+            atomicOr(flag, 1);
+        return;
+    }
+    // ---- queries with three or more candidate tiles: exact scan of the swept tiles ----
+#pragma unroll
+    for (int g = 0; g < NQB; ++g) {
+        unsigned m = over_mask[g];
+        while (m != 0) {
+            const int src = __builtin_ctz(m);
+            m &= m - 1;
+            const float qx = __builtin_bit_cast(
+                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rx[g]), src));
+            const float qy = __builtin_bit_cast(
+                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ry[g]), src));
+            const float qz = __builtin_bit_cast(
+                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rz[g]), src));
+            const int out = __builtin_amdgcn_readlane(qid[g], src);
+            float bestd = INF;
+            int bestj = -1;
+            for (int r = 0; r < rounds; ++r) {
+                if (!((swept >> r) & 1u))
+                    continue;
+                const float4 *p = SK + (int64_t)(r * TK_WAVE + lane) * 32;
+                for (int e = 0; e < 32; ++e) {
+                    const float4 f = p[e];
+                    const float dd = tk_dist2<float>(f.x, f.y, f.z, qx, qy, qz);
+                    const int oj = __builtin_bit_cast(int, f.w);
+                    if (dd < bestd || (dd == bestd && oj < bestj)) {
+                        bestd = dd;
+                        bestj = oj;
+                    }
+                }
+            }
+            const float least = wave_reduce_min(bestd);
+            const int cand = (bestd == least && bestj >= 0) ? bestj : 0x7fffffff;
+            const int first = wave_reduce_min_int(cand);
+            if (lane == 0) {
+                const int64_t o = (int64_t)b * nq + out;
+                a.dist[which][o] = first == 0x7fffffff ? INF : least;
+                a.idx[which][o] = first == 0x7fffffff ? -1 : (int64_t)first;
+            }
+        }
+    }
+}
+
+// The sorted path serves clouds of 2048 to 65536 points each (a lane's 32-bit mask of
+// swept tiles covers 2048 tiles of 32 keys).
+constexpr int64_t CHAMFER_SORTED_MIN = 2048, CHAMFER_SORTED_MAX = 65536;
+
+inline bool chamfer_sorted_serves(int64_t B, int64_t N1, int64_t N2)
+{
+    return B >= 1 && B <= (1 << 20) && N1 >= CHAMFER_SORTED_MIN && N2 >= CHAMFER_SORTED_MIN &&
+           N1 <= CHAMFER_SORTED_MAX && N2 <= CHAMFER_SORTED_MAX;
+}
+
+struct ChamferSortedLayout {
+    size_t hdr, flags, sorted[2], terms[2], boxes[2], total;
+    int64_t npad[2];
+};
+
+inline ChamferSortedLayout chamfer_sorted_layout(int64_t B, int64_t N1, int64_t N2)
+{
+    ChamferSortedLayout l;
+    const int64_t n[2] = {N1, N2};
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        const size_t here = at;
+        at += (bytes + 255) / 256 * 256;
+        return here;
+    };
+    l.hdr = take((size_t)2 * B * sizeof(ChamferSortedHdr));
+    l.flags = take((size_t)2 * B * sizeof(int));
+    for (int w = 0; w < 2; ++w) {
+        l.npad[w] = (n[w] + 127) / 128 * 128;
+        l.sorted[w] = take((size_t)B * l.npad[w] * sizeof(float4));
+        l.terms[w] = take((size_t)B * l.npad[w] * 2 * sizeof(uint4));
+        l.boxes[w] = take((size_t)B * (l.npad[w] / 32) * 2 * sizeof(float4));
+    }
+    l.total = at;
+    return l;
+}
+
+int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
+                           int64_t N2, float *dist1, int64_t *idx1, float *dist2, int64_t *idx2,
+                           void *workspace, hipStream_t s)
+{
+    constexpr int NQB = 2;
+    const ChamferSortedLayout l = chamfer_sorted_layout(B, N1, N2);
+    char *ws = static_cast<char *>(workspace);
+    ChamferSortArgs sa;
+    ChamferPrunedArgs pa;
+    const float *xyz[2] = {xyz1, xyz2};
+    const int64_t n[2] = {N1, N2};
+    for (int w = 0; w < 2; ++w) {
+        sa.xyz[w] = xyz[w];
+        sa.sorted[w] = reinterpret_cast<float4 *>(ws + l.sorted[w]);
+        sa.terms[w] = reinterpret_cast<uint4 *>(ws + l.terms[w]);
+        sa.boxes[w] = reinterpret_cast<float4 *>(ws + l.boxes[w]);
+        sa.n[w] = (int)n[w];
+        sa.npad[w] = (int)l.npad[w];
+        pa.sorted[w] = sa.sorted[w];
+        pa.terms[w] = sa.terms[w];
+        pa.boxes[w] = sa.boxes[w];
+        pa.n[w] = sa.n[w];
+        pa.npad[w] = sa.npad[w];
+        pa.waves_per_cloud[w] = (int)((l.npad[w] + 32 * NQB - 1) / (32 * NQB));
+    }
+    sa.hdr = reinterpret_cast<ChamferSortedHdr *>(ws + l.hdr);
+    sa.flags = reinterpret_cast<int *>(ws + l.flags);
+    sa.B = (int)B;
+    pa.hdr = sa.hdr;
+    pa.flags = sa.flags;
+    pa.dist[0] = dist1;
+    pa.dist[1] = dist2;
+    pa.idx[0] = idx1;
+    pa.idx[1] = idx2;
+    pa.B = (int)B;
+    const int64_t waves0 = B * pa.waves_per_cloud[0], waves1 = B * pa.waves_per_cloud[1];
+    if (waves0 + waves1 > TK_MAX_I32)
+        return TK3D_ERR_UNSUPPORTED;
+    pa.waves0 = (int)waves0;
+    constexpr size_t lds = (size_t)CHAMFER_SORT_CELLS * sizeof(int);
+    const int allowed = tk_allow_dynamic_lds<chamfer_sort_kernel>((int)lds);
+    if (allowed != TK3D_OK)
+        return allowed;
+    hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
+                       dim3(1024), 0, s, sa);
+    hipLaunchKernelGGL(chamfer_sort_kernel, dim3((unsigned)(2 * B)), dim3(1024), lds, s, sa);
+    const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
+    hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s, sa,
+                       (int)tb0);
+    const dim3 grid((unsigned)((waves0 + waves1 + 3) / 4));
+    if (l.npad[0] <= 16384 && l.npad[1] <= 16384)
+        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 8>), grid, dim3(256), 0, s, pa);
+    else
+        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 32>), grid, dim3(256), 0, s, pa);
+    const int rc = tk_launch_status();
+    if (rc != TK3D_OK)
+        return rc;
+    // whatever the waves above handed over (none on ordinary input: its workgroups leave
+    // at once)
+    return chamfer_forward_filter_launch<4, 512, 64, 512>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                          dist2, idx2, s, 1, sa.flags);
+}
+
 template <typename T>
 int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
                      const int64_t *idx1, const int64_t *idx2, int64_t B, int64_t N1,
@@ -1778,6 +2611,26 @@ int tk3d_chamfer_distance_forward_f32(const float *xyz1, const float *xyz2, int6
                                       void *stream)
 {
     return chamfer_forward<float>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
+}
+
+size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2)
+{
+    return chamfer_sorted_serves(B, N1, N2) ? chamfer_sorted_layout(B, N1, N2).total : 0;
+}
+
+int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2, int64_t B,
+                                         int64_t N1, int64_t N2, float *dist1, int64_t *idx1,
+                                         float *dist2, int64_t *idx2, void *workspace,
+                                         size_t workspace_bytes, void *stream)
+{
+    if (workspace == nullptr || !chamfer_sorted_serves(B, N1, N2) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+        workspace_bytes < chamfer_sorted_layout(B, N1, N2).total)
+        return chamfer_forward<float>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
+    if (!xyz1 || !xyz2 || !dist1 || !idx1 || !dist2 || !idx2)
+        return TK3D_ERR_NULL_POINTER;
+    return chamfer_forward_sorted(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, workspace,
+                                  (hipStream_t)stream);
 }
 
 int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2, int64_t B,
