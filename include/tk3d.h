@@ -70,15 +70,18 @@ int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2,
                                       int64_t *idx2, void *stream);
 
 /* The same operation (chamfer_distance_kernel.cu:91-151) for callers that can lend
- * scratch memory: with `workspace` (256-byte aligned device memory of at least
- * tk3d_chamfer_distance_forward_workspace_bytes(B, N1, N2) bytes, contents irrelevant
+ * scratch memory. With `workspace` (256-byte aligned device memory of at least
+ * tk3d_chamfer_distance_forward_workspace_bytes(B, N1, N2, 1) bytes, contents irrelevant
  * before and after) both clouds are first sorted along a space-filling curve, and a wave
- * then sweeps only the key tiles that can hold a nearest neighbour of its queries.
- * Results are bit-identical to tk3d_chamfer_distance_forward_f32 for every input. The
- * size function returns 0 for shapes this path does not serve (clouds under 2048 or over
- * 65536 points); with a null or short workspace the call is
- * tk3d_chamfer_distance_forward_f32. */
-size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2);
+ * then sweeps only the key tiles that can hold a nearest neighbour of its queries; five
+ * kernels are enqueued. Results are bit-identical to tk3d_chamfer_distance_forward_f32 for
+ * every input. The size function returns 0 for shapes the path cannot serve (a cloud of
+ * more than 65536 points, B = 0) and, with always = 0, also for shapes where it is not
+ * the faster route (small or very unequal clouds): callers that pass on that size, and a
+ * null workspace when it is 0, get the faster route for every shape. With a null, short
+ * or misaligned workspace the call is tk3d_chamfer_distance_forward_f32. */
+size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2,
+                                                     int always);
 int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2,
                                          int64_t B, int64_t N1, int64_t N2,
                                          float *dist1, int64_t *idx1, float *dist2,

@@ -78,14 +78,15 @@ def fps_workspace_bytes(b, n, element_size):
 _chamfer_workspace_fn = None
 
 
-def chamfer_workspace_bytes(b, n1, n2):
-    """Scratch bytes ``tk3d_chamfer_distance_forward_ws_f32`` wants for this shape (0: none)."""
+def chamfer_workspace_bytes(b, n1, n2, always=False):
+    """Scratch bytes ``tk3d_chamfer_distance_forward_ws_f32`` wants for this shape: 0 where
+    the sorted path cannot serve it or, unless ``always``, is not the faster route."""
     global _chamfer_workspace_fn
     if _chamfer_workspace_fn is None:
         fn = lib().tk3d_chamfer_distance_forward_workspace_bytes
         fn.restype = ctypes.c_size_t
         _chamfer_workspace_fn = fn
-    return int(_chamfer_workspace_fn(i64(b), i64(n1), i64(n2)))
+    return int(_chamfer_workspace_fn(i64(b), i64(n1), i64(n2), ctypes.c_int(1 if always else 0)))
 
 
 ERR_UNSUPPORTED = -6  # TK3D_ERR_UNSUPPORTED

@@ -1789,7 +1789,8 @@ struct ChamferSortArgs {
     const float *xyz[2];
     float4 *sorted[2];  // [B, npad]: x, y, z, original index (bits); padding: NaN, -1
     uint4 *terms[2];    // [B, npad / 32][2][32]
-    float4 *boxes[2];   // [B, npad / 32][2]: lo, hi in centred, scaled coordinates
+    uint4 *boxes[2];    // [B, npad / 32]: lo and hi corner in centred, scaled coordinates,
+                        // six fp16 values rounded outwards
     ChamferSortedHdr *hdr;  // [2, B]
     int *flags;             // [2, B]
     int n[2], npad[2];
@@ -1848,7 +1849,7 @@ constexpr int CHAMFER_CELL_PARTS = 4;
 
 __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
 {
-    constexpr int NT = 1024, NW = NT / TK_WAVE, U = 8, PARTS = CHAMFER_CELL_PARTS;
+    constexpr int NT = 1024, NW = NT / TK_WAVE, U = 16, PARTS = CHAMFER_CELL_PARTS;
     __shared__ float sred[NW][8];
     __shared__ int sbad;
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
@@ -1967,7 +1968,7 @@ __device__ __forceinline__ int wave_inclusive_sum(int v)
 // One workgroup per cloud: counting sort of the points by cell.
 __global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
 {
-    constexpr int NT = 1024, NW = NT / TK_WAVE, CELLS = CHAMFER_SORT_CELLS, U = 8;
+    constexpr int NT = 1024, NW = NT / TK_WAVE, CELLS = CHAMFER_SORT_CELLS, U = 16;
     extern __shared__ int hist[];  // CELLS counters
     __shared__ int swave[NW];
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
@@ -2069,7 +2070,7 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
         return;
     float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
     uint4 *__restrict__ terms = a.terms[which] + (int64_t)b * npad * 2;
-    float4 *__restrict__ boxes = a.boxes[which] + (int64_t)b * (npad / 32) * 2;
+    uint4 *__restrict__ boxes = a.boxes[which] + (int64_t)b * (npad / 32);
     const float INF = __builtin_huge_valf();
     const float c0 = hdr->c[0], c1 = hdr->c[1], c2 = hdr->c[2], scale = hdr->scale;
     const bool exists = i < n;
@@ -2101,8 +2102,17 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
         kmax2 = __builtin_fmaxf(kmax2, __shfl_xor(kmax2, o));
     }
     if ((i & 31) == 0) {
-        boxes[(i >> 5) * 2 + 0] = make_float4(bl[0], bl[1], bl[2], 0.0f);
-        boxes[(i >> 5) * 2 + 1] = make_float4(bh[0], bh[1], bh[2], 0.0f);
+        // fp16 corners, moved outwards by more than the rounding to nearest can bring them
+        // back (2^-11 relative, 2^-25 in the subnormal range); an empty box stays (+inf, -inf)
+        unsigned h[6];
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            const float wl = __builtin_fabsf(bl[ax]) * 9.765625e-4f + 1.1920929e-7f;
+            const float wh = __builtin_fabsf(bh[ax]) * 9.765625e-4f + 1.1920929e-7f;
+            h[ax] = bl[ax] > 3.0e38f ? 0x7c00u : tk_f16_bits(bl[ax] - wl);
+            h[3 + ax] = bh[ax] < -3.0e38f ? 0xfc00u : tk_f16_bits(bh[ax] + wh);
+        }
+        boxes[i >> 5] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), 0u);
         // non-negative floats order as their bit patterns
         atomicMax(&hdr->kmax2_bits, __builtin_bit_cast(int, kmax2));
     }
@@ -2111,7 +2121,7 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
 struct ChamferPrunedArgs {
     const float4 *sorted[2];
     const uint4 *terms[2];
-    const float4 *boxes[2];
+    const uint4 *boxes[2];
     const ChamferSortedHdr *hdr;
     int *flags;
     float *dist[2];
@@ -2180,7 +2190,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const float4 *__restrict__ SQ = a.sorted[which] + (int64_t)b * npq;
     const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
     const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
-    const float4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32) * 2;
+    const uint4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32);
     const int ntiles = npk / 32;
     const int rounds = (ntiles + TK_WAVE - 1) / TK_WAVE;  // <= RMAX
     const float kmax =
@@ -2228,6 +2238,13 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     }
     if (!(blo[0] <= bhi[0]))  // a wave of padding only (uniform over the wave)
         return;
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {  // (the same in every lane: scalar registers)
+        blo[ax] = __builtin_bit_cast(
+            float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, blo[ax])));
+        bhi[ax] = __builtin_bit_cast(
+            float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, bhi[ax])));
+    }
     qnmax = wave_reduce_max(qnmax);
     const float rw = kmax + qnmax;
     const float slackw = rw * rw * 7.6293945e-06f + guard;  // 2^-17 R of the wave
@@ -2237,20 +2254,26 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     float g2[RMAX];
 #pragma unroll
     for (int r0 = 0; r0 < RMAX; r0 += 8) {  // eight boxes in flight at a time
-        float4 bl[8], bh[8];
+        if (r0 >= rounds) {  // uniform over the wave: no tiles left
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                g2[r0 + r] = INF;
+            continue;
+        }
+        uint4 box[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const int t = (r0 + r) * TK_WAVE + lane;
-            const int tt = t < ntiles ? t : 0;
-            bl[r] = BX[tt * 2];
-            bh[r] = BX[tt * 2 + 1];
+            box[r] = BX[t < ntiles ? t : 0];
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            const float4 l = bl[r], h = bh[r];
-            const float gx = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.x - bhi[0], blo[0] - h.x));
-            const float gy = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.y - bhi[1], blo[1] - h.y));
-            const float gz = __builtin_fmaxf(0.0f, __builtin_fmaxf(l.z - bhi[2], blo[2] - h.z));
+            const float lx = tk_f16_value(box[r].x & 0xffffu), ly = tk_f16_value(box[r].x >> 16);
+            const float lz = tk_f16_value(box[r].y & 0xffffu), hx = tk_f16_value(box[r].y >> 16);
+            const float hy = tk_f16_value(box[r].z & 0xffffu), hz = tk_f16_value(box[r].z >> 16);
+            const float gx = __builtin_fmaxf(0.0f, __builtin_fmaxf(lx - bhi[0], blo[0] - hx));
+            const float gy = __builtin_fmaxf(0.0f, __builtin_fmaxf(ly - bhi[1], blo[1] - hy));
+            const float gz = __builtin_fmaxf(0.0f, __builtin_fmaxf(lz - bhi[2], blo[2] - hz));
             g2[r0 + r] = (r0 + r) * TK_WAVE + lane < ntiles
                              ? __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx))
                              : INF;
@@ -2275,18 +2298,59 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     };
     unsigned swept = 0;  // bit r: tile r * 64 + lane has been swept
     int nswept = 0;
-    auto run_phase = [&](float thr) {
+    // an upper bound of every query's squared distance to its nearest key so far
+    auto bound = [&]() {
+        float ub = -INF;
 #pragma unroll
-        for (int r = 0; r < RMAX; ++r) {
-            if (r >= rounds)
-                break;
-            const int mine = r * TK_WAVE + lane;
-            const bool take = mine < ntiles && !((swept >> r) & 1u) && g2[r] <= thr;
-            unsigned long long m = __builtin_amdgcn_ballot_w64(take);
-            if (take)
-                swept |= 1u << r;
-            if (m == 0)
-                continue;
+        for (int g = 0; g < NQB; ++g) {
+            const float best = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
+            ub = qid[g] >= 0 ? __builtin_fmaxf(ub, best + qn2[g]) : ub;
+        }
+        return wave_reduce_max(ub);
+    };
+    // Three passes (one copy of the code): the tiles that overlap the patch - without any,
+    // the nearest tile -, then everything within reach, nearest first, at T/4 and T.
+#pragma unroll 1
+    for (int phase = 0; phase < 3; ++phase) {
+        float thr = 0.0f;
+        if (phase > 0) {
+            if (nswept == 0) {  // (phase 1 only) uniform over the wave
+                float best = INF;
+                int at = -1;
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r) {
+                    if (g2[r] < best) {
+                        best = g2[r];
+                        at = r * TK_WAVE + lane;
+                    }
+                }
+                const float least = wave_reduce_min(best);
+                const unsigned long long m =
+                    __builtin_amdgcn_ballot_w64(best == least && at >= 0);
+                if (m == 0) {  // no key tile holds a point (cannot happen with nk >= 1)
+                    if (lane == 0)
+                        atomicOr(flag, 1);
+                    return;
+                }
+                const int t = __builtin_amdgcn_readlane(at, (int)__builtin_ctzll(m));
+                if (lane == (t & (TK_WAVE - 1)))
+                    swept |= 1u << (t / TK_WAVE);
+                sweep_tile(__builtin_bit_cast(tk_f16x8, TK[(int64_t)t * 64 + lane]), t);
+                ++nswept;
+            }
+            const float reach = phase == 1 ? 0.25f : 1.001f;
+            // (finite, so that the +inf of a tile that does not exist never passes)
+            thr = __builtin_fminf((bound() + slackw) * reach, 3.0e38f);
+        }
+        unsigned takes = 0;
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+            takes |= g2[r] <= thr ? 1u << r : 0u;
+        takes &= ~swept;
+        swept |= takes;
+#pragma unroll 1
+        for (int r = 0; r < rounds; ++r) {
+            unsigned long long m = __builtin_amdgcn_ballot_w64(((takes >> r) & 1u) != 0);
             while (m != 0) {  // four tiles in flight at a time
                 int t[4];
                 uint4 ka[4];
@@ -2308,47 +2372,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
                 }
             }
         }
-    };
-    // an upper bound of every query's squared distance to its nearest key so far
-    auto bound = [&]() {
-        float ub = -INF;
-#pragma unroll
-        for (int g = 0; g < NQB; ++g) {
-            const float best = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
-            ub = qid[g] >= 0 ? __builtin_fmaxf(ub, best + qn2[g]) : ub;
-        }
-        return wave_reduce_max(ub);
-    };
-
-    // ---- tiles that overlap the patch; without any, the nearest tile ----
-    run_phase(0.0f);
-    if (nswept == 0) {
-        float best = INF;
-        int at = -1;
-#pragma unroll
-        for (int r = 0; r < RMAX; ++r) {
-            if (g2[r] < best) {
-                best = g2[r];
-                at = r * TK_WAVE + lane;
-            }
-        }
-        const float least = wave_reduce_min(best);
-        const unsigned long long m = __builtin_amdgcn_ballot_w64(best == least && at >= 0);
-        if (m == 0) {  // no key tile holds a point (cannot happen with nk >= 1): hand over
-            if (lane == 0)
-                atomicOr(flag, 1);
-            return;
-        }
-        const int t = __builtin_amdgcn_readlane(at, (int)__builtin_ctzll(m));
-        if (lane == (t & (TK_WAVE - 1)))
-            swept |= 1u << (t / TK_WAVE);
-        sweep_tile(__builtin_bit_cast(tk_f16x8, TK[(int64_t)t * 64 + lane]), t);
-        ++nswept;
     }
-    // ---- everything within reach, nearest first in three passes ----
-    run_phase((bound() + slackw) * 0.0625f);
-    run_phase((bound() + slackw) * 0.25f);
-    run_phase((bound() + slackw) * 1.001f);
 
     // ---- exact evaluation of each half's candidate tiles, then the merge ----
     unsigned over_mask[NQB];
@@ -2454,14 +2478,27 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     }
 }
 
-// The sorted path serves clouds of 2048 to 65536 points each (a lane's 32-bit mask of
-// swept tiles covers 2048 tiles of 32 keys).
-constexpr int64_t CHAMFER_SORTED_MIN = 2048, CHAMFER_SORTED_MAX = 65536;
+// The sorted path can serve clouds of 1 to 65536 points each (a lane's 32-bit mask of
+// swept tiles covers 2048 tiles of 32 keys) ...
+constexpr int64_t CHAMFER_SORTED_MIN = 1, CHAMFER_SORTED_MAX = 65536;
 
-inline bool chamfer_sorted_serves(int64_t B, int64_t N1, int64_t N2)
+inline bool chamfer_sorted_can_serve(int64_t B, int64_t N1, int64_t N2)
 {
     return B >= 1 && B <= (1 << 20) && N1 >= CHAMFER_SORTED_MIN && N2 >= CHAMFER_SORTED_MIN &&
            N1 <= CHAMFER_SORTED_MAX && N2 <= CHAMFER_SORTED_MAX;
+}
+
+// ... and pays where the sweeps it saves outweigh its five launches and the sort: from
+// half a billion pairs per direction on clouds of 4096 points and more whose lengths are
+// within a factor of four (30 timed shapes: B=32, 4096 x 4096 1.08 times faster than the
+// full sweep, B=8, 8192 x 8192 1.16, B=4, 16384 x 16384 1.7, B=32, 16384 x 16384 4.0,
+// B=1, 65536 x 65536 2.4; B=16, 4096 x 4096 0.84 and B=4, 65536 x 2048 0.39 stay with the
+// full sweep).
+inline bool chamfer_sorted_serves(int64_t B, int64_t N1, int64_t N2)
+{
+    const int64_t lo = N1 < N2 ? N1 : N2, hi = N1 < N2 ? N2 : N1;
+    return chamfer_sorted_can_serve(B, N1, N2) && lo >= 4096 && hi <= 4 * lo &&
+           (double)B * (double)N1 * (double)N2 >= 5.0e8;
 }
 
 struct ChamferSortedLayout {
@@ -2485,7 +2522,7 @@ inline ChamferSortedLayout chamfer_sorted_layout(int64_t B, int64_t N1, int64_t 
         l.npad[w] = (n[w] + 127) / 128 * 128;
         l.sorted[w] = take((size_t)B * l.npad[w] * sizeof(float4));
         l.terms[w] = take((size_t)B * l.npad[w] * 2 * sizeof(uint4));
-        l.boxes[w] = take((size_t)B * (l.npad[w] / 32) * 2 * sizeof(float4));
+        l.boxes[w] = take((size_t)B * (l.npad[w] / 32) * sizeof(uint4));
     }
     l.total = at;
     return l;
@@ -2506,7 +2543,7 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
         sa.xyz[w] = xyz[w];
         sa.sorted[w] = reinterpret_cast<float4 *>(ws + l.sorted[w]);
         sa.terms[w] = reinterpret_cast<uint4 *>(ws + l.terms[w]);
-        sa.boxes[w] = reinterpret_cast<float4 *>(ws + l.boxes[w]);
+        sa.boxes[w] = reinterpret_cast<uint4 *>(ws + l.boxes[w]);
         sa.n[w] = (int)n[w];
         sa.npad[w] = (int)l.npad[w];
         pa.sorted[w] = sa.sorted[w];
@@ -2613,9 +2650,12 @@ int tk3d_chamfer_distance_forward_f32(const float *xyz1, const float *xyz2, int6
     return chamfer_forward<float>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
 }
 
-size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2)
+size_t tk3d_chamfer_distance_forward_workspace_bytes(int64_t B, int64_t N1, int64_t N2,
+                                                     int always)
 {
-    return chamfer_sorted_serves(B, N1, N2) ? chamfer_sorted_layout(B, N1, N2).total : 0;
+    const bool wanted =
+        always ? chamfer_sorted_can_serve(B, N1, N2) : chamfer_sorted_serves(B, N1, N2);
+    return wanted ? chamfer_sorted_layout(B, N1, N2).total : 0;
 }
 
 int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2, int64_t B,
@@ -2623,7 +2663,7 @@ int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2, i
                                          float *dist2, int64_t *idx2, void *workspace,
                                          size_t workspace_bytes, void *stream)
 {
-    if (workspace == nullptr || !chamfer_sorted_serves(B, N1, N2) ||
+    if (workspace == nullptr || !chamfer_sorted_can_serve(B, N1, N2) ||
         (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
         workspace_bytes < chamfer_sorted_layout(B, N1, N2).total)
         return chamfer_forward<float>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
