@@ -2308,11 +2308,14 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         }
         return wave_reduce_max(ub);
     };
-    // Three passes (one copy of the code): the tiles that overlap the patch - without any,
-    // the nearest tile -, then everything within reach, nearest first, at T/4 and T.
+    // Up to three passes (one copy of the code): the tiles that overlap the patch - without
+    // any, the nearest tile -, then everything within reach at T. When the first pass met
+    // fewer than four tiles T is still loose, and a pass at T/4 tightens it first.
 #pragma unroll 1
     for (int phase = 0; phase < 3; ++phase) {
         float thr = 0.0f;
+        if (phase == 1 && nswept >= 4)  // uniform over the wave
+            continue;
         if (phase > 0) {
             if (nswept == 0) {  // (phase 1 only) uniform over the wave
                 float best = INF;
