@@ -2432,9 +2432,11 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     }
     if (nover == 0)
         return;
-    // Exact scans cost a pass over the swept tiles each: beyond a budget the cloud is
-    // handed to the other kernel (heavy ties: quantised or duplicated points).
-    if ((int64_t)nover * nswept > 16384) {
+    // An exact scan costs about 13 instructions per two swept tiles (a normal wave issues
+    // 2100 in all): beyond 8192 (query, tile) pairs - half of what sweeping the whole cloud
+    // exactly would cost the wave - the cloud is handed to the other kernel (heavy ties:
+    // quantised or duplicated points).
+    if ((int64_t)nover * nswept > 8192) {
         if (lane == 0)
             atomicOr(flag, 1);
         return;
@@ -2455,17 +2457,27 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             const int out = __builtin_amdgcn_readlane(qid[g], src);
             float bestd = INF;
             int bestj = -1;
+            // two swept tiles at a time, lane l taking key l % 32 of the tile of its half
+#pragma unroll 1
             for (int r = 0; r < rounds; ++r) {
-                if (!((swept >> r) & 1u))
-                    continue;
-                const float4 *p = SK + (int64_t)(r * TK_WAVE + lane) * 32;
-                for (int e = 0; e < 32; ++e) {
-                    const float4 f = p[e];
-                    const float dd = tk_dist2<float>(f.x, f.y, f.z, qx, qy, qz);
-                    const int oj = __builtin_bit_cast(int, f.w);
-                    if (dd < bestd || (dd == bestd && oj < bestj)) {
-                        bestd = dd;
-                        bestj = oj;
+                unsigned long long mm = __builtin_amdgcn_ballot_w64(((swept >> r) & 1u) != 0);
+                while (mm != 0) {
+                    const int t0 = r * TK_WAVE + (int)__builtin_ctzll(mm);
+                    mm &= mm - 1;
+                    int t1 = -1;
+                    if (mm != 0) {
+                        t1 = r * TK_WAVE + (int)__builtin_ctzll(mm);
+                        mm &= mm - 1;
+                    }
+                    const int mine = half == 0 ? t0 : t1;
+                    if (mine >= 0) {
+                        const float4 f = SK[(int64_t)mine * 32 + col];
+                        const float dd = tk_dist2<float>(f.x, f.y, f.z, qx, qy, qz);
+                        const int oj = __builtin_bit_cast(int, f.w);
+                        if (dd < bestd || (dd == bestd && oj < bestj)) {
+                            bestd = dd;
+                            bestj = oj;
+                        }
                     }
                 }
             }
