@@ -190,3 +190,52 @@ def test_full_size_through_the_python_api_uses_the_sorted_path(cuda):
     torch.cuda.synchronize()
     for name, a_, b_ in zip(("dist1", "idx1", "dist2", "idx2"), got, ref):
         assert torch.equal(a_, b_), name
+
+
+def test_captured_in_a_hip_graph_and_replayed(cuda):
+    # five launches, no allocation, no memset, flags cleared by a kernel: the call records
+    # into a graph as it is; replays on new input contents, with eager work in between,
+    # must equal the oracle every time (workspace and outputs held outside the graph)
+    from torkit3d_amd import _lib
+    from torkit3d_amd._lib import i64, ptr, stream_of
+
+    b, n1, n2 = 2, 5000, 6000
+    assert _lib.chamfer_workspace_bytes(b, n1, n2, True) > 0
+    g = gen(17)
+    x1 = sphere_cloud(g, b, n1).to(cuda)
+    x2 = sphere_cloud(g, b, n2).to(cuda)
+    ws = torch.empty((_lib.chamfer_workspace_bytes(b, n1, n2, True),), dtype=torch.uint8,
+                     device=cuda)
+    out = [torch.empty((b, n1), device=cuda), torch.empty((b, n1), dtype=torch.int64, device=cuda),
+           torch.empty((b, n2), device=cuda), torch.empty((b, n2), dtype=torch.int64, device=cuda)]
+    fn = _lib.lib().tk3d_chamfer_distance_forward_ws_f32
+    fn.restype = ctypes.c_int
+
+    def call():
+        assert fn(ptr(x1), ptr(x2), i64(b), i64(n1), i64(n2), *[ptr(t) for t in out],
+                  ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()),
+                  stream_of(x1)) == 0
+
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(side):
+        call()                        # warm-up outside the capture
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for seed, kind in ((18, sphere_cloud), (19, uniform_cloud), (20, lattice_cloud)):
+        g = gen(seed)
+        a = kind(g, b, n1) if kind is not lattice_cloud else lattice_cloud(g, b, n1, 8)
+        c = kind(g, b, n2) if kind is not lattice_cloud else lattice_cloud(g, b, n2, 8)
+        x1.copy_(a)
+        x2.copy_(c)
+        for t in out:
+            t.zero_()
+        (x1.sum() + x2.sum()).item()  # eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle.chamfer_forward(a.numpy(), c.numpy())
+        for name, got, exp in zip(("dist1", "idx1", "dist2", "idx2"), out, want):
+            np.testing.assert_array_equal(got.cpu().numpy(), exp, err_msg="%s seed %d" % (name, seed))
