@@ -2168,6 +2168,27 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const ChamferSortedHdr *hq = a.hdr + which * a.B + b;
     const ChamferSortedHdr *hk = a.hdr + (1 - which) * a.B + b;
     int *flag = a.flags + which * a.B + b;
+    const float4 *__restrict__ SQ = a.sorted[which] + (int64_t)b * npq;
+    const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
+    const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
+    const uint4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32);
+    const int ntiles = npk / 32;
+    const int rounds = (ntiles + TK_WAVE - 1) / TK_WAVE;  // <= RMAX
+    // The wave's queries and the first boxes are requested before anything is known about
+    // the clouds (the addresses are inside the workspace whatever it holds): one round
+    // trip to memory instead of three in a row.
+    float4 squery[NQB];
+    uint4 box0[8];
+#pragma unroll
+    for (int g = 0; g < NQB; ++g)
+        squery[g] = SQ[(qw * NQB + g) * 32 + col];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int t = r * TK_WAVE + lane;
+        box0[r] = BX[t < ntiles ? t : 0];
+    }
+    const int handed_over = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_sched_barrier(0);
     const float c0 = hk->c[0], c1 = hk->c[1], c2 = hk->c[2], scale = hk->scale;
     // the query cloud's farthest corner from the key cloud's centre, in key extents
     float far2 = 0.0f;
@@ -2185,14 +2206,8 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             atomicOr(flag, 1);
         return;
     }
-    if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+    if (handed_over != 0)
         return;  // the cloud goes to the other kernel anyway
-    const float4 *__restrict__ SQ = a.sorted[which] + (int64_t)b * npq;
-    const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
-    const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
-    const uint4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32);
-    const int ntiles = npk / 32;
-    const int rounds = (ntiles + TK_WAVE - 1) / TK_WAVE;  // <= RMAX
     const float kmax =
         __builtin_sqrtf(__builtin_bit_cast(float, hk->kmax2_bits)) * 1.000001f;
     const float guard = 1e-36f * scale * scale;
@@ -2207,7 +2222,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     float qnmax = 0.0f;
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
-        const float4 s = SQ[(qw * NQB + g) * 32 + col];
+        const float4 s = squery[g];
         qid[g] = __builtin_bit_cast(int, s.w);
         const bool ok = qid[g] >= 0;
         rx[g] = s.x;
@@ -2264,7 +2279,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const int t = (r0 + r) * TK_WAVE + lane;
-            box[r] = BX[t < ntiles ? t : 0];
+            box[r] = r0 == 0 ? box0[r] : BX[t < ntiles ? t : 0];
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
