@@ -40,7 +40,7 @@ template <typename T> struct ChamferFwdArgs {
     ChamferDir<T> dir[2];
     int nblocks0;  // workgroups of direction 0; the rest belong to direction 1
     // When set: [2, nbatch] flags, and a workgroup of direction w and batch element b
-    // works only if only_if[w * nbatch + b] is non-zero (vector pre-filter kernel only).
+    // works only if only_if[w * nbatch + b] is non-zero (chamfer_forward_mfma_flagged_kernel only).
     const int *only_if;
     int nbatch;
 };
@@ -320,7 +320,7 @@ __device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict
     out_j = gj == 0x7fffffff ? -1 : gj;
 }
 
-template <int QPL, int BLOCK, int TILE, int STAGE, bool GATED = false>
+template <int QPL, int BLOCK, int TILE, int STAGE>
 __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFwdArgs<float> args)
 {
     static_assert(STAGE % TILE == 0 && TILE % 2 == 0, "tile shapes");
@@ -339,10 +339,6 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
     const int wave = tid / TK_WAVE;
     int b, qblock, slice;
     const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
-    if constexpr (GATED) {
-        if (args.only_if[(int)(&d - args.dir) * args.nbatch + b] == 0)
-            return;  // uniform over the workgroup
-    }
     const int nq = d.nq;
     // This workgroup sweeps keys [k0, k0 + nk); to the filter that slice is the key cloud.
     const int k0 = slice * d.slice_len;
@@ -744,9 +740,11 @@ __device__ __forceinline__ float chamfer_fold16(float m, const tk_f32x16 &acc)
     return m;
 }
 
+// One workgroup's share: query block `qblock` of batch element `b` against key slice
+// `slice` of direction `d`.
 template <int NQB, int BLOCK, int STAGE>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
-chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
+__device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, const int b,
+                                                   const int qblock, const int slice)
 {
     constexpr int NW = BLOCK / TK_WAVE;
     constexpr int QB = NW * NQB * 32;  // queries per workgroup
@@ -770,8 +768,6 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
     const int lane = tid & (TK_WAVE - 1);
     const int wave = tid / TK_WAVE;
     const int col = lane & 31, half = lane >> 5;
-    int b, qblock, slice;
-    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
     const int nq = d.nq;
     const int k0 = slice * d.slice_len;
     const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
@@ -1134,6 +1130,36 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
                                         Q[(int64_t)qi * 3 + 2], &sred[0][0], sidx, bd, bj);
         if (tid == 0)
             chamfer_emit<float>(d, b, qi, k0, bd, bj);
+    }
+}
+
+template <int NQB, int BLOCK, int STAGE>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
+chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
+{
+    int b, qblock, slice;
+    const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
+    chamfer_mfma_block<NQB, BLOCK, STAGE>(d, b, qblock, slice);
+}
+
+// The same sweep for the clouds another kernel has flagged (args.only_if): a fixed, small
+// number of workgroups go through all (direction, batch element, query block) shares and
+// work on those whose cloud carries a flag, so a launch that finds no flag costs little.
+template <int NQB, int BLOCK, int STAGE>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
+chamfer_forward_mfma_flagged_kernel(ChamferFwdArgs<float> args, int total)
+{
+    for (int lb = blockIdx.x; lb < total; lb += gridDim.x) {
+        const int which = lb >= args.nblocks0;
+        const int rest0 = lb - (which ? args.nblocks0 : 0);
+        const ChamferDir<float> &d = args.dir[which];
+        const int b = rest0 / d.blocks_per_batch;
+        const int rest = rest0 - b * d.blocks_per_batch;
+        const int qblock = rest / d.slices, slice = rest - qblock * d.slices;
+        if (args.only_if[which * args.nbatch + b] == 0)  // uniform over the workgroup
+            continue;
+        chamfer_mfma_block<NQB, BLOCK, STAGE>(d, b, qblock, slice);
+        __syncthreads();  // the next share reuses the stage buffers
     }
 }
 
@@ -1574,8 +1600,7 @@ int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
 template <int QPL, int BLOCK = 256, int TILE = 64, int STAGE = 1024>
 int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                                   int64_t N2, float *dist1, int64_t *idx1, float *dist2,
-                                  int64_t *idx2, hipStream_t stream, int slices = 1,
-                                  const int *only_if = nullptr)
+                                  int64_t *idx2, hipStream_t stream, int slices = 1)
 {
     ChamferFwdArgs<float> a;
     int64_t nblocks;
@@ -1583,13 +1608,30 @@ int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t 
         a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, slices, nblocks);
     if (rc != TK3D_OK)
         return rc;
-    a.only_if = only_if;
-    if (only_if != nullptr)
-        return chamfer_forward_run<float>(
-            chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE, true>, BLOCK, a, nblocks, B,
-            stream);
     return chamfer_forward_run<float>(chamfer_forward_filter_kernel<QPL, BLOCK, TILE, STAGE>,
                                       BLOCK, a, nblocks, B, stream);
+}
+
+// The matrix pre-filter on the clouds flagged in `only_if` ([2, B]), unsplit.
+template <int NQB, int BLOCK = 256, int STAGE = 512>
+int chamfer_forward_mfma_flagged_launch(const float *xyz1, const float *xyz2, int64_t B,
+                                        int64_t N1, int64_t N2, float *dist1, int64_t *idx1,
+                                        float *dist2, int64_t *idx2, hipStream_t stream,
+                                        const int *only_if)
+{
+    ChamferFwdArgs<float> a;
+    int64_t nblocks;
+    const int rc = chamfer_fill_args<float, (BLOCK / TK_WAVE) * NQB * 32, 128>(
+        a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, 1, nblocks, 1);
+    if (rc != TK3D_OK)
+        return rc;
+    a.only_if = only_if;
+    const int64_t grid = nblocks < 4 * tk_cu_count() ? nblocks : 4 * tk_cu_count();
+    if (grid == 0)
+        return TK3D_OK;
+    hipLaunchKernelGGL((chamfer_forward_mfma_flagged_kernel<NQB, BLOCK, STAGE>),
+                       dim3((unsigned)grid), dim3(BLOCK), 0, stream, a, (int)nblocks);
+    return tk_launch_status();
 }
 
 template <int NQB, int BLOCK = 256, int STAGE = 512>
@@ -1775,7 +1817,7 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // Input the bound does not cover (non-finite coordinates, extents outside 2^+-40, queries
 // further than 8000 extents from the key cloud) and waves whose exact scans would take
 // long (heavy ties on many swept tiles) raise a flag for their cloud and direction; the
-// vector pre-filter kernel runs behind this one and serves exactly the flagged ones.
+// matrix pre-filter runs behind this one and serves exactly the flagged ones.
 struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
     float c[3];            // centre of the bounding box
     float scale;           // 2^-(exponent of the largest half extent)
@@ -2617,8 +2659,8 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
         return rc;
     // whatever the waves above handed over (none on ordinary input: its workgroups leave
     // at once)
-    return chamfer_forward_filter_launch<4, 512, 64, 512>(xyz1, xyz2, B, N1, N2, dist1, idx1,
-                                                          dist2, idx2, s, 1, sa.flags);
+    return chamfer_forward_mfma_flagged_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+                                                  idx2, s, sa.flags);
 }
 
 template <typename T>
