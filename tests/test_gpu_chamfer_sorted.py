@@ -127,9 +127,11 @@ def test_disjoint_and_nested_clouds(cuda):
     a, c = sphere_cloud(g, 2, 3000), sphere_cloud(g, 2, 4000)
     ws = check_sorted(a + 3.0, c, cuda)            # no key tile overlaps any patch
     assert sum(handed_over(ws, 2)) == 0
-    ws = check_sorted(a * 0.01, c, cuda)           # all queries deep inside the key cloud
-    assert sum(handed_over(ws, 2)) == 0
-    ws = check_sorted(a, c * 0.01, cuda)           # all keys in one small region
+    ws = check_sorted(a * 0.01, c, cuda)           # all queries deep inside the key cloud;
+    assert handed_over(ws, 2) == [0, 0, 1, 1]      # the other way round the keys are dwarfed
+    ws = check_sorted(a, c * 0.01, cuda)           # all keys in one small region:
+    assert handed_over(ws, 2) == [1, 1, 0, 0]      # boxes cannot prune for the far queries
+    ws = check_sorted(a, c * 0.3, cuda)            # a key cloud of a third of the extent stays
     assert sum(handed_over(ws, 2)) == 0
 
 

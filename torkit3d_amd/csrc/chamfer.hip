@@ -1815,8 +1815,10 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // shrinks as tiles are swept, so a tile skipped under an earlier T stays skipped rightly.
 //
 // Input the bound does not cover (non-finite coordinates, extents outside 2^+-40, queries
-// further than 8000 extents from the key cloud) and waves whose exact scans would take
-// long (heavy ties on many swept tiles) raise a flag for their cloud and direction; the
+// further than 8000 extents from the key cloud), a key cloud under a quarter of the query
+// cloud's extent (boxes cannot prune for queries far from all keys) and waves whose exact
+// scans would take long (heavy ties on many swept tiles) raise a flag for their cloud and
+// direction; the
 // matrix pre-filter runs behind this one and serves exactly the flagged ones.
 struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
     float c[3];            // centre of the bounding box
@@ -2243,7 +2245,17 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             far2 = __builtin_fmaf(m, m, far2);
         }
     }
-    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f)) {  // uniform over the wave
+    // A key cloud much smaller than the query cloud: most queries are far from it compared
+    // with its size, every one of its tiles is within their reach, and this kernel would
+    // sweep all pairs at four times the matrix kernel's cost per tile.
+    float extent_q = 0.0f, extent_k = 0.0f;
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        extent_q = __builtin_fmaxf(extent_q, hq->hi[ax] - hq->lo[ax]);
+        extent_k = __builtin_fmaxf(extent_k, hk->hi[ax] - hk->lo[ax]);
+    }
+    const bool dwarfed = ntiles >= 16 && extent_k < 0.25f * extent_q;
+    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f) || dwarfed) {  // uniform
         if (lane == 0)
             atomicOr(flag, 1);
         return;
