@@ -241,3 +241,30 @@ def test_captured_in_a_hip_graph_and_replayed(cuda):
         want = oracle.chamfer_forward(a.numpy(), c.numpy())
         for name, got, exp in zip(("dist1", "idx1", "dist2", "idx2"), out, want):
             np.testing.assert_array_equal(got.cpu().numpy(), exp, err_msg="%s seed %d" % (name, seed))
+
+
+def test_stray_points_stay_on_the_sorted_path(cuda):
+    # a few points far outside the cloud would blow up its bounding box, and with it the
+    # cells of the sort and the scale of the fp16 terms: the frame is trimmed instead and
+    # the strays are compared with every query directly
+    g = gen(21)
+    a, c = sphere_cloud(g, 3, 5000), sphere_cloud(g, 3, 6000)
+    c[0, 17] = torch.tensor([300.0, -2.0, 5.0])            # one stray key
+    c[1, ::1000] = c[1, ::1000] * 50.0 + 40.0              # six of them
+    c[1, 4000] = c[1, 3000]                                # two strays at one position: the lower index wins
+    a[2, 123] = torch.tensor([-80.0, 90.0, 10.0])          # a stray query
+    a[2, 124] = c[2, 5999] = torch.tensor([25.0, 25.0, 25.0])  # a stray query on a stray key
+    ws = check_sorted(a, c, cuda)
+    assert sum(handed_over(ws, 3)) == 0
+    far_keys = ws[: 2 * 3 * 64].view(torch.int32).view(2, 3, 16)[:, :, 13].cpu().tolist()
+    assert far_keys[1][0] == 1 and far_keys[1][1] == 6 and far_keys[1][2] == 1 and far_keys[0][2] == 2
+    # more strays than the list holds: the cloud is handed over
+    c2 = sphere_cloud(g, 1, 6000)
+    c2[0, ::60] = c2[0, ::60] * 100.0
+    ws = check_sorted(sphere_cloud(g, 1, 5000), c2, cuda)
+    assert handed_over(ws, 1)[0] == 1
+    # strays that are the nearest keys of far queries, and a far cloud of queries
+    a3, c3 = sphere_cloud(g, 2, 4000), sphere_cloud(g, 2, 4000)
+    c3[:, 5] = torch.tensor([60.0, 0.0, 0.0])
+    a3[:, 100:140] = a3[:, 100:140] + torch.tensor([59.0, 0.0, 0.0])
+    check_sorted(a3, c3, cuda)

@@ -1820,13 +1820,17 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // scans would take long (heavy ties on many swept tiles) raise a flag for their cloud and
 // direction; the
 // matrix pre-filter runs behind this one and serves exactly the flagged ones.
+constexpr int CHAMFER_FAR_KEYS = 64;  // keys far outside the frame that a cloud may have
+
 struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
-    float c[3];            // centre of the bounding box
-    float scale;           // 2^-(exponent of the largest half extent)
-    int kmax2_bits;        // largest |k'|^2 (bit pattern of the float)
+    float c[3];            // centre of the frame (the trimmed bounding box)
+    float scale;           // 2^-(exponent of the frame's largest half extent)
+    int kmax2_bits;        // largest |k'|^2 of the keys inside 4 units (bit pattern)
     int unsafe;            // the bound does not cover this cloud
-    float lo[3], hi[3];    // bounding box, caller's units
-    int pad[4];
+    float lo[3], hi[3];    // bounding box of all points, caller's units
+    float extent;          // largest extent of the frame, caller's units
+    int far_keys;          // keys beyond 4 units of the frame, kept on a list of their own
+    int pad[2];
 };
 
 struct ChamferSortArgs {
@@ -1835,6 +1839,7 @@ struct ChamferSortArgs {
     uint4 *terms[2];    // [B, npad / 32][2][32]
     uint4 *boxes[2];    // [B, npad / 32]: lo and hi corner in centred, scaled coordinates,
                         // six fp16 values rounded outwards
+    float4 *far_keys[2];  // [B, CHAMFER_FAR_KEYS]: x, y, z, original index
     ChamferSortedHdr *hdr;  // [2, B]
     int *flags;             // [2, B]
     int n[2], npad[2];
@@ -1895,6 +1900,7 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
 {
     constexpr int NT = 1024, NW = NT / TK_WAVE, U = 16, PARTS = CHAMFER_CELL_PARTS;
     __shared__ float sred[NW][8];
+    __shared__ float sdev[NW][4];
     __shared__ int sbad;
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
     const int cloud = (int)blockIdx.x / PARTS, part = (int)blockIdx.x - cloud * PARTS;
@@ -1907,7 +1913,11 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
     const float INF = __builtin_huge_valf();
 
+    // A pilot centre that a few stray points cannot move: per axis the median of three
+    // medians of three, over nine points spread through the cloud.
+    float pilot[3] = {0.0f, 0.0f, 0.0f};
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    float dev[3] = {0.0f, 0.0f, 0.0f};  // sum of |x - pilot|
     bool bad = false;
     for (int base = 0; base < n; base += NT * U) {
         TkPoint3<float> p[U];
@@ -1916,14 +1926,31 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
             const int j = base + u * NT + tid;
             p[u] = tk_load3<float>(P + (int64_t)(j < n ? j : n - 1) * 3);
         }
+        if (base == 0) {  // (requested together with the first points: one round trip)
+            TkPoint3<float> q[9];
+#pragma unroll
+            for (int i = 0; i < 9; ++i)
+                q[i] = tk_load3<float>(P + (((int64_t)n * (2 * i + 1)) / 19) * 3);
+            auto ninther = [](float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                              float v7, float v8) {
+                return __builtin_amdgcn_fmed3f(__builtin_amdgcn_fmed3f(v0, v1, v2),
+                                               __builtin_amdgcn_fmed3f(v3, v4, v5),
+                                               __builtin_amdgcn_fmed3f(v6, v7, v8));
+            };
+            pilot[0] = ninther(q[0].x, q[1].x, q[2].x, q[3].x, q[4].x, q[5].x, q[6].x, q[7].x, q[8].x);
+            pilot[1] = ninther(q[0].y, q[1].y, q[2].y, q[3].y, q[4].y, q[5].y, q[6].y, q[7].y, q[8].y);
+            pilot[2] = ninther(q[0].z, q[1].z, q[2].z, q[3].z, q[4].z, q[5].z, q[6].z, q[7].z, q[8].z);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const float v[3] = {p[u].x, p[u].y, p[u].z};
+            const bool counts = base + u * NT + tid < n;
 #pragma unroll
             for (int ax = 0; ax < 3; ++ax) {
                 bad |= !(v[ax] - v[ax] == 0.0f);
                 lo[ax] = __builtin_fminf(lo[ax], v[ax]);
                 hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
+                dev[ax] += counts ? __builtin_fabsf(v[ax] - pilot[ax]) : 0.0f;
             }
         }
     }
@@ -1931,6 +1958,9 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     for (int ax = 0; ax < 3; ++ax) {
         lo[ax] = wave_reduce_min(lo[ax]);
         hi[ax] = wave_reduce_max(hi[ax]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            dev[ax] += __shfl_xor(dev[ax], o);
     }
     if (tid == 0)
         sbad = 0;
@@ -1940,24 +1970,34 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
         for (int ax = 0; ax < 3; ++ax) {
             sred[wave][ax] = lo[ax];
             sred[wave][3 + ax] = hi[ax];
+            sdev[wave][ax] = dev[ax];
         }
     }
     if (bad)
         sbad = 1;
     __syncthreads();
-    float cc[3], ext = 0.0f;
+    // The frame: the bounding box, trimmed to six mean deviations around the pilot centre.
+    // A cloud without stray points keeps its bounding box (six mean deviations reach
+    // beyond it from wherever the pilot lies); a few points far away no longer decide
+    // the cells and the scale of everything else - they go on a list of their own.
+    float cc[3], ext = 0.0f, flo[3];
 #pragma unroll
     for (int ax = 0; ax < 3; ++ax) {
-        float l = sred[0][ax], h = sred[0][3 + ax];
+        float l = sred[0][ax], h = sred[0][3 + ax], dsum = sdev[0][ax];
 #pragma unroll
         for (int w = 1; w < NW; ++w) {
             l = __builtin_fminf(l, sred[w][ax]);
             h = __builtin_fmaxf(h, sred[w][3 + ax]);
+            dsum += sdev[w][ax];
         }
         lo[ax] = l;
         hi[ax] = h;
-        cc[ax] = 0.5f * l + 0.5f * h;
-        ext = __builtin_fmaxf(ext, 0.5f * h - 0.5f * l);
+        const float reach = 6.0f * (dsum / (float)n);
+        const float fl = __builtin_fmaxf(l, pilot[ax] - reach);
+        const float fh = __builtin_fminf(h, pilot[ax] + reach);
+        flo[ax] = fl;
+        cc[ax] = 0.5f * fl + 0.5f * fh;
+        ext = __builtin_fmaxf(ext, 0.5f * fh - 0.5f * fl);
     }
     const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
     const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
@@ -1973,6 +2013,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
             ext == 0.0f ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
         hdr->kmax2_bits = 0;
         hdr->unsafe = safe ? 0 : 1;
+        hdr->extent = 2.0f * ext;
+        hdr->far_keys = 0;
 #pragma unroll
         for (int ax = 0; ax < 3; ++ax) {
             hdr->lo[ax] = lo[ax];
@@ -1981,17 +2023,17 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     }
     if (!safe)  // uniform over the workgroup
         return;
-    // cells: 32 per axis over the largest extent (a point on the upper face: cell 31)
+    // cells: 32 per axis over the frame's largest extent (a point on the upper face, or
+    // beyond the frame: the outermost cell)
     const float inv = ext > 0.0f ? (16.0f / ext) * 0.99999f : 0.0f;
     const int share = (n + PARTS - 1) / PARTS;
     const int first = part * share, last = first + share < n ? first + share : n;
     for (int j = first + tid; j < last; j += NT) {
         const TkPoint3<float> p = tk_load3<float>(P + (int64_t)j * 3);
-        int ix = (int)((p.x - lo[0]) * inv), iy = (int)((p.y - lo[1]) * inv);
-        int iz = (int)((p.z - lo[2]) * inv);
-        ix = ix > 31 ? 31 : ix;
-        iy = iy > 31 ? 31 : iy;
-        iz = iz > 31 ? 31 : iz;
+        const float ux = __builtin_fminf(__builtin_fmaxf((p.x - flo[0]) * inv, 0.0f), 31.0f);
+        const float uy = __builtin_fminf(__builtin_fmaxf((p.y - flo[1]) * inv, 0.0f), 31.0f);
+        const float uz = __builtin_fminf(__builtin_fmaxf((p.z - flo[2]) * inv, 0.0f), 31.0f);
+        const int ix = (int)ux, iy = (int)uy, iz = (int)uz;
         cells[j] = (unsigned short)chamfer_hilbert15((unsigned)ix, (unsigned)iy, (unsigned)iz);
     }
 }
@@ -2128,14 +2170,24 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
     const float y = ((exists ? s.y : c1) - c1) * scale;
     const float z = ((exists ? s.z : c2) - c2) * scale;
     const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+    // A key beyond 4 units of the frame (the frame itself reaches 3.5) would widen the
+    // error bound of every pair through max|k'|: the sweep sees it as padding, and every
+    // wave compares its queries with the few such keys directly.
+    const bool far = exists && !(nn <= 16.0f);
+    if (far) {
+        const int slot = atomicAdd(&hdr->far_keys, 1);
+        if (slot < CHAMFER_FAR_KEYS)
+            a.far_keys[which][(int64_t)b * CHAMFER_FAR_KEYS + slot] = s;
+    }
+    const bool swept = exists && !far;
     uint4 h0, h1;
-    chamfer_key_terms(x, y, z, nn, exists, h0, h1);
+    chamfer_key_terms(x, y, z, nn, swept, h0, h1);
     uint4 *tile = terms + (i >> 5) * 64 + (i & 31);
     tile[0] = h0;
     tile[32] = h1;
-    float bl[3] = {exists ? x : INF, exists ? y : INF, exists ? z : INF};
-    float bh[3] = {exists ? x : -INF, exists ? y : -INF, exists ? z : -INF};
-    float kmax2 = nn;  // (0 for padding)
+    float bl[3] = {swept ? x : INF, swept ? y : INF, swept ? z : INF};
+    float bh[3] = {swept ? x : -INF, swept ? y : -INF, swept ? z : -INF};
+    float kmax2 = swept ? nn : 0.0f;
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) {
 #pragma unroll
@@ -2166,6 +2218,7 @@ struct ChamferPrunedArgs {
     const float4 *sorted[2];
     const uint4 *terms[2];
     const uint4 *boxes[2];
+    const float4 *far_keys[2];
     const ChamferSortedHdr *hdr;
     int *flags;
     float *dist[2];
@@ -2216,6 +2269,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
     const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
     const uint4 *__restrict__ BX = a.boxes[1 - which] + (int64_t)b * (npk / 32);
+    const float4 *__restrict__ FK = a.far_keys[1 - which] + (int64_t)b * CHAMFER_FAR_KEYS;
     const int ntiles = npk / 32;
     const int rounds = (ntiles + TK_WAVE - 1) / TK_WAVE;  // <= RMAX
     // The wave's queries and the first boxes are requested before anything is known about
@@ -2245,17 +2299,13 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             far2 = __builtin_fmaf(m, m, far2);
         }
     }
-    // A key cloud much smaller than the query cloud: most queries are far from it compared
-    // with its size, every one of its tiles is within their reach, and this kernel would
-    // sweep all pairs at four times the matrix kernel's cost per tile.
-    float extent_q = 0.0f, extent_k = 0.0f;
-#pragma unroll
-    for (int ax = 0; ax < 3; ++ax) {
-        extent_q = __builtin_fmaxf(extent_q, hq->hi[ax] - hq->lo[ax]);
-        extent_k = __builtin_fmaxf(extent_k, hk->hi[ax] - hk->lo[ax]);
-    }
-    const bool dwarfed = ntiles >= 16 && extent_k < 0.25f * extent_q;
-    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f) || dwarfed) {  // uniform
+    // A key cloud much smaller than the query cloud (by their frames): most queries are far
+    // from it compared with its size, every one of its tiles is within their reach, and
+    // this kernel would sweep all pairs at four times the matrix kernel's cost per tile.
+    const bool dwarfed = ntiles >= 16 && hk->extent < 0.25f * hq->extent;
+    const int nfar = hk->far_keys;  // keys kept out of the sweep (far outside the frame)
+    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f) || dwarfed ||
+        nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
         if (lane == 0)
             atomicOr(flag, 1);
         return;
@@ -2491,6 +2541,15 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             bestd = od;
             bestj = oj;
         }
+        for (int e = 0; e < nfar; ++e) {  // (uniform; usually none)
+            const float4 f = FK[e];
+            const float dd = tk_dist2<float>(f.x, f.y, f.z, rx[g], ry[g], rz[g]);
+            const int fj = __builtin_bit_cast(int, f.w);
+            if (dd < bestd || (dd == bestd && fj < bestj)) {
+                bestd = dd;
+                bestj = fj;
+            }
+        }
         if (half == 0 && ok && !over) {
             const int64_t o = (int64_t)b * nq + qid[g];
             a.dist[which][o] = bestd;
@@ -2550,6 +2609,15 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
                     }
                 }
             }
+            if (lane < nfar) {  // the keys kept out of the sweep, one per lane
+                const float4 f = FK[lane];
+                const float dd = tk_dist2<float>(f.x, f.y, f.z, qx, qy, qz);
+                const int fj = __builtin_bit_cast(int, f.w);
+                if (dd < bestd || (dd == bestd && fj < bestj)) {
+                    bestd = dd;
+                    bestj = fj;
+                }
+            }
             const float least = wave_reduce_min(bestd);
             const int cand = (bestd == least && bestj >= 0) ? bestj : 0x7fffffff;
             const int first = wave_reduce_min_int(cand);
@@ -2586,7 +2654,7 @@ inline bool chamfer_sorted_serves(int64_t B, int64_t N1, int64_t N2)
 }
 
 struct ChamferSortedLayout {
-    size_t hdr, flags, sorted[2], terms[2], boxes[2], total;
+    size_t hdr, flags, sorted[2], terms[2], boxes[2], far_keys[2], total;
     int64_t npad[2];
 };
 
@@ -2607,6 +2675,7 @@ inline ChamferSortedLayout chamfer_sorted_layout(int64_t B, int64_t N1, int64_t 
         l.sorted[w] = take((size_t)B * l.npad[w] * sizeof(float4));
         l.terms[w] = take((size_t)B * l.npad[w] * 2 * sizeof(uint4));
         l.boxes[w] = take((size_t)B * (l.npad[w] / 32) * sizeof(uint4));
+        l.far_keys[w] = take((size_t)B * CHAMFER_FAR_KEYS * sizeof(float4));
     }
     l.total = at;
     return l;
@@ -2628,11 +2697,13 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
         sa.sorted[w] = reinterpret_cast<float4 *>(ws + l.sorted[w]);
         sa.terms[w] = reinterpret_cast<uint4 *>(ws + l.terms[w]);
         sa.boxes[w] = reinterpret_cast<uint4 *>(ws + l.boxes[w]);
+        sa.far_keys[w] = reinterpret_cast<float4 *>(ws + l.far_keys[w]);
         sa.n[w] = (int)n[w];
         sa.npad[w] = (int)l.npad[w];
         pa.sorted[w] = sa.sorted[w];
         pa.terms[w] = sa.terms[w];
         pa.boxes[w] = sa.boxes[w];
+        pa.far_keys[w] = sa.far_keys[w];
         pa.n[w] = sa.n[w];
         pa.npad[w] = sa.npad[w];
         pa.waves_per_cloud[w] = (int)((l.npad[w] + 32 * NQB - 1) / (32 * NQB));
