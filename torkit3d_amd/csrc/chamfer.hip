@@ -1785,17 +1785,22 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // nearest neighbours, and once both clouds are ordered along a space-filling curve that
 // can be decided for 32 keys and a wave's queries at a time:
 //
-//   chamfer_sort_kernel (one workgroup per cloud): bounding box, centre and scale as in
-//     the matrix pre-filter, a counting sort of the points by the 15-bit Morton code of
-//     their cell in a 32^3 grid over the box, then, per tile of 32 sorted points, the 16
-//     fp16 terms of every key (the layout the matrix kernel stages in LDS) and the tile's
-//     bounding box in centred, scaled coordinates. The sorted points carry their original
-//     index.
+//   chamfer_cell_kernel (four workgroups per cloud): the cloud's frame - its bounding box,
+//     trimmed so that a few points far from the rest do not decide it - with centre and
+//     power-of-two scale as in the matrix pre-filter, and every point's cell in a 32^3
+//     grid over the frame, numbered along the Hilbert curve.
+//   chamfer_sort_kernel (one workgroup per cloud): counting sort of the points by cell.
+//     The sorted points carry their original index.
+//   chamfer_tile_kernel (one lane per point): per tile of 32 sorted points the 16 fp16
+//     terms of every key (the layout the matrix kernel stages in LDS) and the tile's
+//     bounding box in centred, scaled coordinates; keys far outside the frame go on a
+//     short list instead.
 //   chamfer_pruned_kernel (waves work alone, no LDS): a wave takes NQB x 32 consecutive
 //     sorted queries - a compact patch - and sweeps a key tile only if the squared gap
 //     between the patch's box and the tile's box does not exceed T, an upper bound of
 //     every query's distance to the nearest key met so far: first the tiles that overlap
-//     the patch, then in passes at T/16, T/4 and T with T taken anew each time. The
+//     the patch, then (if those were few) the tiles within T/4, then those within T,
+//     with T taken anew each time. The
 //     sweep, the three smallest tile minima per lane and the exact re-evaluation of the
 //     candidate tiles are those of the matrix kernel; ties between equal distances go to
 //     the lower original index, compared explicitly because sorted order is not index
@@ -1818,8 +1823,8 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // further than 8000 extents from the key cloud), a key cloud under a quarter of the query
 // cloud's extent (boxes cannot prune for queries far from all keys) and waves whose exact
 // scans would take long (heavy ties on many swept tiles) raise a flag for their cloud and
-// direction; the
-// matrix pre-filter runs behind this one and serves exactly the flagged ones.
+// direction; the matrix pre-filter runs behind this one and serves exactly the flagged
+// ones.
 constexpr int CHAMFER_FAR_KEYS = 64;  // keys far outside the frame that a cloud may have
 
 struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
