@@ -1981,10 +1981,12 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     if (bad)
         sbad = 1;
     __syncthreads();
-    // The frame: the bounding box, trimmed to six mean deviations around the pilot centre.
-    // A cloud without stray points keeps its bounding box (six mean deviations reach
-    // beyond it from wherever the pilot lies); a few points far away no longer decide
-    // the cells and the scale of everything else - they go on a list of their own.
+    // The frame: the bounding box, trimmed to three mean deviations around the pilot centre.
+    // A uniform or a Gaussian cloud keeps (nearly) its bounding box - three mean deviations
+    // are 1.5 half extents of the first and 2.4 sigma of the second, and keys up to twice
+    // as far out as the frame are still swept like any other; a few points far away no
+    // longer decide the cells and the scale of everything else - they go on a list of
+    // their own.
     float cc[3], ext = 0.0f, flo[3];
 #pragma unroll
     for (int ax = 0; ax < 3; ++ax) {
@@ -1997,7 +1999,7 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
         }
         lo[ax] = l;
         hi[ax] = h;
-        const float reach = 6.0f * (dsum / (float)n);
+        const float reach = 3.0f * (dsum / (float)n);
         const float fl = __builtin_fmaxf(l, pilot[ax] - reach);
         const float fh = __builtin_fminf(h, pilot[ax] + reach);
         flo[ax] = fl;
