@@ -48,11 +48,11 @@ MATRIX_FLOP_PER_PAIR = 32         # executed: a 16-term dot product per pair in 
 # FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size: the five launches
 # of the sorted path together, and the single launch of the full sweep
 # (profiles/chamfer_forward_sorted_B32_N16384.md, chamfer_forward_mfma_B32_N16384.md).
-CHAMFER_SORTED_TRAFFIC_BYTES = 265.6e6
+CHAMFER_SORTED_TRAFFIC_BYTES = 261.3e6
 CHAMFER_TRAFFIC_BYTES = 46.7e6
 # Share of the 2*B*N*M pairs whose score the sorted path evaluates on these clouds
 # (matrix instructions counted by SQ_INSTS_MFMA x 1024 pairs each, same profile).
-CHAMFER_SORTED_PAIRS_EVALUATED = 0.035
+CHAMFER_SORTED_PAIRS_EVALUATED = 0.0356
 
 
 def sphere_cloud(gen, b, n, noise=0.01):
