@@ -110,3 +110,35 @@ def test_fps_workspace_size(lib):
     assert fn(i64(8), i64(16384), ctypes.c_size_t(4)) == 0
     need = fn(i64(2), i64(100000), ctypes.c_size_t(4))
     assert need >= 2 * 100000 * 4
+
+
+def test_chamfer_workspace_size_and_argument_checks(lib):
+    # the size function is host code: the dispatch rule of the sorted path, no GPU needed
+    size = lib.tk3d_chamfer_distance_forward_workspace_bytes
+    size.restype = ctypes.c_size_t
+
+    def nbytes(b, n1, n2, always):
+        return size(i64(b), i64(n1), i64(n2), ctypes.c_int(always))
+
+    assert nbytes(32, 16384, 16384, 0) > 0          # the benchmark shape is served
+    assert nbytes(1, 65536, 65536, 0) > 0
+    assert nbytes(2, 1024, 1024, 0) == 0            # too little work to repay the sort
+    assert nbytes(16, 4096, 4096, 0) == 0
+    assert nbytes(4, 65536, 2048, 0) == 0           # lengths more than a factor of four apart
+    assert nbytes(64, 3000, 3000, 0) == 0           # clouds under 4096 points
+    for shape in ((2, 1024, 1024), (16, 4096, 4096), (4, 65536, 2048), (1, 1, 1)):
+        assert nbytes(*shape, 1) > 0                # ... but can be, on request
+    assert nbytes(1, 65537, 4096, 1) == 0 and nbytes(0, 4096, 4096, 1) == 0
+    # 16 + 32 bytes per padded point, a box per 32 points, headers, flags and far-key lists
+    b, n = 3, 5000
+    pad = (n + 127) // 128 * 128
+    low = 2 * b * pad * 48
+    assert low < nbytes(b, n, n, 1) < low + 2 * b * (pad // 2 + 1024) + 4096
+    # null or short workspace: the call is the plain entry point, with its argument checks
+    fn = lib.tk3d_chamfer_distance_forward_ws_f32
+    args = (FAKE, FAKE, i64(1), i64(8), i64(8), FAKE, FAKE, FAKE)
+    assert fn(*args, NULL, NULL, ctypes.c_size_t(0), NULL) == -1          # idx2 missing
+    assert fn(FAKE, FAKE, i64(-1), i64(8), i64(8), FAKE, FAKE, FAKE, FAKE, NULL,
+              ctypes.c_size_t(0), NULL) == -2
+    assert fn(NULL, NULL, i64(0), i64(8), i64(8), NULL, NULL, NULL, NULL, NULL,
+              ctypes.c_size_t(0), NULL) == 0
