@@ -268,3 +268,25 @@ def test_stray_points_stay_on_the_sorted_path(cuda):
     c3[:, 5] = torch.tensor([60.0, 0.0, 0.0])
     a3[:, 100:140] = a3[:, 100:140] + torch.tensor([59.0, 0.0, 0.0])
     check_sorted(a3, c3, cuda)
+
+
+def test_stray_queries_beyond_the_reach_of_the_fp16_terms(cuda):
+    # a few queries more than 8000 key extents away are scanned exactly against all keys;
+    # the cloud stays on the sorted path in both directions (as keys they are far keys)
+    g = gen(22)
+    a, c = sphere_cloud(g, 2, 5000), sphere_cloud(g, 2, 4500)
+    a[0, 11] = torch.tensor([3.0e4, 0.0, 0.0])
+    a[1, 4000] = torch.tensor([-1.0e5, 2.0e5, 7.0e4])
+    a[1, 4999] = torch.tensor([5.0e5, 5.0e5, 5.0e5])
+    ws = check_sorted(a, c, cuda)
+    assert sum(handed_over(ws, 2)) == 0
+    # a wave of nothing but stray queries and padding: 4480 + 30 queries, the last 30 far away
+    a2 = sphere_cloud(g, 1, 4510)
+    a2[0, 4480:] = a2[0, 4480:] * 10.0 + 4.0e4
+    ws = check_sorted(a2, sphere_cloud(g, 1, 4500), cuda)
+    assert sum(handed_over(ws, 1)) == 0
+    # too many of them for exact scans: handed over
+    a3 = sphere_cloud(g, 1, 5000)
+    a3[0, ::3] = a3[0, ::3] + 5.0e4
+    ws = check_sorted(a3, sphere_cloud(g, 1, 4500), cuda)
+    assert handed_over(ws, 1)[0] == 1

@@ -1008,7 +1008,9 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
 #pragma unroll
     for (int w = 0; w < NW; ++w)
         kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
-    if (!(kmax2 <= 32768.0f)) {  // uniform over the workgroup (also +inf)
+    // (also +inf; and a sample of identical keys, scale 1, beside keys that differ from it
+    // by far less than 1: the fp16 terms have no precision for those)
+    if (!(kmax2 <= 32768.0f) || (ext == 0.0f && kmax2 > 0.0f && kmax2 < 0.25f)) {  // uniform
         chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
@@ -1819,8 +1821,9 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 // query than a key already met: it can neither be the minimum nor tie with it. T only
 // shrinks as tiles are swept, so a tile skipped under an earlier T stays skipped rightly.
 //
-// Input the bound does not cover (non-finite coordinates, extents outside 2^+-40, queries
-// further than 8000 extents from the key cloud), a key cloud under a quarter of the query
+// Input the bound does not cover (non-finite coordinates, extents outside 2^+-40, a query
+// cloud whose frame reaches further than 8000 extents from the key cloud or holds many
+// stray queries that far out), a key cloud under a quarter of the query
 // cloud's extent (boxes cannot prune for queries far from all keys) and waves whose exact
 // scans would take long (heavy ties on many swept tiles) raise a flag for their cloud and
 // direction; the matrix pre-filter runs behind this one and serves exactly the flagged
@@ -1921,6 +1924,7 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     // A pilot centre that a few stray points cannot move: per axis the median of three
     // medians of three, over nine points spread through the cloud.
     float pilot[3] = {0.0f, 0.0f, 0.0f};
+    float cap[3] = {INF, INF, INF};  // a deviation counts up to 16 typical ones
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
     float dev[3] = {0.0f, 0.0f, 0.0f};  // sum of |x - pilot|
     bool bad = false;
@@ -1945,6 +1949,20 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
             pilot[0] = ninther(q[0].x, q[1].x, q[2].x, q[3].x, q[4].x, q[5].x, q[6].x, q[7].x, q[8].x);
             pilot[1] = ninther(q[0].y, q[1].y, q[2].y, q[3].y, q[4].y, q[5].y, q[6].y, q[7].y, q[8].y);
             pilot[2] = ninther(q[0].z, q[1].z, q[2].z, q[3].z, q[4].z, q[5].z, q[6].z, q[7].z, q[8].z);
+            // the typical deviation of the nine, the same way; none (the nine coincide): no cap
+            float d[9][3];
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+                d[i][0] = __builtin_fabsf(q[i].x - pilot[0]);
+                d[i][1] = __builtin_fabsf(q[i].y - pilot[1]);
+                d[i][2] = __builtin_fabsf(q[i].z - pilot[2]);
+            }
+#pragma unroll
+            for (int ax = 0; ax < 3; ++ax) {
+                const float typical = ninther(d[0][ax], d[1][ax], d[2][ax], d[3][ax], d[4][ax],
+                                              d[5][ax], d[6][ax], d[7][ax], d[8][ax]);
+                cap[ax] = typical > 0.0f ? 16.0f * typical : INF;
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -1955,7 +1973,7 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
                 bad |= !(v[ax] - v[ax] == 0.0f);
                 lo[ax] = __builtin_fminf(lo[ax], v[ax]);
                 hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
-                dev[ax] += counts ? __builtin_fabsf(v[ax] - pilot[ax]) : 0.0f;
+                dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
             }
         }
     }
@@ -2005,6 +2023,17 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
         flo[ax] = fl;
         cc[ax] = 0.5f * fl + 0.5f * fh;
         ext = __builtin_fmaxf(ext, 0.5f * fh - 0.5f * fl);
+    }
+    if (ext == 0.0f) {
+        // Nearly all points in one place: a frame of no extent would leave the others at
+        // scale 1, possibly far below it, where the fp16 terms have no precision left
+        // (the error bound counts on max|k'| of order 1). The bounding box, then.
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            flo[ax] = lo[ax];
+            cc[ax] = 0.5f * lo[ax] + 0.5f * hi[ax];
+            ext = __builtin_fmaxf(ext, 0.5f * hi[ax] - 0.5f * lo[ax]);
+        }
     }
     const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
     const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
@@ -2295,14 +2324,15 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const int handed_over = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_sched_barrier(0);
     const float c0 = hk->c[0], c1 = hk->c[1], c2 = hk->c[2], scale = hk->scale;
-    // the query cloud's farthest corner from the key cloud's centre, in key extents
+    // the farthest corner of the query cloud's frame from the key cloud's centre, in key
+    // extents (stray queries beyond the frame are looked at one by one below)
     float far2 = 0.0f;
     {
         const float cc[3] = {c0, c1, c2};
 #pragma unroll
         for (int ax = 0; ax < 3; ++ax) {
-            const float m = __builtin_fmaxf(__builtin_fabsf(hq->lo[ax] - cc[ax]),
-                                            __builtin_fabsf(hq->hi[ax] - cc[ax])) * scale;
+            const float m =
+                (__builtin_fabsf(hq->c[ax] - cc[ax]) + 0.5f * hq->extent) * scale;
             far2 = __builtin_fmaf(m, m, far2);
         }
     }
@@ -2327,10 +2357,14 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     tk_f16x8 qterm[NQB];
     float qnorm[NQB], qn2[NQB], rx[NQB], ry[NQB], rz[NQB];
     int qid[NQB];
+    // live: a query the sweep serves; stray: a query too far from the key cloud for the
+    // fp16 terms (beyond 8000 key extents), served by an exact scan of all keys instead
+    bool live[NQB], stray[NQB];
     float v0[NQB], v1[NQB], v2[NQB];
     int id0[NQB], id1[NQB];
     float blo[3] = {INF, INF, INF}, bhi[3] = {-INF, -INF, -INF};
     float qnmax = 0.0f;
+    int nstray = 0;
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
         const float4 s = squery[g];
@@ -2339,15 +2373,22 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         rx[g] = s.x;
         ry[g] = s.y;
         rz[g] = s.z;
-        const float px = ((ok ? s.x : c0) - c0) * scale;
-        const float py = ((ok ? s.y : c1) - c1) * scale;
-        const float pz = ((ok ? s.z : c2) - c2) * scale;
+        float px = ((ok ? s.x : c0) - c0) * scale;
+        float py = ((ok ? s.y : c1) - c1) * scale;
+        float pz = ((ok ? s.z : c2) - c2) * scale;
+        const bool near = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px)) <= 6.4e7f;
+        live[g] = ok && near;
+        stray[g] = ok && !near;
+        nstray += __builtin_popcountll(__builtin_amdgcn_ballot_w64(stray[g] && half == 0));
+        px = near ? px : 0.0f;
+        py = near ? py : 0.0f;
+        pz = near ? pz : 0.0f;
         qn2[g] = __builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px));
         qnorm[g] = 1.000001f * __builtin_sqrtf(qn2[g]);
         qterm[g] = __builtin_bit_cast(tk_f16x8, chamfer_query_terms(px, py, pz, half));
         v0[g] = v1[g] = v2[g] = INF;
         id0[g] = id1[g] = -1;
-        if (ok) {
+        if (live[g]) {
             blo[0] = __builtin_fminf(blo[0], px);
             blo[1] = __builtin_fminf(blo[1], py);
             blo[2] = __builtin_fminf(blo[2], pz);
@@ -2362,8 +2403,16 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         blo[ax] = wave_reduce_min(blo[ax]);
         bhi[ax] = wave_reduce_max(bhi[ax]);
     }
-    if (!(blo[0] <= bhi[0]))  // a wave of padding only (uniform over the wave)
+    const bool nothing_to_sweep = !(blo[0] <= bhi[0]);  // padding and strays only (uniform)
+    if (nothing_to_sweep && nstray == 0)
         return;
+    // An exact scan of all keys costs what scanning every tile costs: more than 16384
+    // (query, tile) pairs of it per wave and the cloud is handed over.
+    if ((int64_t)nstray * ntiles > 16384) {
+        if (lane == 0)
+            atomicOr(flag, 1);
+        return;
+    }
 #pragma unroll
     for (int ax = 0; ax < 3; ++ax) {  // (the same in every lane: scalar registers)
         blo[ax] = __builtin_bit_cast(
@@ -2430,7 +2479,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
 #pragma unroll
         for (int g = 0; g < NQB; ++g) {
             const float best = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
-            ub = qid[g] >= 0 ? __builtin_fmaxf(ub, best + qn2[g]) : ub;
+            ub = live[g] ? __builtin_fmaxf(ub, best + qn2[g]) : ub;
         }
         return wave_reduce_max(ub);
     };
@@ -2438,7 +2487,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // any, the nearest tile -, then everything within reach at T. When the first pass met
     // fewer than four tiles T is still loose, and a pass at T/4 tightens it first.
 #pragma unroll 1
-    for (int phase = 0; phase < 3; ++phase) {
+    for (int phase = 0; phase < (nothing_to_sweep ? 0 : 3); ++phase) {
         float thr = 0.0f;
         if (phase == 1 && nswept >= 4)  // uniform over the wave
             continue;
@@ -2504,11 +2553,12 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     }
 
     // ---- exact evaluation of each half's candidate tiles, then the merge ----
-    unsigned over_mask[NQB];
+    unsigned over_mask[NQB], stray_mask[NQB];
     int nover = 0;
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
-        const bool ok = qid[g] >= 0;
+        const bool ok = live[g];
+        stray_mask[g] = (unsigned)__builtin_amdgcn_ballot_w64(stray[g] && half == 0);
         const float best_score = __builtin_fminf(v0[g], __shfl_xor(v0[g], 32));
         const float r = kmax + qnorm[g];
         const float thr = best_score + (r * r * 7.6293945e-06f + guard);  // 2^-17 R
@@ -2565,7 +2615,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         over_mask[g] = (unsigned)__builtin_amdgcn_ballot_w64(over && half == 0);
         nover += __builtin_popcount(over_mask[g]);
     }
-    if (nover == 0)
+    if (nover == 0 && nstray == 0)
         return;
     // An exact scan costs about 13 instructions per two swept tiles (a normal wave issues
     // 2100 in all): beyond 8192 (query, tile) pairs - half of what sweeping the whole cloud
@@ -2576,13 +2626,15 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             atomicOr(flag, 1);
         return;
     }
-    // ---- queries with three or more candidate tiles: exact scan of the swept tiles ----
+    // ---- queries with three or more candidate tiles: exact scan of the swept tiles;
+    //      stray queries: exact scan of all tiles ----
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
-        unsigned m = over_mask[g];
+        unsigned m = over_mask[g] | stray_mask[g];
         while (m != 0) {
             const int src = __builtin_ctz(m);
             m &= m - 1;
+            const bool all_tiles = ((stray_mask[g] >> src) & 1u) != 0;  // uniform
             const float qx = __builtin_bit_cast(
                 float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rx[g]), src));
             const float qy = __builtin_bit_cast(
@@ -2595,7 +2647,8 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             // two swept tiles at a time, lane l taking key l % 32 of the tile of its half
 #pragma unroll 1
             for (int r = 0; r < rounds; ++r) {
-                unsigned long long mm = __builtin_amdgcn_ballot_w64(((swept >> r) & 1u) != 0);
+                unsigned long long mm = __builtin_amdgcn_ballot_w64(
+                    all_tiles ? r * TK_WAVE + lane < ntiles : ((swept >> r) & 1u) != 0);
                 while (mm != 0) {
                     const int t0 = r * TK_WAVE + (int)__builtin_ctzll(mm);
                     mm &= mm - 1;
