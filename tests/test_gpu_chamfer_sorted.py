@@ -67,7 +67,8 @@ def check_sorted(a, c, cuda, **kw):
 
 @pytest.mark.parametrize("b,n1,n2", [(2, 4096, 4096), (3, 2043, 1999), (1, 1, 1), (2, 5, 700),
                                      (2, 5000, 33), (4, 255, 257), (1, 127, 129), (2, 8193, 3001),
-                                     (1, 16384, 16385), (1, 20000, 40000), (1, 65536, 4100)])
+                                     (1, 16384, 16385), (1, 20000, 40000), (1, 65536, 4100),
+                                     (300, 700, 900), (2, 60000, 16385)])
 def test_shapes_on_uniform_and_sphere_clouds(cuda, b, n1, n2):
     # lengths that are no multiple of a tile (32), of the padding (128) or of a wave's
     # queries (64), one-point clouds, and both register layouts of the tile gaps (up to
