@@ -291,3 +291,17 @@ def test_stray_queries_beyond_the_reach_of_the_fp16_terms(cuda):
     a3[0, ::3] = a3[0, ::3] + 5.0e4
     ws = check_sorted(a3, sphere_cloud(g, 1, 4500), cuda)
     assert handed_over(ws, 1)[0] == 1
+
+
+def test_a_cloud_of_identical_points(cuda):
+    # all keys in one place: the answer is key 0 for every query, without a sweep; the
+    # other way round (identical queries) is an ordinary, small patch
+    g = gen(23)
+    a = sphere_cloud(g, 2, 5000)
+    c = torch.tensor([0.3, -0.2, 0.9]).expand(2, 4500, 3).contiguous()
+    ws = check_sorted(a, c, cuda)
+    assert sum(handed_over(ws, 2)) == 0
+    ws = check_sorted(c, c.clone(), cuda)
+    assert sum(handed_over(ws, 2)) == 0
+    far = (c * 3.0e19).contiguous()          # distances overflow: (+inf, -1)
+    check_sorted(-far, far, cuda)

@@ -2341,8 +2341,28 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // this kernel would sweep all pairs at four times the matrix kernel's cost per tile.
     const bool dwarfed = ntiles >= 16 && hk->extent < 0.25f * hq->extent;
     const int nfar = hk->far_keys;  // keys kept out of the sweep (far outside the frame)
-    if (hq->unsafe != 0 || hk->unsafe != 0 || !(far2 <= 6.4e7f) || dwarfed ||
-        nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
+    if (hq->unsafe != 0 || hk->unsafe != 0) {  // uniform over the wave
+        if (lane == 0)
+            atomicOr(flag, 1);
+        return;
+    }
+    if (hk->lo[0] == hk->hi[0] && hk->lo[1] == hk->hi[1] && hk->lo[2] == hk->hi[2]) {
+        // Every key is the same point (uniform over the wave): each query's nearest key is
+        // key 0 at that point - or none, if the distance overflows (strict '<' from +inf).
+#pragma unroll
+        for (int g = 0; g < NQB; ++g) {
+            const int id = __builtin_bit_cast(int, squery[g].w);
+            const float dd = tk_dist2<float>(hk->lo[0], hk->lo[1], hk->lo[2], squery[g].x,
+                                             squery[g].y, squery[g].z);
+            if (half == 0 && id >= 0) {
+                const int64_t o = (int64_t)b * nq + id;
+                a.dist[which][o] = dd < INF ? dd : INF;
+                a.idx[which][o] = dd < INF ? 0 : -1;
+            }
+        }
+        return;
+    }
+    if (!(far2 <= 6.4e7f) || dwarfed || nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
         if (lane == 0)
             atomicOr(flag, 1);
         return;
