@@ -2587,6 +2587,9 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
             ok && ((__builtin_amdgcn_ballot_w64(crowded) >> col & 0x100000001ull) != 0);
         float bestd = INF;
         int bestj = -1;
+        // (distance bits << 32 | original index): distances are non-negative, so the words
+        // order as (distance, index) pairs; a NaN (padding) is above +inf and never taken
+        unsigned long long best = (0x7f800000ull << 32) | 0xffffffffull;
         if (ok && !over) {
             const int ta = v0[g] <= thr ? id0[g] : -1, tb = v1[g] <= thr ? id1[g] : -1;
 #pragma unroll
@@ -2603,13 +2606,16 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const float dd = tk_dist2<float>(f[e].x, f[e].y, f[e].z, rx[g], ry[g], rz[g]);
-                    const int oj = __builtin_bit_cast(int, f[e].w);
-                    if (dd < bestd || (dd == bestd && oj < bestj)) {
-                        bestd = dd;
-                        bestj = oj;
-                    }
+                    const unsigned long long word =
+                        ((unsigned long long)__builtin_bit_cast(unsigned, dd) << 32) |
+                        __builtin_bit_cast(unsigned, f[e].w);
+                    best = word < best ? word : best;
                 }
             }
+            // (a distance that overflowed is no match: strict '<' from +inf)
+            const float d = __builtin_bit_cast(float, (unsigned)(best >> 32));
+            bestd = d < INF ? d : INF;
+            bestj = d < INF ? (int)(unsigned)best : -1;
         }
         // the other half's result: smaller distance, then lower key index
         const float od = __shfl_xor(bestd, 32);
