@@ -2093,6 +2093,7 @@ __global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
     constexpr int NT = 1024, NW = NT / TK_WAVE, CELLS = CHAMFER_SORT_CELLS, U = 16;
     extern __shared__ int hist[];  // CELLS counters
     __shared__ int swave[NW];
+    __shared__ int sstart[NW];
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
     const int which = (int)blockIdx.x >= a.B;
     const int b = (int)blockIdx.x - which * a.B;
@@ -2136,15 +2137,13 @@ __global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
             swave[wave] = carry;
     }
     __syncthreads();
-    int wave_start[NW];
-    {
+    if (tid < NW) {  // the ranges' own starts, looked up by cell >> 11 below
         int run = 0;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            wave_start[w] = run;
+        for (int w = 0; w < tid; ++w)
             run += swave[w];
-        }
+        sstart[tid] = run;
     }
+    __syncthreads();
     for (int base = 0; base < n; base += NT * U) {
         TkPoint3<float> p[U];
         int cell[U];
@@ -2164,10 +2163,7 @@ __global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int j = base + u * NT + tid;
-            int start = 0;
-#pragma unroll
-            for (int w = 0; w < NW; ++w)
-                start = (cell[u] >> 11) == w ? wave_start[w] : start;
+            const int start = sstart[cell[u] >> 11];
             if (j < n)
                 sorted[pos[u] + start] =
                     make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, j));
