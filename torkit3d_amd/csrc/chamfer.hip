@@ -2271,6 +2271,9 @@ __device__ __forceinline__ int wave_reduce_min_int(int v)
     return v;
 }
 
+// (Launched one wave per workgroup - waves share nothing, and a finished wave frees its
+// slot at once: 2-3 % over four waves per workgroup. The bound of 256 lanes only caps the
+// registers at four waves per SIMD.)
 template <int NQB, int RMAX>
 __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a)
 {
@@ -2285,7 +2288,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         if (lb < full)
             lb = (lb & 7) * per + (lb >> 3);
     }
-    int wid = __builtin_amdgcn_readfirstlane(lb * 4 + tid / TK_WAVE);
+    int wid = __builtin_amdgcn_readfirstlane(lb + tid / TK_WAVE);
     const int which = wid >= a.waves0;
     if (which)
         wid -= a.waves0;
@@ -2814,11 +2817,11 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
     const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
     hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s, sa,
                        (int)tb0);
-    const dim3 grid((unsigned)((waves0 + waves1 + 3) / 4));
+    const dim3 grid((unsigned)((waves0 + waves1)));
     if (l.npad[0] <= 16384 && l.npad[1] <= 16384)
-        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 8>), grid, dim3(256), 0, s, pa);
+        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 8>), grid, dim3(64), 0, s, pa);
     else
-        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 32>), grid, dim3(256), 0, s, pa);
+        hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 32>), grid, dim3(64), 0, s, pa);
     const int rc = tk_launch_status();
     if (rc != TK3D_OK)
         return rc;
