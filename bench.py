@@ -11,11 +11,14 @@ value is pair-distances per second, 2*B*N*M / t_step: nearest neighbours resolve
 second, whatever share of the pairs had to be evaluated. The run also reports, on the
 same JSON line:
 
-  roofline      the step against the fp32 vector peak, from the 8 algorithmic FLOP per
-                pair-distance and the duration measured with events on the launching
-                stream; beside it (full_sweep) the same figures for the entry point
-                that evaluates every pair, which is the measure of the sweep kernel
-                itself;
+  roofline      the dominant kernel (the pruned sweep) by the work it executed: matrix
+                instructions counted by the kernel itself in an untimed repeat of the
+                step, over its own duration measured with events on the launching
+                stream, against the dense 16-bit matrix peak (frac <= 1 by
+                construction); the step's stages timed apart; beside it full_sweep (the
+                launch that scores every pair on the matrix cores), exact_sweep (every
+                pair in the canonical fp32 form on the vector ALUs, against the fp32
+                vector peak) and the same step on volumetric clouds;
   cpu_baseline  the CPU oracle (OpenMP C restatement of the reference algorithm)
                 timed on this box's host cores on a bounded sample of the same
                 workload;
@@ -42,17 +45,16 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3   # MI355X: 256 CU x 256 FLOP/clk x 2.4 GHz
 HBM_PEAK_GBS = 8000.0
 FLOP_PER_PAIR = 8                 # 3 sub, 3 mul, 2 add
 MATRIX_16BIT_PEAK_TFLOPS = 2500.0  # dense 16-bit matrix rate
-MATRIX_FLOP_PER_PAIR = 32         # executed: a 16-term dot product per pair in the pre-filter
+MATRIX_FLOP_PER_PAIR = 32         # executed: a 16-term dot product per scored pair
+PAIRS_PER_MATRIX_INSTRUCTION = 1024  # v_mfma_f32_32x32x16_f16: 32 keys x 32 queries
 
-# HBM bytes per chamfer-forward step at B=32, N=M=16384, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size: the five launches
-# of the sorted path together, and the single launch of the full sweep
-# (profiles/chamfer_forward_sorted_B32_N16384.md, chamfer_forward_mfma_B32_N16384.md).
+# HBM bytes per launch at B=32, N=M=16384 cannot be measured from inside the run: they come
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by a copy kernel of
+# known size, and are kept in the profile summaries named here.
 CHAMFER_SORTED_TRAFFIC_BYTES = 261.3e6
+CHAMFER_SORTED_TRAFFIC_SOURCE = "profiles/chamfer_forward_sorted_B32_N16384.md"
 CHAMFER_TRAFFIC_BYTES = 46.7e6
-# Share of the 2*B*N*M pairs whose score the sorted path evaluates on these clouds
-# (matrix instructions counted by SQ_INSTS_MFMA x 1024 pairs each, same profile).
-CHAMFER_SORTED_PAIRS_EVALUATED = 0.0356
+CHAMFER_TRAFFIC_SOURCE = "profiles/chamfer_forward_mfma_B32_N16384.md"
 
 
 def sphere_cloud(gen, b, n, noise=0.01):
@@ -76,6 +78,73 @@ def gpu_time_ms(fn, steps, warmup):
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
+
+
+def chamfer_outputs(a, c):
+    import torch
+
+    b, n, m = a.shape[0], a.shape[1], c.shape[1]
+    return [torch.empty((b, n), device=a.device), torch.empty((b, n), dtype=torch.int64, device=a.device),
+            torch.empty((b, m), device=a.device), torch.empty((b, m), dtype=torch.int64, device=a.device)]
+
+
+def sorted_stages(a, c, out, ws, stages, counters=None):
+    """The sorted chamfer path stage by stage through the library's test-only entry point
+    (1: sort and key terms, 2: pruned sweep, 4: hand-over check); with `counters` the sweep
+    runs in its counting build."""
+    import ctypes
+
+    from torkit3d_amd import _lib
+
+    fn = _lib.lib().tk3d_debug_chamfer_forward_sorted_counted_f32
+    fn.restype = ctypes.c_int
+    _lib.check(fn(_lib.ptr(a), _lib.ptr(c), _lib.i64(a.shape[0]), _lib.i64(a.shape[1]),
+                  _lib.i64(c.shape[1]), *[_lib.ptr(t) for t in out],
+                  ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()),
+                  ctypes.c_void_p(counters.data_ptr() if counters is not None else 0),
+                  ctypes.c_int(stages), _lib.stream_of(a)),
+               "tk3d_debug_chamfer_forward_sorted_counted_f32")
+
+
+def chamfer_route(a, c, out, route):
+    """Chamfer forward through one named kernel (1: the exact sweep of every pair)."""
+    import ctypes
+
+    from torkit3d_amd import _lib
+
+    fn = _lib.lib().tk3d_debug_chamfer_forward_route_f32
+    fn.restype = ctypes.c_int
+    _lib.check(fn(_lib.ptr(a), _lib.ptr(c), _lib.i64(a.shape[0]), _lib.i64(a.shape[1]),
+                  _lib.i64(c.shape[1]), *[_lib.ptr(t) for t in out], ctypes.c_int(route),
+                  _lib.stream_of(a)), "tk3d_debug_chamfer_forward_route_f32")
+
+
+def sorted_path_breakdown(a, c, steps):
+    """Executed work and per-stage durations of the sorted chamfer path on clouds a, c:
+    matrix instructions counted by the sweep itself in an untimed counting run, stage
+    durations from events around repeated launches of each stage on one workspace."""
+    import torch
+
+    from torkit3d_amd import _lib
+
+    b, n, m = a.shape[0], a.shape[1], c.shape[1]
+    ws = torch.empty((_lib.chamfer_workspace_bytes(b, n, m, True),), dtype=torch.uint8,
+                     device=a.device)
+    out = chamfer_outputs(a, c)
+    counters = torch.zeros(4, dtype=torch.int64, device=a.device)
+    sorted_stages(a, c, out, ws, 7, counters)
+    torch.cuda.synchronize()
+    mfma, waves, scans, handed = counters.cpu().tolist()
+    res = {"matrix_instructions": mfma, "waves": waves, "queries_scanned_exactly": scans,
+           "clouds_handed_over": handed,
+           "pairs_scored": mfma * PAIRS_PER_MATRIX_INSTRUCTION,
+           "pairs_scored_share": mfma * PAIRS_PER_MATRIX_INSTRUCTION / (2.0 * b * n * m)}
+    sorted_stages(a, c, out, ws, 1)  # the workspace the later stages run on
+    res["prepare_ms"] = gpu_time_ms(lambda: sorted_stages(a, c, out, ws, 1), steps, 5)
+    res["sweep_ms"] = gpu_time_ms(lambda: sorted_stages(a, c, out, ws, 2), steps, 5)
+    res["hand_over_check_ms"] = gpu_time_ms(lambda: sorted_stages(a, c, out, ws, 4), steps, 5)
+    res["step_ms"] = gpu_time_ms(lambda: sorted_stages(a, c, out, ws, 7), steps, 5)
+    return res, out
 
 
 def cpu_baseline_chamfer(a, c, budget_s=12.0):
@@ -217,8 +286,8 @@ def cpu_torch_metrics(tensors):
 
 
 def op_roofline(bound, detail, work, ms, unit_work):
-    """Roofline object of one launch: `work` algorithmic bytes (bound "hbm") or FLOP
-    (bound "mfma": the compute class, here the fp32 vector ALUs) over `ms` milliseconds."""
+    """Roofline object of one launch: `work` algorithmic bytes (bound "hbm") or algorithmic
+    fp32 FLOP against the fp32 vector peak (bound "valu") over `ms` milliseconds."""
     if bound == "hbm":
         achieved, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
     else:
@@ -424,9 +493,9 @@ def secondary_metrics(dev, steps, warmup, cpu):
             "hbm", "", 16 * 64 * 4096 * 4 + 16 * 1024 * 32 * 8 + 16 * 64 * 1024 * 32 * 4,
             out["group_bwd_ms"], "bytes"),
         "knn_B32_N8192_M2048_k16": op_roofline(
-            "mfma", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k16_ms"], "flop"),
+            "valu", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k16_ms"], "flop"),
         "knn_B32_N8192_M2048_k3": op_roofline(
-            "mfma", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k3_ms"], "flop"),
+            "valu", valu, 8.0 * 32 * 8192 * 2048, out["knn_B32_N8192_M2048_k3_ms"], "flop"),
         "interpolate_fwd_B32_C128": op_roofline(
             "hbm", "", 32 * 128 * 2048 * 4 + 32 * 8192 * 3 * 12 + 32 * 128 * 8192 * 4,
             out["interpolate_fwd_B32_C128_ms"], "bytes"),
@@ -613,7 +682,6 @@ def main():
 
     pairs = 2.0 * B * N * M
     value = pairs / (wall_ms * 1e-3)
-    achieved_tflops = pairs * FLOP_PER_PAIR / (kernel_ms * 1e-3) / 1e12
 
     # cheap self-check so that a wrong kernel cannot post a number: every reported
     # distance must be the distance to the reported index
@@ -621,6 +689,31 @@ def main():
     near = torch.gather(c, 1, i1[:, :, None].expand(-1, -1, 3))
     if not torch.allclose(((a - near) ** 2).sum(-1), d1, rtol=1e-4, atol=1e-6):
         sys.exit("bench.py: chamfer output failed its self-check")
+
+    # What the step executed: matrix instructions counted by the sweep itself (untimed run of
+    # the counting build), and the duration of each stage on its own.
+    stages, counted_out = sorted_path_breakdown(a, c, max(10, args.steps // 2))
+    for name, got, ref in zip(("dist1", "idx1", "dist2", "idx2"), counted_out, full_out):
+        if not torch.equal(got, ref):
+            sys.exit("bench.py: the counting build of the sorted path differs in " + name)
+    scored = stages["pairs_scored"]
+    sweep_s = stages["sweep_ms"] * 1e-3
+    matrix_tflops = scored * MATRIX_FLOP_PER_PAIR / sweep_s / 1e12
+
+    # the kernel that evaluates every pair in the canonical (x - y)^2 fp32 form, no pre-filter
+    exact_out = chamfer_outputs(a, c)
+    exact_ms = gpu_time_ms(lambda: chamfer_route(a, c, exact_out, 1), max(5, args.steps // 10), 2)
+    for name, got, ref in zip(("dist1", "idx1", "dist2", "idx2"), exact_out, full_out):
+        if not torch.equal(got, ref):
+            sys.exit("bench.py: the exact sweep and the pre-filtered sweep differ in " + name)
+
+    # the same step on volumetric clouds (uniform in the unit cube): the share of pairs the
+    # sorted path has to score depends on the data
+    gen_u = torch.Generator().manual_seed(6)
+    ua, uc = torch.rand(B, N, 3, generator=gen_u).to(dev), torch.rand(B, M, 3, generator=gen_u).to(dev)
+    cube_ms = gpu_time_ms(lambda: _C.chamfer_distance_forward_cuda(ua, uc), max(10, args.steps // 2), 5)
+    cube, _ = sorted_path_breakdown(ua, uc, max(5, args.steps // 5))
+    del ua, uc
 
     line = {
         "metric": "chamfer pair-dists/s at B=32,N=M=16384",
@@ -637,50 +730,98 @@ def main():
         "data": "synthetic",
         "config": {"workload": "chamfer forward (both directions), B=32, N=M=16384 fp32 points "
                                "on unit spheres + N(0,0.01) noise (stress configuration)",
-                   "B": B, "N": N, "M": M},
+                   "B": B, "N": N, "M": M,
+                   "value_is": "nearest neighbours resolved, as pair-distances: 2*B*N*M over the "
+                               "step's duration, whatever share of the pairs the step had to "
+                               "score (roofline.pairs_scored_share); the result is bit-identical "
+                               "to evaluating every pair, checked in this run"},
         "roofline": {
-            # compute-bound; of the two classes the record knows ("hbm" | "mfma") this is
-            # the compute one, measured against the fp32 peak, which on MI355X is the same
-            # 157.3 TFLOP/s for the vector ALUs this kernel uses and for fp32 MFMA
             "bound": "mfma",
-            "bound_detail": "8 algorithmic fp32 FLOP per pair-distance of the 2*B*N*M pairs "
-                            "against the fp32 vector peak, the measure the target is stated "
-                            "in, over the duration of the whole step (cell, sort, tile and "
-                            "pruned-sweep launches plus the hand-over check). frac exceeds 1 "
-                            "because the step is exact without evaluating every pair: key "
-                            "tiles whose box is farther from a wave's queries than their "
-                            "current nearest neighbour are skipped (pairs_evaluated), and "
-                            "the scores of the rest are 16-term dot products on the matrix "
-                            "cores; every reported distance and index comes from the exact "
-                            "fp32 form. full_sweep holds the figures of the launch that "
-                            "evaluates every pair, bit-identical output",
-            "achieved": achieved_tflops,
-            "peak": FP32_VECTOR_PEAK_TFLOPS,
+            "kernel": "chamfer_pruned_kernel",
+            "bound_detail": "work the dominant kernel executed: fp16 matrix instructions "
+                            "(32 keys x 32 queries x 16 terms = 32768 FLOP each) counted by the "
+                            "kernel itself in an untimed repeat of the step, over that kernel's "
+                            "duration (events around launches of the sweep alone on a prepared "
+                            "workspace), against the dense 16-bit matrix peak. The kernel is "
+                            "bound by vector issue and memory latency around the matrix "
+                            "instructions, not by the matrix pipe; valu_equivalent prices the "
+                            "same scored pairs at the 8 fp32 FLOP of the canonical form",
+            "achieved": matrix_tflops,
+            "peak": MATRIX_16BIT_PEAK_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": achieved_tflops / FP32_VECTOR_PEAK_TFLOPS,
-            "traffic": CHAMFER_SORTED_TRAFFIC_BYTES,
-            "kernel": "chamfer_pruned_kernel (with chamfer_cell_kernel, chamfer_sort_kernel, "
-                      "chamfer_tile_kernel before it)",
-            "pairs_evaluated": CHAMFER_SORTED_PAIRS_EVALUATED,
-            "kernel_ms": kernel_ms,
-            "flop_per_pair": FLOP_PER_PAIR,
-            "full_sweep": {
-                "kernel": "chamfer_forward_mfma_kernel",
-                "kernel_ms": full_ms,
-                "pair_dists_per_s": pairs / (full_ms * 1e-3),
-                "achieved": pairs * FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12,
+            "frac": matrix_tflops / MATRIX_16BIT_PEAK_TFLOPS,
+            "kernel_ms": stages["sweep_ms"],
+            "matrix_instructions": stages["matrix_instructions"],
+            "pairs_scored": scored,
+            "pairs_scored_share": stages["pairs_scored_share"],
+            "queries_scanned_exactly": stages["queries_scanned_exactly"],
+            "clouds_handed_over": stages["clouds_handed_over"],
+            "valu_equivalent": {
+                "flop_per_pair": FLOP_PER_PAIR,
+                "achieved": scored * FLOP_PER_PAIR / sweep_s / 1e12,
                 "peak": FP32_VECTOR_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
-                "frac": pairs * FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
-                "traffic": CHAMFER_TRAFFIC_BYTES,
-                "matrix_pipe": {
-                    "flop_per_pair": MATRIX_FLOP_PER_PAIR,
-                    "achieved": pairs * MATRIX_FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12,
-                    "peak": MATRIX_16BIT_PEAK_TFLOPS,
-                    "unit": "TFLOP/s",
-                    "frac": pairs * MATRIX_FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12
-                            / MATRIX_16BIT_PEAK_TFLOPS,
+                "frac": scored * FLOP_PER_PAIR / sweep_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+            },
+            "traffic": CHAMFER_SORTED_TRAFFIC_BYTES,
+            "traffic_source": CHAMFER_SORTED_TRAFFIC_SOURCE,
+            "hbm_frac": CHAMFER_SORTED_TRAFFIC_BYTES / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "step": {
+                "ms": kernel_ms,
+                "prepare_ms": stages["prepare_ms"],
+                "sweep_ms": stages["sweep_ms"],
+                "hand_over_check_ms": stages["hand_over_check_ms"],
+                "matrix_frac": scored * MATRIX_FLOP_PER_PAIR / (kernel_ms * 1e-3) / 1e12
+                               / MATRIX_16BIT_PEAK_TFLOPS,
+                "all_pairs_equivalent": {
+                    "note": "8 fp32 FLOP for every one of the 2*B*N*M pairs over the step's "
+                            "duration against the fp32 vector peak, the measure the target is "
+                            "stated in; above 1 because the step does not evaluate every pair: "
+                            "a speed-up figure, not a roofline fraction",
+                    "achieved": pairs * FLOP_PER_PAIR / (kernel_ms * 1e-3) / 1e12,
+                    "peak": FP32_VECTOR_PEAK_TFLOPS,
+                    "ratio": pairs * FLOP_PER_PAIR / (kernel_ms * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
                 },
+            },
+            "full_sweep": {
+                "kernel": "chamfer_forward_mfma_kernel",
+                "note": "the single launch that scores every pair on the matrix cores",
+                "kernel_ms": full_ms,
+                "pair_dists_per_s": pairs / (full_ms * 1e-3),
+                "bound": "mfma",
+                "achieved": pairs * MATRIX_FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12,
+                "peak": MATRIX_16BIT_PEAK_TFLOPS,
+                "unit": "TFLOP/s",
+                "frac": pairs * MATRIX_FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12
+                        / MATRIX_16BIT_PEAK_TFLOPS,
+                "traffic": CHAMFER_TRAFFIC_BYTES,
+                "traffic_source": CHAMFER_TRAFFIC_SOURCE,
+                "valu_equivalent_frac": pairs * FLOP_PER_PAIR / (full_ms * 1e-3) / 1e12
+                                        / FP32_VECTOR_PEAK_TFLOPS,
+            },
+            "exact_sweep": {
+                "kernel": "chamfer_forward_kernel",
+                "note": "every pair in the canonical (x - y)^2 fp32 form on the vector ALUs, no "
+                        "pre-filter and no matrix cores: the literal form of the target "
+                        "(>= 50 % of the fp32 vector peak)",
+                "kernel_ms": exact_ms,
+                "pair_dists_per_s": pairs / (exact_ms * 1e-3),
+                "bound": "fp32 vector ALUs",
+                "achieved": pairs * FLOP_PER_PAIR / (exact_ms * 1e-3) / 1e12,
+                "peak": FP32_VECTOR_PEAK_TFLOPS,
+                "unit": "TFLOP/s",
+                "frac": pairs * FLOP_PER_PAIR / (exact_ms * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+            },
+            "uniform_cube": {
+                "note": "the same step on clouds uniform in the unit cube (volumetric instead of "
+                        "surface-like)",
+                "ms_per_step": cube_ms,
+                "pair_dists_per_s": pairs / (cube_ms * 1e-3),
+                "pairs_scored_share": cube["pairs_scored_share"],
+                "sweep_ms": cube["sweep_ms"],
+                "prepare_ms": cube["prepare_ms"],
+                "matrix_frac": cube["pairs_scored"] * MATRIX_FLOP_PER_PAIR / (cube["sweep_ms"] * 1e-3)
+                               / 1e12 / MATRIX_16BIT_PEAK_TFLOPS,
             },
         },
     }

@@ -21,6 +21,7 @@
 //
 // Both directions (cloud 1 -> 2 and 2 -> 1) run in one launch.
 #include "tk3d_common.h"
+#include "tk3d_debug.h"
 
 namespace {
 
@@ -676,16 +677,32 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_filter_kernel(ChamferFw
 // i.e. all four piece products of every coordinate plus |k'|^2. Products of two fp16
 // values are exact in fp32. With u = 2^-24, R = (max|k'| + |q'|)^2:
 //     pieces dropped from 2 q'.k'    2 * 2^-23 * sum |x||X| <= 2^-21 |q'||k'| <=    2 u R
-//     subnormal pieces               2^-25 * (sum |X| + sum |x|)              <=      1 u R
+//     the pieces' absolute floor     2^-25 * (sum |X| + sum |x|) <= 1.75 u (max|k'| + |q'|)
+//                                    <= 7 u R given max|k'| >= 1/4                   7 u R
 //     |k'|^2 as staged                                                            3.2 u R
-//     the matrix core's 16 additions, one unit in the last place of the largest
-//         partial sum each (round to nearest would be half a unit; measured on
-//         this GPU: at most 9.3 u times the largest product)                        32 u R
+//     the matrix core's 16 additions                                               33 u R
 //     canonical d2 against the exact distance of the centred points               7.1 u R
-// so |s + |q'|^2 - canonical d2| <= E = 45.3 u R, and a key whose canonical distance
+// so |s + |q'|^2 - canonical d2| <= E = 52.3 u R, and a key whose canonical distance
 // equals the minimum has s <= min(s) + 2 E. The kernel uses slack = 128 u R = 2^-17 R
 // (+ 1e-36 in the caller's units against underflow of the canonical distance).
 // A query beyond fp16's range (|q'| > 16000) goes to the exact scan.
+//
+// The floor of the pieces is why max|k'| >= 1/4 is required and checked: a key cloud whose
+// keys all sit within 0.02 of the centre at this scale has scores off by a thousand u R. Here
+// the scale comes from the sampled extent, a sampled key lies on the sample's bounding box,
+// so max|k'| >= 1 unless the sample has no extent; then (scale 1) a cloud with
+// 0 < max|k'| < 1/2 takes the exact sweep.
+//
+// The additions. The matrix core aligns the 16 products to the largest exponent among them
+// and cuts them off about 25 bits below it, where a product's exponent is the sum of its
+// factors' exponent fields: a subnormal fp16 factor counts as 2^-14 however small it is.
+// With m(v) = max(|v|, 2^-14) for v != 0, the budget is one unit in the last place of the
+// running sum per addition, |result - sum a_i b_i| <= 32 u sum m(a_i) m(b_i) (measured: 4.5 u;
+// against true magnitudes the error reaches 147 u times the largest product when subnormal
+// and huge factors meet). For the terms above a subnormal piece is seen as at most 2^-14 times
+// the other factor, below 2^-10 R per term given max|k'| >= 1/4, so the sum of seen magnitudes
+// is below 1.02 R. tests/test_gpu_mfma_bound.py checks the budget and the whole score against
+// exact arithmetic on this GPU.
 //
 // Layout. In the 32 x 32 result a lane holds 16 keys (rows 8a + 4h + c, a, c < 4, h =
 // lane / 32) of one query (column lane % 32): lanes l and l + 32 serve the same query
@@ -1008,9 +1025,10 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
 #pragma unroll
     for (int w = 0; w < NW; ++w)
         kmax2 = __builtin_fmaxf(kmax2, sred[w][6]);
-    // (also +inf; and a sample of identical keys, scale 1, beside keys that differ from it
-    // by far less than 1: the fp16 terms have no precision for those)
-    if (!(kmax2 <= 32768.0f) || (ext == 0.0f && kmax2 > 0.0f && kmax2 < 0.25f)) {  // uniform
+    // (also +inf; and keys that all differ from the centre by far less than 1 - a sample of
+    // identical keys, scale 1, beside keys that differ a little: the fp16 terms have no
+    // precision for those; with a sample that has an extent max|k'| >= 1)
+    if (!(kmax2 <= 32768.0f) || (kmax2 > 0.0f && kmax2 < 0.25f)) {  // uniform
         chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
@@ -1811,7 +1829,7 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
 //
 // Why a skipped tile cannot matter. With the notation of the matrix kernel (k', q' the
 // centred, scaled points as rounded, u = 2^-24, R = (max|k'| + |q'|)^2): the score of a
-// swept key satisfies |s + |q'|^2 - d2| <= 45.3 u R for its canonical distance d2 (in
+// swept key satisfies |s + |q'|^2 - d2| <= 52.3 u R for its canonical distance d2 (in
 // scaled units), so ub = min s + |q'|^2 + 128 u R (the sum in fp32: 4 u R more) is at
 // least the canonical distance of some swept key. For a key of a skipped tile,
 // d2 >= |q' - k'|^2 - 7.1 u R >= gap^2 - 7.1 u R, where gap^2, evaluated in fp32 from box
@@ -2259,6 +2277,7 @@ struct ChamferPrunedArgs {
     int B;
     int waves_per_cloud[2];
     int waves0;  // waves of direction 0 (queries: cloud 0); the rest belong to direction 1
+    unsigned long long *counters;  // COUNT builds only: executed work, four words
 };
 
 __device__ __forceinline__ int wave_reduce_min_int(int v)
@@ -2274,7 +2293,7 @@ __device__ __forceinline__ int wave_reduce_min_int(int v)
 // (Launched one wave per workgroup - waves share nothing, and a finished wave frees its
 // slot at once: 2-3 % over four waves per workgroup. The bound of 256 lanes only caps the
 // registers at four waves per SIMD.)
-template <int NQB, int RMAX>
+template <int NQB, int RMAX, bool COUNT = false>
 __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a)
 {
     const int tid = threadIdx.x;
@@ -2361,7 +2380,11 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         }
         return;
     }
-    if (!(far2 <= 6.4e7f) || dwarfed || nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
+    // The error bound of the scores counts on a swept key with |k'| >= 1/4 (the fp16 pieces
+    // have an absolute floor): a frame that outliers stretched far beyond the bulk of the
+    // keys does not give one.
+    const bool flat_terms = hk->kmax2_bits < 0x3d800000;  // |k'|^2 < 1/16 for every swept key
+    if (!(far2 <= 6.4e7f) || dwarfed || flat_terms || nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
         if (lane == 0)
             atomicOr(flag, 1);
         return;
@@ -2571,6 +2594,12 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         }
     }
 
+    if constexpr (COUNT) {  // matrix instructions issued and waves that swept
+        if (lane == 0 && nswept > 0) {
+            atomicAdd(a.counters + 0, (unsigned long long)nswept * NQB);
+            atomicAdd(a.counters + 1, 1ull);
+        }
+    }
     // ---- exact evaluation of each half's candidate tiles, then the merge ----
     unsigned over_mask[NQB], stray_mask[NQB];
     int nover = 0;
@@ -2642,6 +2671,10 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     }
     if (nover == 0 && nstray == 0)
         return;
+    if constexpr (COUNT) {  // queries that take an exact scan
+        if (lane == 0)
+            atomicAdd(a.counters + 2, (unsigned long long)(nover + nstray));
+    }
     // An exact scan costs about 13 instructions per two swept tiles (a normal wave issues
     // 2100 in all): beyond 8192 (query, tile) pairs - half of what sweeping the whole cloud
     // exactly would cost the wave - the cloud is handed to the other kernel (heavy ties:
@@ -2766,10 +2799,29 @@ inline ChamferSortedLayout chamfer_sorted_layout(int64_t B, int64_t N1, int64_t 
     return l;
 }
 
+__global__ __launch_bounds__(256) void chamfer_count_clear_kernel(unsigned long long *counters)
+{
+    if (threadIdx.x < 4)
+        counters[threadIdx.x] = 0ull;
+}
+
+__global__ __launch_bounds__(256) void chamfer_count_flags_kernel(const int *flags, int n,
+                                                                 unsigned long long *counters)
+{
+    unsigned long long mine = 0;
+    for (int i = threadIdx.x; i < n; i += 256)
+        mine += flags[i] != 0 ? 1ull : 0ull;
+    if (mine != 0)
+        atomicAdd(counters + 3, mine);
+}
+
 int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                            int64_t N2, float *dist1, int64_t *idx1, float *dist2, int64_t *idx2,
-                           void *workspace, hipStream_t s)
+                           void *workspace, hipStream_t s, unsigned long long *counters = nullptr,
+                           int stages = 7)
 {
+    // stages (tests and the benchmark time them apart): 1 the preparing launches, 2 the
+    // pruned sweep, 4 the hand-over check
     constexpr int NQB = 2;
     const ChamferSortedLayout l = chamfer_sorted_layout(B, N1, N2);
     char *ws = static_cast<char *>(workspace);
@@ -2807,24 +2859,41 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
     if (waves0 + waves1 > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
     pa.waves0 = (int)waves0;
+    pa.counters = counters;
+    if (counters != nullptr)
+        hipLaunchKernelGGL(chamfer_count_clear_kernel, dim3(1), dim3(256), 0, s, counters);
     constexpr size_t lds = (size_t)CHAMFER_SORT_CELLS * sizeof(int);
     const int allowed = tk_allow_dynamic_lds<chamfer_sort_kernel>((int)lds);
     if (allowed != TK3D_OK)
         return allowed;
-    hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
-                       dim3(1024), 0, s, sa);
-    hipLaunchKernelGGL(chamfer_sort_kernel, dim3((unsigned)(2 * B)), dim3(1024), lds, s, sa);
-    const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
-    hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s, sa,
-                       (int)tb0);
+    if (stages & 1) {
+        hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
+                           dim3(1024), 0, s, sa);
+        hipLaunchKernelGGL(chamfer_sort_kernel, dim3((unsigned)(2 * B)), dim3(1024), lds, s, sa);
+        const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
+        hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s, sa,
+                           (int)tb0);
+    }
     const dim3 grid((unsigned)((waves0 + waves1)));
-    if (l.npad[0] <= 16384 && l.npad[1] <= 16384)
+    const bool small = l.npad[0] <= 16384 && l.npad[1] <= 16384;
+    if (!(stages & 2)) {
+    } else if (counters != nullptr) {  // (the counting build: tests and the benchmark's untimed repeat)
+        if (small)
+            hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 8, true>), grid, dim3(64), 0, s, pa);
+        else
+            hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 32, true>), grid, dim3(64), 0, s, pa);
+        hipLaunchKernelGGL(chamfer_count_flags_kernel, dim3(1), dim3(256), 0, s, sa.flags,
+                           (int)(2 * B), counters);
+    } else if (small) {
         hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 8>), grid, dim3(64), 0, s, pa);
-    else
+    } else {
         hipLaunchKernelGGL((chamfer_pruned_kernel<NQB, 32>), grid, dim3(64), 0, s, pa);
+    }
     const int rc = tk_launch_status();
     if (rc != TK3D_OK)
         return rc;
+    if (!(stages & 4))
+        return TK3D_OK;
     // whatever the waves above handed over (none on ordinary input: its workgroups leave
     // at once)
     return chamfer_forward_mfma_flagged_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
@@ -2876,6 +2945,91 @@ int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
                        dim3(256), 0, s, gd1, gd2, xyz1, xyz2, idx1, idx2, t1, t2, (int)N1,
                        (int)N2, gx1, gx2);
     return tk_launch_status();
+}
+
+// ---- entry points for the tests and the benchmark (tk3d_debug.h) ----------------------
+
+// One matrix instruction per tile on caller-supplied fp16 terms. Lane l supplies terms
+// 8 (l / 32) .. + 7 of key l % 32 as the first operand and of query l % 32 as the second;
+// in the result, register r of lane l is key 8 (r / 4) + 4 (l / 32) + r % 4, query l % 32.
+__global__ __launch_bounds__(64) void debug_mfma_dot16_kernel(const uint4 *__restrict__ key_terms,
+                                                              const uint4 *__restrict__ query_terms,
+                                                              float *__restrict__ scores)
+{
+    const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    const int64_t t = blockIdx.x;
+    const uint4 ka = key_terms[(t * 32 + col) * 2 + half];
+    const uint4 qb = query_terms[(t * 32 + col) * 2 + half];
+    const tk_f32x16 zero = {};
+    const tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(tk_f16x8, ka), __builtin_bit_cast(tk_f16x8, qb), zero, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        scores[(t * 32 + 8 * (r / 4) + 4 * half + r % 4) * 32 + col] = acc[r];
+}
+
+// The chamfer pre-filter's score for centred, scaled points, terms staged as the kernels do.
+__global__ __launch_bounds__(64) void debug_chamfer_scores_kernel(const float *__restrict__ keys,
+                                                                  const float *__restrict__ queries,
+                                                                  float *__restrict__ scores)
+{
+    const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    const int64_t t = blockIdx.x;
+    const float *k = keys + (t * 32 + col) * 3, *q = queries + (t * 32 + col) * 3;
+    const float nn = __builtin_fmaf(k[2], k[2], __builtin_fmaf(k[1], k[1], k[0] * k[0]));
+    uint4 h0, h1;
+    chamfer_key_terms(k[0], k[1], k[2], nn, true, h0, h1);
+    const uint4 ka = half == 0 ? h0 : h1;
+    const uint4 qb = chamfer_query_terms(q[0], q[1], q[2], half);
+    const tk_f32x16 zero = {};
+    const tk_f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(tk_f16x8, ka), __builtin_bit_cast(tk_f16x8, qb), zero, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        scores[(t * 32 + 8 * (r / 4) + 4 * half + r % 4) * 32 + col] = acc[r];
+}
+
+int chamfer_forward_route(const float *xyz1, const float *xyz2, int64_t B, int64_t N1, int64_t N2,
+                          float *dist1, int64_t *idx1, float *dist2, int64_t *idx2, int route,
+                          hipStream_t s)
+{
+    if (B < 0 || N1 < 0 || N2 < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (N1 > TK_MAX_I32 / 4 || N2 > TK_MAX_I32 / 4 || !tk_fits(TK_MAX_ELEMS, B, N1, 3) ||
+        !tk_fits(TK_MAX_ELEMS, B, N2, 3))
+        return TK3D_ERR_UNSUPPORTED;
+    if (B * N1 > 0 && (!xyz1 || !dist1 || !idx1))
+        return TK3D_ERR_NULL_POINTER;
+    if (B * N2 > 0 && (!xyz2 || !dist2 || !idx2))
+        return TK3D_ERR_NULL_POINTER;
+    const int64_t lo = N1 < N2 ? N1 : N2, hi = N1 < N2 ? N2 : N1;
+    switch (route) {
+    case TK3D_CHAMFER_ROUTE_EXACT:
+        return chamfer_forward_launch<float, 4, 512, 64>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
+                                                         idx2, s);
+    case TK3D_CHAMFER_ROUTE_VECTOR:
+        if (lo < 512)
+            return TK3D_ERR_UNSUPPORTED;
+        return chamfer_forward_filter_launch<4, 512, 64, 512>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                              dist2, idx2, s);
+    case TK3D_CHAMFER_ROUTE_MATRIX4:
+    case TK3D_CHAMFER_ROUTE_MATRIX2:
+    case TK3D_CHAMFER_ROUTE_MATRIX_SLICED: {
+        if (lo < 1 || hi < 1024)
+            return TK3D_ERR_UNSUPPORTED;
+        if (route == TK3D_CHAMFER_ROUTE_MATRIX2)
+            return chamfer_forward_mfma_launch<2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
+                                                  s);
+        if (route == TK3D_CHAMFER_ROUTE_MATRIX4)
+            return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
+                                                  s);
+        const int64_t w0 = (N2 + 1023) / 1024, w1 = (N1 + 1023) / 1024;
+        return chamfer_forward_mfma_launch<2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, s,
+                                              (int)(w0 > 256 ? 256 : w0), (int)(w1 > 256 ? 256 : w1));
+    }
+    default:
+        return TK3D_ERR_UNSUPPORTED;
+    }
 }
 
 }  // namespace
@@ -2941,6 +3095,64 @@ int tk3d_chamfer_distance_backward_f64(const double *grad_dist1,
 {
     return chamfer_backward<double>(grad_dist1, grad_dist2, xyz1, xyz2, idx1, idx2, B, N1,
                                     N2, grad_xyz1, grad_xyz2, stream);
+}
+
+int tk3d_debug_chamfer_forward_route_f32(const float *xyz1, const float *xyz2, int64_t B,
+                                         int64_t N1, int64_t N2, float *dist1, int64_t *idx1,
+                                         float *dist2, int64_t *idx2, int route, void *stream)
+{
+    return chamfer_forward_route(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, route,
+                                 (hipStream_t)stream);
+}
+
+int tk3d_debug_chamfer_forward_sorted_counted_f32(const float *xyz1, const float *xyz2,
+                                                  int64_t B, int64_t N1, int64_t N2,
+                                                  float *dist1, int64_t *idx1, float *dist2,
+                                                  int64_t *idx2, void *workspace,
+                                                  size_t workspace_bytes,
+                                                  unsigned long long *counters, int stages,
+                                                  void *stream)
+{
+    if (!workspace || !xyz1 || !xyz2 || !dist1 || !idx1 || !dist2 || !idx2)
+        return TK3D_ERR_NULL_POINTER;
+    if (!chamfer_sorted_can_serve(B, N1, N2))
+        return TK3D_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+        workspace_bytes < chamfer_sorted_layout(B, N1, N2).total)
+        return TK3D_ERR_WORKSPACE;
+    return chamfer_forward_sorted(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, workspace,
+                                  (hipStream_t)stream, counters, stages);
+}
+
+int tk3d_debug_mfma_dot16_f16(const uint16_t *key_terms, const uint16_t *query_terms, int64_t T,
+                              float *scores, void *stream)
+{
+    if (T < 0 || T > TK_MAX_I32)
+        return TK3D_ERR_BAD_SIZE;
+    if (T == 0)
+        return TK3D_OK;
+    if (!key_terms || !query_terms || !scores)
+        return TK3D_ERR_NULL_POINTER;
+    if (((reinterpret_cast<uintptr_t>(key_terms) | reinterpret_cast<uintptr_t>(query_terms)) & 15) != 0)
+        return TK3D_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(debug_mfma_dot16_kernel, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint4 *>(key_terms),
+                       reinterpret_cast<const uint4 *>(query_terms), scores);
+    return tk_launch_status();
+}
+
+int tk3d_debug_chamfer_scores_f32(const float *keys, const float *queries, int64_t T,
+                                  float *scores, void *stream)
+{
+    if (T < 0 || T > TK_MAX_I32)
+        return TK3D_ERR_BAD_SIZE;
+    if (T == 0)
+        return TK3D_OK;
+    if (!keys || !queries || !scores)
+        return TK3D_ERR_NULL_POINTER;
+    hipLaunchKernelGGL(debug_chamfer_scores_kernel, dim3((unsigned)T), dim3(64), 0,
+                       (hipStream_t)stream, keys, queries, scores);
+    return tk_launch_status();
 }
 
 }  // extern "C"

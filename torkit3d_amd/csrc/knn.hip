@@ -16,6 +16,7 @@
 #include <type_traits>
 
 #include "tk3d_common.h"
+#include "tk3d_debug.h"
 
 namespace {
 
@@ -433,11 +434,12 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 // one above (products of the second pieces are left out, thr is rounded to two pieces):
 //     pieces dropped from 2 q'.k', subnormal pieces                       5 u R
 //     |k'|^2 and thr in two pieces                           4 u R + 4 u (M + R)
-//     the matrix core's 16 additions, one unit in the last place of the largest
-//         partial sum each (measured: at most 9.3 u times the largest product)
-//                                                                    32 u (M + R)
+//     the matrix core's 16 additions: 32 u times the sum of the products' magnitudes
+//         as the matrix core sees them (a subnormal fp16 factor counts as 2^-14; see
+//         the chamfer kernel and tests/test_gpu_mfma_bound.py), which is below
+//         1.02 (M + R) here because the scale makes max|k'| >= 1     33 u (M + R)
 //     canonical d2, |k'|^2 as staged, thr itself             10 u R + 3 u (M + R)
-// below 58 u R + 39 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
+// below 59 u R + 40 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
 // from the centre (rescaled; thr would leave fp16's range) take every key as a candidate.
 template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK>
 __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
@@ -2112,15 +2114,24 @@ inline bool knn_filter_pays(int64_t queries, int n2, int k)
     return n2 >= (k <= 8 ? 512 : 1024) || (n2 >= 512 && queries >= 131072);
 }
 
+// Whether knn_filter_launch takes this launch: the one test both entry points and the
+// launch itself go by.
+inline bool knn_filter_takes(int64_t B, int n1, int n2, int k)
+{
+    const int64_t bpb = ((int64_t)n1 + 511) / 512;
+    return k <= 16 && knn_filter_pays(B * n1, n2, k) && B * bpb <= TK_MAX_I32;
+}
+
 template <int KMAX, bool SOA, bool WEIGHTS>
 int knn_filter_launch(const float *query, const float *key, float *distance, int64_t *index,
-                      float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
+                      float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s,
+                      bool whatever_the_size = false)
 {
     // One query per lane, 512 lanes: two workgroups (16 waves) per CU. Two queries per lane
     // in 256 lanes need twice the registers, which leaves two waves per SIMD, and were 1.1
     // to 1.4 times slower on every shape (k = 16 at B=32, 8192 x 2048: 222 -> 191 us).
     const int64_t bpb = ((int64_t)n1 + 511) / 512;
-    if (!knn_filter_pays(B * n1, n2, k) || B * bpb > TK_MAX_I32)
+    if (B * bpb > TK_MAX_I32 || !(whatever_the_size || knn_filter_takes(B, n1, n2, k)))
         return TK3D_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512>),
                        dim3((unsigned)(B * bpb)), dim3(512), 0, s, query, key, distance, index,
@@ -2262,12 +2273,12 @@ int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int
     if (B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
     const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
-    if (sizeof(T) == 4 && k > 4 && (k > 16 || !knn_filter_pays(B * N1, n2, kk)))
-        return TK3D_ERR_UNSUPPORTED;
     if (B * N1 == 0)
         return TK3D_OK;
     if (!query || !key || !distance || !index)
         return TK3D_ERR_NULL_POINTER;
+    if (sizeof(T) == 4 && k > 4 && !knn_filter_takes(B, n1, n2, kk))
+        return TK3D_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if constexpr (sizeof(T) == 4) {
         int rc = TK3D_ERR_UNSUPPORTED;
@@ -2386,6 +2397,33 @@ int tk3d_knn_distance_f64(const double *query, const double *key, int64_t B, int
                           int64_t *index, void *stream)
 {
     return knn<double>(query, key, B, N1, N2, k, version, distance, index, stream);
+}
+
+int tk3d_debug_knn_filter_f32(const float *query, const float *key, int64_t B, int64_t N1,
+                              int64_t N2, int64_t k, float *distance, int64_t *index,
+                              void *stream)
+{
+    if (B < 0 || N1 < 0 || N2 < 0)
+        return TK3D_ERR_BAD_SIZE;
+    if (k <= 0 || k > N2)
+        return TK3D_ERR_BAD_K;
+    if (k > 16 || N2 < 256 || N1 > TK_MAX_I32 / 4 || N2 > TK_MAX_I32 / 4 ||
+        !tk_fits(TK_MAX_ELEMS, B, N1, k) || !tk_fits(TK_MAX_ELEMS, B, N2, 3))
+        return TK3D_ERR_UNSUPPORTED;
+    if (B * N1 == 0)
+        return TK3D_OK;
+    if (!query || !key || !distance || !index)
+        return TK3D_ERR_NULL_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    const int n1 = (int)N1, n2 = (int)N2, kk = (int)k;
+    if (k <= 4)
+        return knn_filter_launch<4, false, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                  n1, n2, kk, s, true);
+    if (k <= 8)
+        return knn_filter_launch<8, false, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                  n1, n2, kk, s, true);
+    return knn_filter_launch<16, false, false>(query, key, distance, index, nullptr, 0.0f, B, n1,
+                                               n2, kk, s, true);
 }
 
 }  // extern "C"
