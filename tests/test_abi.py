@@ -22,8 +22,11 @@ def lib():
     return _lib.lib()
 
 
-def declared_symbols():
-    text = open(HEADER).read()
+DEBUG_HEADER = os.path.join(REPO, "torkit3d_amd", "csrc", "tk3d_debug.h")
+
+
+def declared_symbols(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tk3d_[a-z0-9_]+)\s*\(", text)))
 
@@ -41,6 +44,22 @@ def test_header_declares_the_expected_families():
 def test_every_declared_symbol_is_exported(lib):
     for name in declared_symbols():
         assert hasattr(lib, name), "%s declared in tk3d.h but not exported" % name
+
+
+def test_test_only_entry_points_are_exported_and_outside_the_boundary(lib):
+    # what the tests and the benchmark call besides the boundary: declared in a header of its
+    # own, none of it in include/tk3d.h
+    debug = declared_symbols(DEBUG_HEADER)
+    assert debug and all(name.startswith("tk3d_debug_") for name in debug)
+    assert not any(name.startswith("tk3d_debug_") for name in declared_symbols())
+    for name in debug:
+        assert hasattr(lib, name), "%s declared in tk3d_debug.h but not exported" % name
+    fn = lib.tk3d_debug_chamfer_forward_route_f32
+    fn.restype = ctypes.c_int
+    null = ctypes.c_void_p(0)
+    # argument checks come before any launch
+    assert fn(null, null, i64(-1), i64(4), i64(4), null, null, null, null, ctypes.c_int(1), null) == -2
+    assert fn(null, null, i64(1), i64(4), i64(4), null, null, null, null, ctypes.c_int(1), null) == -1
 
 
 def test_version_and_error_strings(lib):
