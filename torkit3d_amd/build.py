@@ -29,6 +29,8 @@ HIPCC_FLAGS = [
     # matrix instructions write ordinary vector registers (no copies out of the
     # accumulation registers before the vector ALU can use a result)
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # the Hilbert curve table of the chamfer sort is worked out at compile time
+    "-fconstexpr-steps=200000000",
     "-Wall",
     "-Wno-unused-function",
 ]

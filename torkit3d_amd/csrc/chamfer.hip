@@ -23,6 +23,8 @@
 #include "tk3d_common.h"
 #include "tk3d_debug.h"
 
+#include <type_traits>
+
 namespace {
 
 template <typename T> struct ChamferDir {
@@ -1162,13 +1164,17 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
     chamfer_mfma_block<NQB, BLOCK, STAGE>(d, b, qblock, slice);
 }
 
-// The same sweep for the clouds another kernel has flagged (args.only_if): a fixed, small
+// The same sweep for the clouds another kernel has flagged (args.only_if: a word per
+// direction and batch element, then one that is set when any of them is): a fixed, small
 // number of workgroups go through all (direction, batch element, query block) shares and
-// work on those whose cloud carries a flag, so a launch that finds no flag costs little.
+// work on those whose cloud carries a flag; a launch that finds no flag at all leaves at
+// once.
 template <int NQB, int BLOCK, int STAGE>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 chamfer_forward_mfma_flagged_kernel(ChamferFwdArgs<float> args, int total)
 {
+    if (args.only_if[2 * args.nbatch] == 0)  // no cloud carries a flag: nothing to do
+        return;
     for (int lb = blockIdx.x; lb < total; lb += gridDim.x) {
         const int which = lb >= args.nblocks0;
         const int rest0 = lb - (which ? args.nblocks0 : 0);
@@ -1867,12 +1873,14 @@ struct ChamferSortArgs {
                         // six fp16 values rounded outwards
     float4 *far_keys[2];  // [B, CHAMFER_FAR_KEYS]: x, y, z, original index
     ChamferSortedHdr *hdr;  // [2, B]
-    int *flags;             // [2, B]
+    int *flags;             // [2, B], then one word that is set when any of them is
     int n[2], npad[2];
     int B;
+    int three_launches[2];  // this cloud is prepared by the cell, sort and tile kernels
+                            // (beyond 16384 points); else by chamfer_prepare_kernel
 };
 
-__device__ __forceinline__ int chamfer_morton5(int v)
+__host__ __device__ constexpr int chamfer_morton5(int v)
 {
     v &= 0x1f;
     v = (v | (v << 8)) & 0x100f;
@@ -1885,7 +1893,7 @@ __device__ __forceinline__ int chamfer_morton5(int v)
 // (Skilling's transposed form, then the bits interleaved): consecutive positions are
 // neighbouring cells, so a run of consecutive sorted points is a compact patch, which a
 // run along the Morton curve, with its jumps, often is not.
-__device__ __forceinline__ int chamfer_hilbert15(unsigned x, unsigned y, unsigned z)
+__host__ __device__ constexpr int chamfer_hilbert15(unsigned x, unsigned y, unsigned z)
 {
     unsigned X[3] = {x, y, z};
 #pragma unroll
@@ -1913,6 +1921,103 @@ __device__ __forceinline__ int chamfer_hilbert15(unsigned x, unsigned y, unsigne
            chamfer_morton5((int)X[2]);
 }
 
+// A pilot centre that a few stray points cannot move: per axis the median of three medians
+// of three, over nine points spread through the cloud; and `cap`, 16 times the typical
+// deviation of the nine from it (none, i.e. the nine coincide: no cap).
+__device__ __forceinline__ void chamfer_pilot(const float *__restrict__ P, int n, float (&pilot)[3],
+                                              float (&cap)[3])
+{
+    const float INF = __builtin_huge_valf();
+    TkPoint3<float> q[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i)
+        q[i] = tk_load3<float>(P + (((int64_t)n * (2 * i + 1)) / 19) * 3);
+    auto ninther = [](float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                      float v7, float v8) {
+        return __builtin_amdgcn_fmed3f(__builtin_amdgcn_fmed3f(v0, v1, v2),
+                                       __builtin_amdgcn_fmed3f(v3, v4, v5),
+                                       __builtin_amdgcn_fmed3f(v6, v7, v8));
+    };
+    pilot[0] = ninther(q[0].x, q[1].x, q[2].x, q[3].x, q[4].x, q[5].x, q[6].x, q[7].x, q[8].x);
+    pilot[1] = ninther(q[0].y, q[1].y, q[2].y, q[3].y, q[4].y, q[5].y, q[6].y, q[7].y, q[8].y);
+    pilot[2] = ninther(q[0].z, q[1].z, q[2].z, q[3].z, q[4].z, q[5].z, q[6].z, q[7].z, q[8].z);
+    float d[9][3];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        d[i][0] = __builtin_fabsf(q[i].x - pilot[0]);
+        d[i][1] = __builtin_fabsf(q[i].y - pilot[1]);
+        d[i][2] = __builtin_fabsf(q[i].z - pilot[2]);
+    }
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        const float typical = ninther(d[0][ax], d[1][ax], d[2][ax], d[3][ax], d[4][ax],
+                                      d[5][ax], d[6][ax], d[7][ax], d[8][ax]);
+        cap[ax] = typical > 0.0f ? 16.0f * typical : INF;
+    }
+}
+
+// The frame of a cloud from the waves' partial results (sred: lo and hi per axis, sdev: sums
+// of capped deviations): the bounding box, trimmed to three mean deviations around the pilot
+// centre. A uniform or a Gaussian cloud keeps (nearly) its bounding box - three mean
+// deviations are 1.5 half extents of the first and 2.4 sigma of the second, and keys up to
+// twice as far out as the frame are still swept like any other; a few points far away no
+// longer decide the cells and the scale of everything else - they go on a list of their own.
+// Returns the bounding box (lo, hi), the frame's centre cc, lower corner flo and largest half
+// extent ext.
+template <int NW>
+__device__ __forceinline__ void chamfer_frame(const float (*sred)[8], const float (*sdev)[4],
+                                              const float (&pilot)[3], int n, float (&lo)[3],
+                                              float (&hi)[3], float (&cc)[3], float (&flo)[3],
+                                              float &ext)
+{
+    ext = 0.0f;
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        float l = sred[0][ax], h = sred[0][3 + ax], dsum = sdev[0][ax];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) {
+            l = __builtin_fminf(l, sred[w][ax]);
+            h = __builtin_fmaxf(h, sred[w][3 + ax]);
+            dsum += sdev[w][ax];
+        }
+        lo[ax] = l;
+        hi[ax] = h;
+        const float reach = 3.0f * (dsum / (float)n);
+        const float fl = __builtin_fmaxf(l, pilot[ax] - reach);
+        const float fh = __builtin_fminf(h, pilot[ax] + reach);
+        flo[ax] = fl;
+        cc[ax] = 0.5f * fl + 0.5f * fh;
+        ext = __builtin_fmaxf(ext, 0.5f * fh - 0.5f * fl);
+    }
+    if (ext == 0.0f) {
+        // Nearly all points in one place: a frame of no extent would leave the others at
+        // scale 1, possibly far below it, where the fp16 terms have no precision left
+        // (the error bound counts on max|k'| of order 1). The bounding box, then.
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            flo[ax] = lo[ax];
+            cc[ax] = 0.5f * lo[ax] + 0.5f * hi[ax];
+            ext = __builtin_fmaxf(ext, 0.5f * hi[ax] - 0.5f * lo[ax]);
+        }
+    }
+}
+
+// A tile's box as six fp16 corners, moved outwards by more than the rounding to nearest can
+// bring them back (2^-11 relative, 2^-25 in the subnormal range); an empty box stays
+// (+inf, -inf).
+__device__ __forceinline__ uint4 chamfer_box_bits(const float (&bl)[3], const float (&bh)[3])
+{
+    unsigned h[6];
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        const float wl = __builtin_fabsf(bl[ax]) * 9.765625e-4f + 1.1920929e-7f;
+        const float wh = __builtin_fabsf(bh[ax]) * 9.765625e-4f + 1.1920929e-7f;
+        h[ax] = bl[ax] > 3.0e38f ? 0x7c00u : tk_f16_bits(bl[ax] - wl);
+        h[3 + ax] = bh[ax] < -3.0e38f ? 0xfc00u : tk_f16_bits(bh[ax] + wh);
+    }
+    return make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), 0u);
+}
+
 constexpr int CHAMFER_SORT_CELLS = 32768;
 
 // Bounding box of a cloud and the cell of every point. CHAMFER_CELL_PARTS workgroups per
@@ -1931,6 +2036,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
     const int cloud = (int)blockIdx.x / PARTS, part = (int)blockIdx.x - cloud * PARTS;
     const int which = cloud >= a.B;
+    if (!a.three_launches[which])  // uniform over the workgroup
+        return;
     const int b = cloud - which * a.B;
     const int n = a.n[which], npad = a.npad[which];
     const float *__restrict__ P = a.xyz[which] + (int64_t)b * n * 3;
@@ -1953,35 +2060,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
             const int j = base + u * NT + tid;
             p[u] = tk_load3<float>(P + (int64_t)(j < n ? j : n - 1) * 3);
         }
-        if (base == 0) {  // (requested together with the first points: one round trip)
-            TkPoint3<float> q[9];
-#pragma unroll
-            for (int i = 0; i < 9; ++i)
-                q[i] = tk_load3<float>(P + (((int64_t)n * (2 * i + 1)) / 19) * 3);
-            auto ninther = [](float v0, float v1, float v2, float v3, float v4, float v5, float v6,
-                              float v7, float v8) {
-                return __builtin_amdgcn_fmed3f(__builtin_amdgcn_fmed3f(v0, v1, v2),
-                                               __builtin_amdgcn_fmed3f(v3, v4, v5),
-                                               __builtin_amdgcn_fmed3f(v6, v7, v8));
-            };
-            pilot[0] = ninther(q[0].x, q[1].x, q[2].x, q[3].x, q[4].x, q[5].x, q[6].x, q[7].x, q[8].x);
-            pilot[1] = ninther(q[0].y, q[1].y, q[2].y, q[3].y, q[4].y, q[5].y, q[6].y, q[7].y, q[8].y);
-            pilot[2] = ninther(q[0].z, q[1].z, q[2].z, q[3].z, q[4].z, q[5].z, q[6].z, q[7].z, q[8].z);
-            // the typical deviation of the nine, the same way; none (the nine coincide): no cap
-            float d[9][3];
-#pragma unroll
-            for (int i = 0; i < 9; ++i) {
-                d[i][0] = __builtin_fabsf(q[i].x - pilot[0]);
-                d[i][1] = __builtin_fabsf(q[i].y - pilot[1]);
-                d[i][2] = __builtin_fabsf(q[i].z - pilot[2]);
-            }
-#pragma unroll
-            for (int ax = 0; ax < 3; ++ax) {
-                const float typical = ninther(d[0][ax], d[1][ax], d[2][ax], d[3][ax], d[4][ax],
-                                              d[5][ax], d[6][ax], d[7][ax], d[8][ax]);
-                cap[ax] = typical > 0.0f ? 16.0f * typical : INF;
-            }
-        }
+        if (base == 0)  // (requested together with the first points: one round trip)
+            chamfer_pilot(P, n, pilot, cap);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const float v[3] = {p[u].x, p[u].y, p[u].z};
@@ -2017,42 +2097,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
     if (bad)
         sbad = 1;
     __syncthreads();
-    // The frame: the bounding box, trimmed to three mean deviations around the pilot centre.
-    // A uniform or a Gaussian cloud keeps (nearly) its bounding box - three mean deviations
-    // are 1.5 half extents of the first and 2.4 sigma of the second, and keys up to twice
-    // as far out as the frame are still swept like any other; a few points far away no
-    // longer decide the cells and the scale of everything else - they go on a list of
-    // their own.
-    float cc[3], ext = 0.0f, flo[3];
-#pragma unroll
-    for (int ax = 0; ax < 3; ++ax) {
-        float l = sred[0][ax], h = sred[0][3 + ax], dsum = sdev[0][ax];
-#pragma unroll
-        for (int w = 1; w < NW; ++w) {
-            l = __builtin_fminf(l, sred[w][ax]);
-            h = __builtin_fmaxf(h, sred[w][3 + ax]);
-            dsum += sdev[w][ax];
-        }
-        lo[ax] = l;
-        hi[ax] = h;
-        const float reach = 3.0f * (dsum / (float)n);
-        const float fl = __builtin_fmaxf(l, pilot[ax] - reach);
-        const float fh = __builtin_fminf(h, pilot[ax] + reach);
-        flo[ax] = fl;
-        cc[ax] = 0.5f * fl + 0.5f * fh;
-        ext = __builtin_fmaxf(ext, 0.5f * fh - 0.5f * fl);
-    }
-    if (ext == 0.0f) {
-        // Nearly all points in one place: a frame of no extent would leave the others at
-        // scale 1, possibly far below it, where the fp16 terms have no precision left
-        // (the error bound counts on max|k'| of order 1). The bounding box, then.
-#pragma unroll
-        for (int ax = 0; ax < 3; ++ax) {
-            flo[ax] = lo[ax];
-            cc[ax] = 0.5f * lo[ax] + 0.5f * hi[ax];
-            ext = __builtin_fmaxf(ext, 0.5f * hi[ax] - 0.5f * lo[ax]);
-        }
-    }
+    float cc[3], ext, flo[3];
+    chamfer_frame<NW>(sred, sdev, pilot, n, lo, hi, cc, flo, ext);
     const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
     const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
     const bool safe = n > 0 && sbad == 0 && (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) &&
@@ -2060,6 +2106,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
                       (ext == 0.0f || (ebits >= -40 && ebits <= 40));
     if (tid == 0 && part == 0) {
         a.flags[which * a.B + b] = 0;
+        if (cloud == 0)
+            a.flags[2 * a.B] = 0;
         hdr->c[0] = c0;
         hdr->c[1] = c1;
         hdr->c[2] = c2;
@@ -2116,7 +2164,7 @@ __global__ __launch_bounds__(1024) void chamfer_sort_kernel(ChamferSortArgs a)
     const int which = (int)blockIdx.x >= a.B;
     const int b = (int)blockIdx.x - which * a.B;
     const int n = a.n[which], npad = a.npad[which];
-    if (a.hdr[which * a.B + b].unsafe != 0)  // uniform over the workgroup
+    if (!a.three_launches[which] || a.hdr[which * a.B + b].unsafe != 0)  // uniform
         return;
     const float *__restrict__ P = a.xyz[which] + (int64_t)b * n * 3;
     float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
@@ -2202,6 +2250,8 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
     const int b = lb / bpc;
     const int i = (lb - b * bpc) * 256 + tid;
     ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
+    if (!a.three_launches[which])
+        return;
     if (hdr->unsafe != 0 || i >= npad)  // (uniform over each half wave: npad % 32 == 0)
         return;
     float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
@@ -2248,19 +2298,297 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
         kmax2 = __builtin_fmaxf(kmax2, __shfl_xor(kmax2, o));
     }
     if ((i & 31) == 0) {
-        // fp16 corners, moved outwards by more than the rounding to nearest can bring them
-        // back (2^-11 relative, 2^-25 in the subnormal range); an empty box stays (+inf, -inf)
-        unsigned h[6];
-#pragma unroll
-        for (int ax = 0; ax < 3; ++ax) {
-            const float wl = __builtin_fabsf(bl[ax]) * 9.765625e-4f + 1.1920929e-7f;
-            const float wh = __builtin_fabsf(bh[ax]) * 9.765625e-4f + 1.1920929e-7f;
-            h[ax] = bl[ax] > 3.0e38f ? 0x7c00u : tk_f16_bits(bl[ax] - wl);
-            h[3 + ax] = bh[ax] < -3.0e38f ? 0xfc00u : tk_f16_bits(bh[ax] + wh);
-        }
-        boxes[i >> 5] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), 0u);
+        boxes[i >> 5] = chamfer_box_bits(bl, bh);
         // non-negative floats order as their bit patterns
         atomicMax(&hdr->kmax2_bits, __builtin_bit_cast(int, kmax2));
+    }
+}
+
+// The Hilbert position of every cell of the 32^3 grid, worked out when the library is
+// compiled: the kernel below looks a cell up (one 2-byte load from a 64 KiB table that stays
+// in the L2s) instead of spending 135 instructions on it.
+struct ChamferHilbertTable {
+    unsigned short at[CHAMFER_SORT_CELLS];
+};
+constexpr ChamferHilbertTable chamfer_make_hilbert_table()
+{
+    ChamferHilbertTable t = {};
+    for (unsigned x = 0; x < 32; ++x)
+        for (unsigned y = 0; y < 32; ++y)
+            for (unsigned z = 0; z < 32; ++z)
+                t.at[(x << 10) | (y << 5) | z] = (unsigned short)chamfer_hilbert15(x, y, z);
+    return t;
+}
+__device__ const ChamferHilbertTable chamfer_hilbert_table = chamfer_make_hilbert_table();
+
+// Minimum (MAX: maximum) over each half of the wave, left in lanes 31 and 63: a scan along
+// rows of 16 lanes with row shifts, then row 0's result carried into row 1 (2's into 3).
+template <bool MAX> __device__ __forceinline__ float half_wave_reduce_to_last(float v)
+{
+    auto step = [](float x, float y) { return MAX ? __builtin_fmaxf(x, y) : __builtin_fminf(x, y); };
+    auto dpp = [](float x, auto ctrl, auto rows) {
+        const int i = __builtin_bit_cast(int, x);
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_update_dpp(i, i, decltype(ctrl)::value, decltype(rows)::value,
+                                               0xf, false));
+    };
+    using all = std::integral_constant<int, 0xf>;
+    v = step(v, dpp(v, std::integral_constant<int, 0x111>{}, all{}));  // row_shr:1
+    v = step(v, dpp(v, std::integral_constant<int, 0x112>{}, all{}));  // row_shr:2
+    v = step(v, dpp(v, std::integral_constant<int, 0x114>{}, all{}));  // row_shr:4
+    v = step(v, dpp(v, std::integral_constant<int, 0x118>{}, all{}));  // row_shr:8
+    v = step(v, dpp(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{}));
+    return v;  // (row_bcast:15 into rows 1 and 3)
+}
+
+// Everything the pruned sweep needs of one cloud of up to 16384 points, in one launch: one
+// workgroup of 1024 lanes per cloud reads its points once (16 per lane) and works out
+//   the frame (bounding box, trimmed as in chamfer_cell_kernel), the largest swept |k'|^2 and
+//     the list of keys far outside the frame,
+//   the cells (a table look-up) and their histogram in LDS (two 16-bit counters per word:
+//     64 KiB), the prefix sums and every point's position in sorted order,
+//   and the write-out: sorted positions are taken in windows of PREP_WINDOW points - the lanes
+//     drop the points that belong to the window into LDS, and the workgroup then walks the
+//     window in sorted order, a lane per point, storing the sorted point, its 16 fp16 terms
+//     and, per 32 points, the tile's box, all as runs of consecutive addresses. (Storing each
+//     point at its sorted position straight from the lane that holds it is one cache line per
+//     lane and store: it took 16 of the 23 us of the counting sort that three separate
+//     launches used to run.)
+// Points within a cell land in arbitrary order; nothing depends on it.
+constexpr int PREP_MAX_POINTS = 16384;
+constexpr int PREP_WINDOW = 5632;  // 176 tiles; three windows cover 16384 points
+constexpr size_t PREP_LDS_BYTES =
+    (size_t)(CHAMFER_SORT_CELLS / 2) * sizeof(unsigned) + (size_t)PREP_WINDOW * sizeof(float4);
+
+__global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a, int first_cloud)
+{
+    constexpr int NT = 1024, NW = NT / TK_WAVE, U = PREP_MAX_POINTS / NT, W = PREP_WINDOW;
+    constexpr int WORDS = CHAMFER_SORT_CELLS / 2;
+    extern __shared__ __align__(16) unsigned prep_lds[];
+    unsigned *const hist = prep_lds;                                  // WORDS packed counters
+    float4 *const win = reinterpret_cast<float4 *>(prep_lds + WORDS);  // W sorted points
+    __shared__ float sred[NW][8];
+    __shared__ float sdev[NW][4];
+    __shared__ int swave[NW];
+    __shared__ int sstart[NW];
+    __shared__ float4 sfar_list[CHAMFER_FAR_KEYS];
+    __shared__ int sbad, sfar;
+    const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
+    const int cloud = first_cloud + (int)blockIdx.x;
+    const int which = cloud >= a.B;
+    const int b = cloud - which * a.B;
+    const int n = a.n[which], npad = a.npad[which];
+    const float *__restrict__ P = a.xyz[which] + (int64_t)b * n * 3;
+    ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
+    const float INF = __builtin_huge_valf();
+
+    // ---- the points (once), the pilot centre, the bounding box and the deviations ----
+    TkPoint3<float> p[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int j = u * NT + tid;
+        p[u] = tk_load3<float>(P + (int64_t)(j < n ? j : n - 1) * 3);
+    }
+    float pilot[3], cap[3];
+    chamfer_pilot(P, n, pilot, cap);
+    for (int i = tid; i < WORDS; i += NT)
+        hist[i] = 0u;
+    float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    float dev[3] = {0.0f, 0.0f, 0.0f};
+    bool bad = false;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float v[3] = {p[u].x, p[u].y, p[u].z};
+        const bool counts = u * NT + tid < n;
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            bad |= !(v[ax] - v[ax] == 0.0f);
+            lo[ax] = __builtin_fminf(lo[ax], v[ax]);
+            hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
+            dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        lo[ax] = wave_reduce_min(lo[ax]);
+        hi[ax] = wave_reduce_max(hi[ax]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            dev[ax] += __shfl_xor(dev[ax], o);
+    }
+    if (tid == 0) {
+        sbad = 0;
+        sfar = 0;
+    }
+    __syncthreads();
+    if (lane == 0) {
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            sred[wave][ax] = lo[ax];
+            sred[wave][3 + ax] = hi[ax];
+            sdev[wave][ax] = dev[ax];
+        }
+    }
+    if (bad)
+        sbad = 1;
+    __syncthreads();
+    float cc[3], flo[3], ext;
+    chamfer_frame<NW>(sred, sdev, pilot, n, lo, hi, cc, flo, ext);
+    const float c0 = cc[0], c1 = cc[1], c2 = cc[2];
+    const int ebits = (int)((__builtin_bit_cast(unsigned, ext) >> 23) & 0xffu) - 127;
+    const bool safe = n > 0 && sbad == 0 && (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) &&
+                      (c2 - c2 == 0.0f) && (ext - ext == 0.0f) &&
+                      (ext == 0.0f || (ebits >= -40 && ebits <= 40));
+    const float scale =
+        ext == 0.0f ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
+    if (tid == 0) {
+        a.flags[which * a.B + b] = 0;
+        if (cloud == 0)
+            a.flags[2 * a.B] = 0;
+        hdr->c[0] = c0;
+        hdr->c[1] = c1;
+        hdr->c[2] = c2;
+        hdr->scale = scale;
+        hdr->unsafe = safe ? 0 : 1;
+        hdr->extent = 2.0f * ext;
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            hdr->lo[ax] = lo[ax];
+            hdr->hi[ax] = hi[ax];
+        }
+        if (!safe) {
+            hdr->kmax2_bits = 0;
+            hdr->far_keys = 0;
+        }
+    }
+    if (!safe)  // uniform over the workgroup
+        return;
+
+    // ---- cells and their histogram; the far keys and the largest swept |k'|^2 ----
+    const float inv = ext > 0.0f ? (16.0f / ext) * 0.99999f : 0.0f;
+    int cell[U];  // later: the point's position in sorted order
+    float kmax2 = 0.0f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float ux = __builtin_fminf(__builtin_fmaxf((p[u].x - flo[0]) * inv, 0.0f), 31.0f);
+        const float uy = __builtin_fminf(__builtin_fmaxf((p[u].y - flo[1]) * inv, 0.0f), 31.0f);
+        const float uz = __builtin_fminf(__builtin_fmaxf((p[u].z - flo[2]) * inv, 0.0f), 31.0f);
+        cell[u] = chamfer_hilbert_table.at[((int)ux << 10) | ((int)uy << 5) | (int)uz];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int j = u * NT + tid;
+        const float x = (p[u].x - c0) * scale, y = (p[u].y - c1) * scale, z = (p[u].z - c2) * scale;
+        const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+        // (a key beyond 4 units of the frame: see chamfer_tile_kernel)
+        const bool far = j < n && !(nn <= 16.0f);
+        if (far) {
+            const int slot = atomicAdd(&sfar, 1);
+            if (slot < CHAMFER_FAR_KEYS)
+                sfar_list[slot] = make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, j));
+        }
+        kmax2 = __builtin_fmaxf(kmax2, (j < n && !far) ? nn : 0.0f);
+        if (j < n)
+            atomicAdd(&hist[cell[u] >> 1], 1u << ((cell[u] & 1) * 16));
+    }
+    kmax2 = wave_reduce_max(kmax2);
+    __syncthreads();
+    if (lane == 0)
+        sred[wave][0] = kmax2;
+    // Every wave turns the 2048 counters of its range into starting positions within the
+    // range (at most 16384: they fit the 16 bits, and so does every position taken below);
+    // the ranges' own starts are added when a position is taken.
+    {
+        constexpr int PER_WAVE = WORDS / NW;
+        int carry = 0;
+        for (int i = 0; i < PER_WAVE; i += TK_WAVE) {
+            const int at = wave * PER_WAVE + i + lane;
+            const unsigned both = hist[at];
+            const int even = (int)(both & 0xffffu), odd = (int)(both >> 16);
+            const int incl = wave_inclusive_sum(even + odd);
+            const int start = carry + incl - (even + odd);
+            hist[at] = (unsigned)start | ((unsigned)(start + even) << 16);
+            carry += __builtin_amdgcn_readlane(incl, TK_WAVE - 1);
+        }
+        if (lane == 0)
+            swave[wave] = carry;
+    }
+    __syncthreads();
+    if (tid < NW) {
+        int run = 0;
+        for (int w = 0; w < tid; ++w)
+            run += swave[w];
+        sstart[tid] = run;
+    }
+    {  // what belongs to the cloud as a whole
+        const int nfar = sfar;
+        if (tid == 0) {
+            float m = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                m = __builtin_fmaxf(m, sred[w][0]);
+            hdr->kmax2_bits = __builtin_bit_cast(int, m);
+            hdr->far_keys = nfar;
+        }
+        if (tid < nfar && tid < CHAMFER_FAR_KEYS)
+            a.far_keys[which][(int64_t)b * CHAMFER_FAR_KEYS + tid] = sfar_list[tid];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int shift = (cell[u] & 1) * 16;
+        int pos = -1;
+        if (u * NT + tid < n)
+            pos = (int)((atomicAdd(&hist[cell[u] >> 1], 1u << shift) >> shift) & 0xffffu) +
+                  sstart[cell[u] >> 11];
+        cell[u] = pos;
+    }
+
+    // ---- write-out in windows of sorted positions ----
+    float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
+    uint4 *__restrict__ terms = a.terms[which] + (int64_t)b * npad * 2;
+    uint4 *__restrict__ boxes = a.boxes[which] + (int64_t)b * (npad / 32);
+    const float qnan = __builtin_nanf("");
+    for (int base = 0; base < npad; base += W) {
+        const int width = npad - base < W ? npad - base : W;
+        if (base > 0)
+            __syncthreads();  // the window's previous contents have been read
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned at = (unsigned)(cell[u] - base);  // (a lane past the end holds -1)
+            if (at < (unsigned)width && cell[u] >= 0)
+                win[at] = make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, u * NT + tid));
+        }
+        __syncthreads();
+        for (int s0 = 0; s0 < width; s0 += NT) {
+            const int i = base + s0 + tid;
+            if (s0 + tid >= width)  // (uniform over each half wave: width is a multiple of 32)
+                continue;
+            const bool exists = i < n;
+            float4 s = make_float4(qnan, qnan, qnan, __builtin_bit_cast(float, -1));
+            if (exists)
+                s = win[s0 + tid];
+            sorted[i] = s;
+            const float x = ((exists ? s.x : c0) - c0) * scale;
+            const float y = ((exists ? s.y : c1) - c1) * scale;
+            const float z = ((exists ? s.z : c2) - c2) * scale;
+            const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+            const bool swept = exists && nn <= 16.0f;
+            uint4 h0, h1;
+            chamfer_key_terms(x, y, z, nn, swept, h0, h1);
+            uint4 *tile = terms + (i >> 5) * 64 + (i & 31);
+            tile[0] = h0;
+            tile[32] = h1;
+            float bl[3], bh[3];
+            bl[0] = half_wave_reduce_to_last<false>(swept ? x : INF);
+            bl[1] = half_wave_reduce_to_last<false>(swept ? y : INF);
+            bl[2] = half_wave_reduce_to_last<false>(swept ? z : INF);
+            bh[0] = half_wave_reduce_to_last<true>(swept ? x : -INF);
+            bh[1] = half_wave_reduce_to_last<true>(swept ? y : -INF);
+            bh[2] = half_wave_reduce_to_last<true>(swept ? z : -INF);
+            if ((i & 31) == 31)
+                boxes[i >> 5] = chamfer_box_bits(bl, bh);
+        }
     }
 }
 
@@ -2307,18 +2635,25 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         if (lb < full)
             lb = (lb & 7) * per + (lb >> 3);
     }
-    int wid = __builtin_amdgcn_readfirstlane(lb + tid / TK_WAVE);
-    const int which = wid >= a.waves0;
-    if (which)
-        wid -= a.waves0;
-    const int wpc = a.waves_per_cloud[which];
-    if (wid >= a.B * wpc)
+    // A batch element's two directions follow each other, so that the XCD whose L2 holds its
+    // two sorted clouds serves both.
+    const int wid = __builtin_amdgcn_readfirstlane(lb + tid / TK_WAVE);
+    const int wpb = a.waves_per_cloud[0] + a.waves_per_cloud[1];
+    const int b = wid / wpb;
+    if (b >= a.B)
         return;
-    const int b = wid / wpc, qw = wid - b * wpc;
+    const int within = wid - b * wpb;
+    const int which = within >= a.waves_per_cloud[0];
+    const int qw = within - (which ? a.waves_per_cloud[0] : 0);
     const int nq = a.n[which], npq = a.npad[which], npk = a.npad[1 - which];
     const ChamferSortedHdr *hq = a.hdr + which * a.B + b;
     const ChamferSortedHdr *hk = a.hdr + (1 - which) * a.B + b;
     int *flag = a.flags + which * a.B + b;
+    // this cloud and direction goes to the sweep of all pairs (one word says that any does)
+    auto hand_over = [&]() {
+        atomicOr(flag, 1);
+        atomicOr(a.flags + 2 * a.B, 1);
+    };
     const float4 *__restrict__ SQ = a.sorted[which] + (int64_t)b * npq;
     const float4 *__restrict__ SK = a.sorted[1 - which] + (int64_t)b * npk;
     const uint4 *__restrict__ TK = a.terms[1 - which] + (int64_t)b * npk * 2;
@@ -2361,7 +2696,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const int nfar = hk->far_keys;  // keys kept out of the sweep (far outside the frame)
     if (hq->unsafe != 0 || hk->unsafe != 0) {  // uniform over the wave
         if (lane == 0)
-            atomicOr(flag, 1);
+            hand_over();
         return;
     }
     if (hk->lo[0] == hk->hi[0] && hk->lo[1] == hk->hi[1] && hk->lo[2] == hk->hi[2]) {
@@ -2386,7 +2721,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     const bool flat_terms = hk->kmax2_bits < 0x3d800000;  // |k'|^2 < 1/16 for every swept key
     if (!(far2 <= 6.4e7f) || dwarfed || flat_terms || nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
         if (lane == 0)
-            atomicOr(flag, 1);
+            hand_over();
         return;
     }
     if (handed_over != 0)
@@ -2452,7 +2787,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // (query, tile) pairs of it per wave and the cloud is handed over.
     if ((int64_t)nstray * ntiles > 16384) {
         if (lane == 0)
-            atomicOr(flag, 1);
+            hand_over();
         return;
     }
 #pragma unroll
@@ -2549,7 +2884,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
                     __builtin_amdgcn_ballot_w64(best == least && at >= 0);
                 if (m == 0) {  // no key tile holds a point (cannot happen with nk >= 1)
                     if (lane == 0)
-                        atomicOr(flag, 1);
+                        hand_over();
                     return;
                 }
                 const int t = __builtin_amdgcn_readlane(at, (int)__builtin_ctzll(m));
@@ -2681,7 +3016,7 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // quantised or duplicated points).
     if ((int64_t)nover * nswept > 8192) {
         if (lane == 0)
-            atomicOr(flag, 1);
+            hand_over();
         return;
     }
     // ---- queries with three or more candidate tiles: exact scan of the swept tiles;
@@ -2787,7 +3122,7 @@ inline ChamferSortedLayout chamfer_sorted_layout(int64_t B, int64_t N1, int64_t 
         return here;
     };
     l.hdr = take((size_t)2 * B * sizeof(ChamferSortedHdr));
-    l.flags = take((size_t)2 * B * sizeof(int));
+    l.flags = take((size_t)(2 * B + 1) * sizeof(int));
     for (int w = 0; w < 2; ++w) {
         l.npad[w] = (n[w] + 127) / 128 * 128;
         l.sorted[w] = take((size_t)B * l.npad[w] * sizeof(float4));
@@ -2867,12 +3202,31 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
     if (allowed != TK3D_OK)
         return allowed;
     if (stages & 1) {
-        hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
-                           dim3(1024), 0, s, sa);
-        hipLaunchKernelGGL(chamfer_sort_kernel, dim3((unsigned)(2 * B)), dim3(1024), lds, s, sa);
-        const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
-        hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s, sa,
-                           (int)tb0);
+        // clouds of up to 16384 points: one launch; longer ones: cell, sort and tile kernels
+        int first = 2 * (int)B, count = 0;
+        for (int w = 1; w >= 0; --w) {
+            sa.three_launches[w] = n[w] > PREP_MAX_POINTS;
+            if (!sa.three_launches[w]) {
+                first = w * (int)B;
+                count += (int)B;
+            }
+        }
+        // (both clouds short: first = 0, count = 2 B; one: its own B clouds)
+        if (count > 0) {
+            const int ok = tk_allow_dynamic_lds<chamfer_prepare_kernel>((int)PREP_LDS_BYTES);
+            if (ok != TK3D_OK)
+                return ok;
+            hipLaunchKernelGGL(chamfer_prepare_kernel, dim3((unsigned)count), dim3(1024),
+                               PREP_LDS_BYTES, s, sa, first);
+        }
+        if (sa.three_launches[0] || sa.three_launches[1]) {
+            hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
+                               dim3(1024), 0, s, sa);
+            hipLaunchKernelGGL(chamfer_sort_kernel, dim3((unsigned)(2 * B)), dim3(1024), lds, s, sa);
+            const int64_t tb0 = B * ((l.npad[0] + 255) / 256), tb1 = B * ((l.npad[1] + 255) / 256);
+            hipLaunchKernelGGL(chamfer_tile_kernel, dim3((unsigned)(tb0 + tb1)), dim3(256), 0, s,
+                               sa, (int)tb0);
+        }
     }
     const dim3 grid((unsigned)((waves0 + waves1)));
     const bool small = l.npad[0] <= 16384 && l.npad[1] <= 16384;
