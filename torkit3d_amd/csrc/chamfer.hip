@@ -260,19 +260,37 @@ __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T
 // exact sweep for the whole workgroup or the exact scan for the query.
 // Results are therefore bit-identical to the exact sweep for every input.
 
+// Minimum / maximum over the wave, the same value in every lane (NaNs are passed over, as
+// fminf / fmaxf do). A scan along rows of 16 lanes with row shifts, the rows' results carried
+// on with row broadcasts, the total read from lane 63: six short steps on the vector ALU where
+// six exchanges through the LDS crossbar (ds_bpermute) took a hundred clocks each.
+template <bool MAX> __device__ __forceinline__ float wave_reduce_extreme(float v)
+{
+#define TK_WAVE_STEP(ctrl, rows)                                                              \
+    {                                                                                         \
+        const float o = __builtin_bit_cast(                                                   \
+            float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),                    \
+                                               __builtin_bit_cast(int, v), ctrl, rows, 0xf,   \
+                                               false));                                       \
+        v = MAX ? __builtin_fmaxf(v, o) : __builtin_fminf(v, o);                              \
+    }
+    TK_WAVE_STEP(0x111, 0xf)  // row_shr:1
+    TK_WAVE_STEP(0x112, 0xf)  // row_shr:2
+    TK_WAVE_STEP(0x114, 0xf)  // row_shr:4
+    TK_WAVE_STEP(0x118, 0xf)  // row_shr:8
+    TK_WAVE_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+    TK_WAVE_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef TK_WAVE_STEP
+    return __builtin_bit_cast(float,
+                              __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), TK_WAVE - 1));
+}
 __device__ __forceinline__ float wave_reduce_min(float v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1)
-        v = __builtin_fminf(v, __shfl_xor(v, o));
-    return v;
+    return wave_reduce_extreme<false>(v);
 }
 __device__ __forceinline__ float wave_reduce_max(float v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1)
-        v = __builtin_fmaxf(v, __shfl_xor(v, o));
-    return v;
+    return wave_reduce_extreme<true>(v);
 }
 
 // Exact nearest neighbour of one query, the whole workgroup cooperating: lane t scans
@@ -2069,8 +2087,8 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
 #pragma unroll
             for (int ax = 0; ax < 3; ++ax) {
                 bad |= !(v[ax] - v[ax] == 0.0f);
-                lo[ax] = __builtin_fminf(lo[ax], v[ax]);
-                hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
+                lo[ax] = __builtin_fminf(lo[ax], counts ? v[ax] : INF);
+                hi[ax] = __builtin_fmaxf(hi[ax], counts ? v[ax] : -INF);
                 dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
             }
         }
@@ -2321,60 +2339,84 @@ constexpr ChamferHilbertTable chamfer_make_hilbert_table()
 }
 __device__ const ChamferHilbertTable chamfer_hilbert_table = chamfer_make_hilbert_table();
 
-// Minimum (MAX: maximum) over each half of the wave, left in lanes 31 and 63: a scan along
-// rows of 16 lanes with row shifts, then row 0's result carried into row 1 (2's into 3).
-template <bool MAX> __device__ __forceinline__ float half_wave_reduce_to_last(float v)
+// Floats as signed integers that order the same way (an involution; -0 sorts below +0).
+__device__ __forceinline__ int tk_float_order(float x)
 {
-    auto step = [](float x, float y) { return MAX ? __builtin_fmaxf(x, y) : __builtin_fminf(x, y); };
-    auto dpp = [](float x, auto ctrl, auto rows) {
-        const int i = __builtin_bit_cast(int, x);
-        return __builtin_bit_cast(
-            float, __builtin_amdgcn_update_dpp(i, i, decltype(ctrl)::value, decltype(rows)::value,
-                                               0xf, false));
-    };
-    using all = std::integral_constant<int, 0xf>;
-    v = step(v, dpp(v, std::integral_constant<int, 0x111>{}, all{}));  // row_shr:1
-    v = step(v, dpp(v, std::integral_constant<int, 0x112>{}, all{}));  // row_shr:2
-    v = step(v, dpp(v, std::integral_constant<int, 0x114>{}, all{}));  // row_shr:4
-    v = step(v, dpp(v, std::integral_constant<int, 0x118>{}, all{}));  // row_shr:8
-    v = step(v, dpp(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{}));
-    return v;  // (row_bcast:15 into rows 1 and 3)
+    const int i = __builtin_bit_cast(int, x);
+    return i ^ ((i >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ float tk_order_float(int i)
+{
+    return __builtin_bit_cast(float, i ^ ((i >> 31) & 0x7fffffff));
 }
 
-// Everything the pruned sweep needs of one cloud of up to 16384 points, in one launch: one
-// workgroup of 1024 lanes per cloud reads its points once (16 per lane) and works out
+// Minimum (MAX: maximum) over each half of the wave, left in lanes 31 and 63: a scan along
+// rows of 16 lanes with row shifts, then row 0's result carried into row 1 (2's into 3).
+// On integers: a floating-point minimum quiets its operands first, one more instruction per
+// step and operand (57 of the 271 instructions a sorted point cost went there).
+template <bool MAX> __device__ __forceinline__ int half_wave_reduce_to_last(int v)
+{
+#define TK_HALF_WAVE_STEP(ctrl, rows)                                                  \
+    {                                                                                  \
+        const int o = __builtin_amdgcn_update_dpp(v, v, ctrl, rows, 0xf, false);       \
+        v = MAX ? (o > v ? o : v) : (o < v ? o : v);                                   \
+    }
+    TK_HALF_WAVE_STEP(0x111, 0xf)  // row_shr:1
+    TK_HALF_WAVE_STEP(0x112, 0xf)  // row_shr:2
+    TK_HALF_WAVE_STEP(0x114, 0xf)  // row_shr:4
+    TK_HALF_WAVE_STEP(0x118, 0xf)  // row_shr:8
+    TK_HALF_WAVE_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+#undef TK_HALF_WAVE_STEP
+    return v;
+}
+
+// Everything the pruned sweep needs of one cloud of up to 16384 points, in one launch.
+// `parts` workgroups of 1024 lanes (16 points per lane) serve a cloud. Each works out, for
+// itself, what needs the whole cloud:
 //   the frame (bounding box, trimmed as in chamfer_cell_kernel), the largest swept |k'|^2 and
 //     the list of keys far outside the frame,
-//   the cells (a table look-up) and their histogram in LDS (two 16-bit counters per word:
-//     64 KiB), the prefix sums and every point's position in sorted order,
-//   and the write-out: sorted positions are taken in windows of PREP_WINDOW points - the lanes
-//     drop the points that belong to the window into LDS, and the workgroup then walks the
-//     window in sorted order, a lane per point, storing the sorted point, its 16 fp16 terms
-//     and, per 32 points, the tile's box, all as runs of consecutive addresses. (Storing each
-//     point at its sorted position straight from the lane that holds it is one cache line per
-//     lane and store: it took 16 of the 23 us of the counting sort that three separate
-//     launches used to run.)
-// Points within a cell land in arbitrary order; nothing depends on it.
+//   the cells (a table look-up), their histogram in LDS (two 16-bit counters per word:
+//     64 KiB; the atomic that counts a point also hands it its rank within the cell) and the
+//     prefix sums, hence every point's position in sorted order.
+// The write-out is divided by cells: the sixteen ranges of 2048 cells are dealt to the parts
+// in runs of about equal numbers of points, and a part writes the sorted positions of its own
+// cells (the rank within a cell is whatever order the part's own atomics arrived in, so two
+// parts must not share a cell). It takes its positions in windows of PREP_WINDOW - the lanes
+// drop the points that belong to the window into LDS, and the workgroup then walks the window
+// in sorted order, a lane per point, storing the sorted point, its 16 fp16 terms and, per 32
+// points, the tile's box, all as runs of consecutive addresses. (Storing each point at its
+// sorted position straight from the lane that holds it is one cache line per lane and store:
+// it took 16 of the 23 us of the counting sort that three separate launches used to run.)
+// A tile of 32 positions that two parts share gets its box from the part that owns its first
+// position: exact for that part's points, and for the rest the box of every point of the
+// later cells that begin inside the tile - a superset of the tile's points, which is all a
+// box has to be. What every part repeats is about a third of the work of a cloud, and no
+// workgroup waits for another.
 constexpr int PREP_MAX_POINTS = 16384;
-constexpr int PREP_WINDOW = 5632;  // 176 tiles; three windows cover 16384 points
-constexpr size_t PREP_LDS_BYTES =
-    (size_t)(CHAMFER_SORT_CELLS / 2) * sizeof(unsigned) + (size_t)PREP_WINDOW * sizeof(float4);
+constexpr int PREP_WINDOW = 5600;  // 175 tiles; three windows cover 16384 points
+constexpr size_t PREP_LDS_BYTES = (size_t)(CHAMFER_SORT_CELLS / 2) * sizeof(unsigned) +
+                                  (size_t)(PREP_WINDOW + TK_WAVE) * sizeof(float4);
 
-__global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a, int first_cloud)
+__global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a, int first_cloud,
+                                                               int parts)
 {
     constexpr int NT = 1024, NW = NT / TK_WAVE, U = PREP_MAX_POINTS / NT, W = PREP_WINDOW;
     constexpr int WORDS = CHAMFER_SORT_CELLS / 2;
+    constexpr int ORDER_POS_INF = 0x7f800000, ORDER_NEG_INF = (int)0x807fffffu;
     extern __shared__ __align__(16) unsigned prep_lds[];
     unsigned *const hist = prep_lds;                                  // WORDS packed counters
-    float4 *const win = reinterpret_cast<float4 *>(prep_lds + WORDS);  // W sorted points
+    float4 *const win = reinterpret_cast<float4 *>(prep_lds + WORDS);  // W sorted points, then
+                                                                       // a spare slot per lane
     __shared__ float sred[NW][8];
     __shared__ float sdev[NW][4];
     __shared__ int swave[NW];
-    __shared__ int sstart[NW];
+    __shared__ int sstart[NW + 1];
     __shared__ float4 sfar_list[CHAMFER_FAR_KEYS];
     __shared__ int sbad, sfar;
+    __shared__ int sextra[8];  // box of the later parts' points in this part's last tile
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
-    const int cloud = first_cloud + (int)blockIdx.x;
+    const int cloud = first_cloud + (int)blockIdx.x / parts;
+    const int part = (int)blockIdx.x % parts;
     const int which = cloud >= a.B;
     const int b = cloud - which * a.B;
     const int n = a.n[which], npad = a.npad[which];
@@ -2382,30 +2424,58 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     ChamferSortedHdr *hdr = a.hdr + which * a.B + b;
     const float INF = __builtin_huge_valf();
 
-    // ---- the points (once), the pilot centre, the bounding box and the deviations ----
-    TkPoint3<float> p[U];
+    // The lane's 16 points, all loads in flight together. Each pass below asks for them anew
+    // (after the first they come from the L2) rather than holding 48 registers across the
+    // kernel, and through a buffer descriptor: one 32-bit offset per point against a base in
+    // scalar registers (a lane past the end of the cloud reads the last point again). With
+    // sixteen 64-bit addresses, the same in every pass, the compiler kept the addresses alive
+    // across the kernel and spilled them, and a spilled address is a round trip to memory in
+    // front of its load.
+    const __amdgpu_buffer_rsrc_t cloud_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P), 0, n * 12, 0x00020000);
+    auto load_points = [&](TkPoint3<float>(&p)[U]) {
+        // (the lane number is made opaque per pass, or the compiler merges the passes' loads
+        // into one set of 48 registers that lives across the kernel)
+        int t = tid;
+        asm volatile("" : "+v"(t));
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int j = u * NT + tid;
-        p[u] = tk_load3<float>(P + (int64_t)(j < n ? j : n - 1) * 3);
-    }
+        for (int u = 0; u < U; ++u) {
+            typedef float f3 __attribute__((ext_vector_type(3)));
+            const int j = u * NT + t;
+            const f3 v = __builtin_bit_cast(
+                f3, __builtin_amdgcn_raw_buffer_load_b96(cloud_rsrc, (j < n ? j : n - 1) * 12, 0, 0));
+            p[u].x = v.x;
+            p[u].y = v.y;
+            p[u].z = v.z;
+        }
+    };
+
+    // ---- the pilot centre, the bounding box and the deviations ----
     float pilot[3], cap[3];
     chamfer_pilot(P, n, pilot, cap);
     for (int i = tid; i < WORDS; i += NT)
         hist[i] = 0u;
+    if (tid < 8)
+        sextra[tid] = tid < 3 ? ORDER_POS_INF : ORDER_NEG_INF;
+    __builtin_amdgcn_sched_barrier(0);  // (the pilot's nine points and the lane's sixteen at
+                                        // once do not fit the registers)
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
     float dev[3] = {0.0f, 0.0f, 0.0f};
     bool bad = false;
+    {
+        TkPoint3<float> p[U];
+        load_points(p);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const float v[3] = {p[u].x, p[u].y, p[u].z};
-        const bool counts = u * NT + tid < n;
+        for (int u = 0; u < U; ++u) {
+            const float v[3] = {p[u].x, p[u].y, p[u].z};
+            const bool counts = u * NT + tid < n;
 #pragma unroll
-        for (int ax = 0; ax < 3; ++ax) {
-            bad |= !(v[ax] - v[ax] == 0.0f);
-            lo[ax] = __builtin_fminf(lo[ax], v[ax]);
-            hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
-            dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
+            for (int ax = 0; ax < 3; ++ax) {
+                bad |= !(v[ax] - v[ax] == 0.0f);
+                lo[ax] = __builtin_fminf(lo[ax], v[ax]);
+                hi[ax] = __builtin_fmaxf(hi[ax], v[ax]);
+                dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
+            }
         }
     }
 #pragma unroll
@@ -2441,7 +2511,7 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
                       (ext == 0.0f || (ebits >= -40 && ebits <= 40));
     const float scale =
         ext == 0.0f ? 1.0f : __builtin_bit_cast(float, (unsigned)(127 - ebits) << 23);
-    if (tid == 0) {
+    if (tid == 0 && part == 0) {
         a.flags[which * a.B + b] = 0;
         if (cloud == 0)
             a.flags[2 * a.B] = 0;
@@ -2464,40 +2534,53 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     if (!safe)  // uniform over the workgroup
         return;
 
-    // ---- cells and their histogram; the far keys and the largest swept |k'|^2 ----
+    // ---- cells, their histogram and the points' ranks within their cells; the far keys
+    //      and the largest swept |k'|^2 ----
     const float inv = ext > 0.0f ? (16.0f / ext) * 0.99999f : 0.0f;
-    int cell[U];  // later: the point's position in sorted order
+    int where[U];  // cell | rank << 15; later the position in sorted order; -1: no point
     float kmax2 = 0.0f;
+    {
+        TkPoint3<float> p[U];
+        load_points(p);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const float ux = __builtin_fminf(__builtin_fmaxf((p[u].x - flo[0]) * inv, 0.0f), 31.0f);
-        const float uy = __builtin_fminf(__builtin_fmaxf((p[u].y - flo[1]) * inv, 0.0f), 31.0f);
-        const float uz = __builtin_fminf(__builtin_fmaxf((p[u].z - flo[2]) * inv, 0.0f), 31.0f);
-        cell[u] = chamfer_hilbert_table.at[((int)ux << 10) | ((int)uy << 5) | (int)uz];
+        for (int u = 0; u < U; ++u) {
+            const float ux = __builtin_fminf(__builtin_fmaxf((p[u].x - flo[0]) * inv, 0.0f), 31.0f);
+            const float uy = __builtin_fminf(__builtin_fmaxf((p[u].y - flo[1]) * inv, 0.0f), 31.0f);
+            const float uz = __builtin_fminf(__builtin_fmaxf((p[u].z - flo[2]) * inv, 0.0f), 31.0f);
+            where[u] = chamfer_hilbert_table.at[((int)ux << 10) | ((int)uy << 5) | (int)uz];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = u * NT + tid;
+            const float x = (p[u].x - c0) * scale, y = (p[u].y - c1) * scale,
+                        z = (p[u].z - c2) * scale;
+            const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
+            // (a key beyond 4 units of the frame: see chamfer_tile_kernel)
+            const bool far = j < n && !(nn <= 16.0f);
+            if (far) {
+                const int slot = atomicAdd(&sfar, 1);
+                if (slot < CHAMFER_FAR_KEYS)
+                    sfar_list[slot] =
+                        make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, j));
+            }
+            kmax2 = __builtin_fmaxf(kmax2, (j < n && !far) ? nn : 0.0f);
+        }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int j = u * NT + tid;
-        const float x = (p[u].x - c0) * scale, y = (p[u].y - c1) * scale, z = (p[u].z - c2) * scale;
-        const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
-        // (a key beyond 4 units of the frame: see chamfer_tile_kernel)
-        const bool far = j < n && !(nn <= 16.0f);
-        if (far) {
-            const int slot = atomicAdd(&sfar, 1);
-            if (slot < CHAMFER_FAR_KEYS)
-                sfar_list[slot] = make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, j));
-        }
-        kmax2 = __builtin_fmaxf(kmax2, (j < n && !far) ? nn : 0.0f);
-        if (j < n)
-            atomicAdd(&hist[cell[u] >> 1], 1u << ((cell[u] & 1) * 16));
+        const int cell = where[u], shift = (cell & 1) * 16;
+        int packed = -1;
+        if (u * NT + tid < n)
+            packed = cell | (int)(((atomicAdd(&hist[cell >> 1], 1u << shift) >> shift) & 0xffffu) << 15);
+        where[u] = packed;
     }
     kmax2 = wave_reduce_max(kmax2);
     __syncthreads();
     if (lane == 0)
         sred[wave][0] = kmax2;
     // Every wave turns the 2048 counters of its range into starting positions within the
-    // range (at most 16384: they fit the 16 bits, and so does every position taken below);
-    // the ranges' own starts are added when a position is taken.
+    // range (at most 16384: they fit the 16 bits); the ranges' own starts are added when a
+    // position is looked up.
     {
         constexpr int PER_WAVE = WORDS / NW;
         int carry = 0;
@@ -2514,13 +2597,13 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
             swave[wave] = carry;
     }
     __syncthreads();
-    if (tid < NW) {
+    if (tid <= NW) {
         int run = 0;
         for (int w = 0; w < tid; ++w)
             run += swave[w];
-        sstart[tid] = run;
+        sstart[tid] = run;  // (sstart[NW] = n)
     }
-    {  // what belongs to the cloud as a whole
+    if (part == 0) {  // what belongs to the cloud as a whole leaves with its first workgroup
         const int nfar = sfar;
         if (tid == 0) {
             float m = 0.0f;
@@ -2534,60 +2617,125 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
             a.far_keys[which][(int64_t)b * CHAMFER_FAR_KEYS + tid] = sfar_list[tid];
     }
     __syncthreads();
+    // This part's run of cell ranges [r_lo, r_hi) and of sorted positions [s_lo, s_hi): range
+    // boundary q is the first range that starts at or beyond q / parts of the points.
+    int r_lo = 0, r_hi = NW;
+    if (part > 0 || part + 1 < parts) {
+        const int want_lo = (int)(((int64_t)n * part) / parts);
+        const int want_hi = (int)(((int64_t)n * (part + 1)) / parts);
+        int first_lo = NW, first_hi = NW;
+        for (int w = NW - 1; w >= 0; --w) {
+            const int at = sstart[w];
+            first_lo = at >= want_lo ? w : first_lo;
+            first_hi = at >= want_hi ? w : first_hi;
+        }
+        r_lo = part > 0 ? first_lo : 0;
+        r_hi = part + 1 < parts ? first_hi : NW;
+    }
+    const bool last = part + 1 == parts;
+    const int s_lo = sstart[r_lo], s_hi = sstart[r_hi];
+    // the part's last tile is shared with later parts when its positions end inside a tile
+    const int shared_end = (!last && (s_hi & 31) != 0 && s_hi > s_lo) ? ((s_hi + 31) & ~31) : -1;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int shift = (cell[u] & 1) * 16;
-        int pos = -1;
-        if (u * NT + tid < n)
-            pos = (int)((atomicAdd(&hist[cell[u] >> 1], 1u << shift) >> shift) & 0xffffu) +
-                  sstart[cell[u] >> 11];
-        cell[u] = pos;
+        const int cell = where[u] & 0x7fff, rank = where[u] >> 15;
+        const unsigned both = hist[cell >> 1];
+        const int start = (int)((cell & 1) ? both >> 16 : both & 0xffffu) + sstart[cell >> 11];
+        // bit 20: a point of a later part whose cell begins inside this part's last tile
+        const int later = ((cell >> 11) >= r_hi && start < shared_end) ? 1 << 20 : 0;
+        where[u] = where[u] < 0 ? -1 : ((start + rank) | later);
     }
 
-    // ---- write-out in windows of sorted positions ----
+    // ---- write-out of the part's positions, in windows ----
     float4 *__restrict__ sorted = a.sorted[which] + (int64_t)b * npad;
     uint4 *__restrict__ terms = a.terms[which] + (int64_t)b * npad * 2;
     uint4 *__restrict__ boxes = a.boxes[which] + (int64_t)b * (npad / 32);
     const float qnan = __builtin_nanf("");
-    for (int base = 0; base < npad; base += W) {
-        const int width = npad - base < W ? npad - base : W;
-        if (base > 0)
-            __syncthreads();  // the window's previous contents have been read
+    const int t_lo = s_lo & ~31, t_hi = last ? npad : ((s_hi + 31) & ~31);
+    for (int base = t_lo; base < t_hi; base += W) {
+        const int width = t_hi - base < W ? t_hi - base : W;
+        {
+            TkPoint3<float> p[U];
+            load_points(p);
+            if (base > t_lo)
+                __syncthreads();  // the window's previous contents have been read
+            int extra_lo[3] = {ORDER_POS_INF, ORDER_POS_INF, ORDER_POS_INF};
+            int extra_hi[3] = {ORDER_NEG_INF, ORDER_NEG_INF, ORDER_NEG_INF};
+            bool any_extra = false;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const unsigned at = (unsigned)(cell[u] - base);  // (a lane past the end holds -1)
-            if (at < (unsigned)width && cell[u] >= 0)
-                win[at] = make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, u * NT + tid));
+            for (int u = 0; u < U; ++u) {
+                const int pos = where[u] & 0xfffff;
+                const bool mine = where[u] >= 0 && pos >= s_lo && pos < s_hi;
+                const unsigned at = (unsigned)(pos - base);
+                // (a point of another window or another part goes to the lane's spare slot:
+                // a store that is skipped costs a branch per point)
+                win[(mine && at < (unsigned)width) ? at : (unsigned)(W + lane)] =
+                    make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, u * NT + tid));
+                if (base == t_lo && where[u] >= 0 && (where[u] & (1 << 20)) != 0) {  // (rare)
+                    const float x = (p[u].x - c0) * scale, y = (p[u].y - c1) * scale,
+                                z = (p[u].z - c2) * scale;
+                    if (__builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)) <= 16.0f) {
+                        const int o[3] = {tk_float_order(x), tk_float_order(y), tk_float_order(z)};
+#pragma unroll
+                        for (int ax = 0; ax < 3; ++ax) {
+                            extra_lo[ax] = o[ax] < extra_lo[ax] ? o[ax] : extra_lo[ax];
+                            extra_hi[ax] = o[ax] > extra_hi[ax] ? o[ax] : extra_hi[ax];
+                        }
+                        any_extra = true;
+                    }
+                }
+            }
+            if (any_extra) {
+#pragma unroll
+                for (int ax = 0; ax < 3; ++ax) {
+                    atomicMin(&sextra[ax], extra_lo[ax]);
+                    atomicMax(&sextra[3 + ax], extra_hi[ax]);
+                }
+            }
         }
         __syncthreads();
         for (int s0 = 0; s0 < width; s0 += NT) {
             const int i = base + s0 + tid;
             if (s0 + tid >= width)  // (uniform over each half wave: width is a multiple of 32)
                 continue;
-            const bool exists = i < n;
+            const bool owned = (i >= s_lo && i < s_hi) || (last && i >= n);
+            const bool exists = owned && i < n;
             float4 s = make_float4(qnan, qnan, qnan, __builtin_bit_cast(float, -1));
             if (exists)
                 s = win[s0 + tid];
-            sorted[i] = s;
             const float x = ((exists ? s.x : c0) - c0) * scale;
             const float y = ((exists ? s.y : c1) - c1) * scale;
             const float z = ((exists ? s.z : c2) - c2) * scale;
             const float nn = __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x));
             const bool swept = exists && nn <= 16.0f;
-            uint4 h0, h1;
-            chamfer_key_terms(x, y, z, nn, swept, h0, h1);
-            uint4 *tile = terms + (i >> 5) * 64 + (i & 31);
-            tile[0] = h0;
-            tile[32] = h1;
-            float bl[3], bh[3];
-            bl[0] = half_wave_reduce_to_last<false>(swept ? x : INF);
-            bl[1] = half_wave_reduce_to_last<false>(swept ? y : INF);
-            bl[2] = half_wave_reduce_to_last<false>(swept ? z : INF);
-            bh[0] = half_wave_reduce_to_last<true>(swept ? x : -INF);
-            bh[1] = half_wave_reduce_to_last<true>(swept ? y : -INF);
-            bh[2] = half_wave_reduce_to_last<true>(swept ? z : -INF);
-            if ((i & 31) == 31)
-                boxes[i >> 5] = chamfer_box_bits(bl, bh);
+            if (owned) {
+                sorted[i] = s;
+                uint4 h0, h1;
+                chamfer_key_terms(x, y, z, nn, swept, h0, h1);
+                uint4 *tile = terms + (i >> 5) * 64 + (i & 31);
+                tile[0] = h0;
+                tile[32] = h1;
+            }
+            int bl[3], bh[3];
+            bl[0] = half_wave_reduce_to_last<false>(swept ? tk_float_order(x) : ORDER_POS_INF);
+            bl[1] = half_wave_reduce_to_last<false>(swept ? tk_float_order(y) : ORDER_POS_INF);
+            bl[2] = half_wave_reduce_to_last<false>(swept ? tk_float_order(z) : ORDER_POS_INF);
+            bh[0] = half_wave_reduce_to_last<true>(swept ? tk_float_order(x) : ORDER_NEG_INF);
+            bh[1] = half_wave_reduce_to_last<true>(swept ? tk_float_order(y) : ORDER_NEG_INF);
+            bh[2] = half_wave_reduce_to_last<true>(swept ? tk_float_order(z) : ORDER_NEG_INF);
+            // the tile's box comes from the part that owns the tile's first position
+            if ((i & 31) == 31 && i - 31 >= s_lo) {
+                if (i + 1 == shared_end) {
+#pragma unroll
+                    for (int ax = 0; ax < 3; ++ax) {
+                        bl[ax] = sextra[ax] < bl[ax] ? sextra[ax] : bl[ax];
+                        bh[ax] = sextra[3 + ax] > bh[ax] ? sextra[3 + ax] : bh[ax];
+                    }
+                }
+                const float fl[3] = {tk_order_float(bl[0]), tk_order_float(bl[1]), tk_order_float(bl[2])};
+                const float fh[3] = {tk_order_float(bh[0]), tk_order_float(bh[1]), tk_order_float(bh[2])};
+                boxes[i >> 5] = chamfer_box_bits(fl, fh);
+            }
         }
     }
 }
@@ -3216,8 +3364,16 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
             const int ok = tk_allow_dynamic_lds<chamfer_prepare_kernel>((int)PREP_LDS_BYTES);
             if (ok != TK3D_OK)
                 return ok;
-            hipLaunchKernelGGL(chamfer_prepare_kernel, dim3((unsigned)count), dim3(1024),
-                               PREP_LDS_BYTES, s, sa, first);
+            // workgroups per cloud: as many (4, 2 or 1) as one round over the chip's compute
+            // units allows, each with about 2048 sorted positions or more to write out
+            const int64_t shortest = sa.three_launches[0] ? n[1] : sa.three_launches[1] ? n[0]
+                                     : (n[0] < n[1] ? n[0] : n[1]);
+            int parts = 1;
+            while (parts < 4 && (int64_t)count * parts * 2 <= tk_cu_count() + tk_cu_count() / 4 &&
+                   shortest >= 2048 * parts * 2)
+                parts *= 2;
+            hipLaunchKernelGGL(chamfer_prepare_kernel, dim3((unsigned)(count * parts)), dim3(1024),
+                               PREP_LDS_BYTES, s, sa, first, parts);
         }
         if (sa.three_launches[0] || sa.three_launches[1]) {
             hipLaunchKernelGGL(chamfer_cell_kernel, dim3((unsigned)(2 * B * CHAMFER_CELL_PARTS)),
