@@ -2323,8 +2323,8 @@ __global__ __launch_bounds__(256) void chamfer_tile_kernel(ChamferSortArgs a, in
 }
 
 // The Hilbert position of every cell of the 32^3 grid, worked out when the library is
-// compiled: the kernel below looks a cell up (one 2-byte load from a 64 KiB table that stays
-// in the L2s) instead of spending 135 instructions on it.
+// compiled: the kernel below copies the 64 KiB table into LDS and looks a cell up there
+// instead of spending 135 instructions on it.
 struct ChamferHilbertTable {
     unsigned short at[CHAMFER_SORT_CELLS];
 };
@@ -2415,8 +2415,13 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     __shared__ int sbad, sfar;
     __shared__ int sextra[8];  // box of the later parts' points in this part's last tile
     const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
-    const int cloud = first_cloud + (int)blockIdx.x / parts;
-    const int part = (int)blockIdx.x % parts;
+    // (the parts of a cloud on one XCD, whose L2 then fetches the cloud once: consecutive
+    // workgroup ids go to the eight XCDs in turn)
+    int unit = (int)blockIdx.x;
+    if ((int)gridDim.x % (8 * parts) == 0)
+        unit = (unit & 7) * ((int)gridDim.x >> 3) + (unit >> 3);
+    const int cloud = first_cloud + unit / parts;
+    const int part = unit % parts;
     const int which = cloud >= a.B;
     const int b = cloud - which * a.B;
     const int n = a.n[which], npad = a.npad[which];
@@ -2453,8 +2458,8 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     // ---- the pilot centre, the bounding box and the deviations ----
     float pilot[3], cap[3];
     chamfer_pilot(P, n, pilot, cap);
-    for (int i = tid; i < WORDS; i += NT)
-        hist[i] = 0u;
+    for (int i = tid; i < WORDS / 4; i += NT)
+        reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0u, 0u, 0u, 0u);
     if (tid < 8)
         sextra[tid] = tid < 3 ? ORDER_POS_INF : ORDER_NEG_INF;
     __builtin_amdgcn_sched_barrier(0);  // (the pilot's nine points and the lane's sixteen at
@@ -2462,9 +2467,18 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
     float dev[3] = {0.0f, 0.0f, 0.0f};
     bool bad = false;
+    // (the table of Hilbert positions comes along, into the LDS that the windows use later:
+    // looked up in global memory, one cache line per lane, the look-ups took 8 us)
+    unsigned short *const cell_of = reinterpret_cast<unsigned short *>(win);
+    static_assert(sizeof(ChamferHilbertTable) <= (size_t)PREP_WINDOW * sizeof(float4), "table fits");
     {
         TkPoint3<float> p[U];
         load_points(p);
+        constexpr int QUADS = (int)(sizeof(ChamferHilbertTable) / sizeof(uint4)) / NT;
+        uint4 table[QUADS];
+#pragma unroll
+        for (int k = 0; k < QUADS; ++k)
+            table[k] = reinterpret_cast<const uint4 *>(chamfer_hilbert_table.at)[k * NT + tid];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const float v[3] = {p[u].x, p[u].y, p[u].z};
@@ -2477,6 +2491,9 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
                 dev[ax] += counts ? __builtin_fminf(__builtin_fabsf(v[ax] - pilot[ax]), cap[ax]) : 0.0f;
             }
         }
+#pragma unroll
+        for (int k = 0; k < QUADS; ++k)
+            reinterpret_cast<uint4 *>(win)[k * NT + tid] = table[k];
     }
 #pragma unroll
     for (int ax = 0; ax < 3; ++ax) {
@@ -2547,7 +2564,7 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
             const float ux = __builtin_fminf(__builtin_fmaxf((p[u].x - flo[0]) * inv, 0.0f), 31.0f);
             const float uy = __builtin_fminf(__builtin_fmaxf((p[u].y - flo[1]) * inv, 0.0f), 31.0f);
             const float uz = __builtin_fminf(__builtin_fmaxf((p[u].z - flo[2]) * inv, 0.0f), 31.0f);
-            where[u] = chamfer_hilbert_table.at[((int)ux << 10) | ((int)uy << 5) | (int)uz];
+            where[u] = cell_of[((int)ux << 10) | ((int)uy << 5) | (int)uz];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -2659,9 +2676,7 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
             load_points(p);
             if (base > t_lo)
                 __syncthreads();  // the window's previous contents have been read
-            int extra_lo[3] = {ORDER_POS_INF, ORDER_POS_INF, ORDER_POS_INF};
-            int extra_hi[3] = {ORDER_NEG_INF, ORDER_NEG_INF, ORDER_NEG_INF};
-            bool any_extra = false;
+            int marked = 0;  // bit u: a later part's point whose cell begins in the last tile
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int pos = where[u] & 0xfffff;
@@ -2671,21 +2686,25 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
                 // a store that is skipped costs a branch per point)
                 win[(mine && at < (unsigned)width) ? at : (unsigned)(W + lane)] =
                     make_float4(p[u].x, p[u].y, p[u].z, __builtin_bit_cast(float, u * NT + tid));
-                if (base == t_lo && where[u] >= 0 && (where[u] & (1 << 20)) != 0) {  // (rare)
+                marked |= (where[u] >= 0 && (where[u] & (1 << 20)) != 0) ? 1 << u : 0;
+            }
+            if (base == t_lo && marked != 0) {  // (a handful of lanes, if any)
+                int extra_lo[3] = {ORDER_POS_INF, ORDER_POS_INF, ORDER_POS_INF};
+                int extra_hi[3] = {ORDER_NEG_INF, ORDER_NEG_INF, ORDER_NEG_INF};
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
                     const float x = (p[u].x - c0) * scale, y = (p[u].y - c1) * scale,
                                 z = (p[u].z - c2) * scale;
-                    if (__builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)) <= 16.0f) {
+                    if (((marked >> u) & 1) != 0 &&
+                        __builtin_fmaf(z, z, __builtin_fmaf(y, y, x * x)) <= 16.0f) {
                         const int o[3] = {tk_float_order(x), tk_float_order(y), tk_float_order(z)};
 #pragma unroll
                         for (int ax = 0; ax < 3; ++ax) {
                             extra_lo[ax] = o[ax] < extra_lo[ax] ? o[ax] : extra_lo[ax];
                             extra_hi[ax] = o[ax] > extra_hi[ax] ? o[ax] : extra_hi[ax];
                         }
-                        any_extra = true;
                     }
                 }
-            }
-            if (any_extra) {
 #pragma unroll
                 for (int ax = 0; ax < 3; ++ax) {
                     atomicMin(&sextra[ax], extra_lo[ax]);
