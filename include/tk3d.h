@@ -88,6 +88,21 @@ int tk3d_chamfer_distance_forward_ws_f32(const float *xyz1, const float *xyz2,
                                          int64_t *idx2, void *workspace,
                                          size_t workspace_bytes, void *stream);
 
+/* chamfer_distance_forward_cuda on channel-first clouds xyz1 [B,3,N1], xyz2 [B,3,N2], read
+ * in place: what the reference's chamfer_distance / nn_distance with transpose=True compute
+ * after copying both clouds to [B,N,3] (torkit3d/ops/chamfer_distance.py:52-55,68-70).
+ * Outputs as above. `workspace` may be NULL; with the workspace of the call above (fp32,
+ * both clouds of at most 16384 points) the sorted path is taken. */
+int tk3d_chamfer_distance_forward_bcn_f32(const float *xyz1, const float *xyz2,
+                                          int64_t B, int64_t N1, int64_t N2,
+                                          float *dist1, int64_t *idx1, float *dist2,
+                                          int64_t *idx2, void *workspace,
+                                          size_t workspace_bytes, void *stream);
+int tk3d_chamfer_distance_forward_bcn_f64(const double *xyz1, const double *xyz2,
+                                          int64_t B, int64_t N1, int64_t N2,
+                                          double *dist1, int64_t *idx1, double *dist2,
+                                          int64_t *idx2, void *stream);
+
 /* Replaces chamfer_distance_backward_cuda
  * (chamfer_distance.h:10-16, chamfer_distance_kernel.cu:200-274).
  * grad_xyz1[b,i] = 2*gd1[b,i]*(x1[b,i]-x2[b,idx1[b,i]])

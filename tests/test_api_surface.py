@@ -262,3 +262,17 @@ def test_pointnet_runs_on_cpu_with_feature_and_mask():
     # Masked points contribute zeros, which post-ReLU features can only tie, never beat.
     short = net(points[..., :10], feature[..., :10])
     torch.testing.assert_close(out["feature"], short["feature"])
+
+
+def test_other_spellings_of_the_ops():
+    # knn_distance (the compiled op's name), farthest_point_sample, three_interpolate and
+    # gather_points name the same functions, in the op modules and at the package root
+    import torkit3d_amd
+    from torkit3d_amd.ops import group_points, interpolate_feature, knn_points, sample_farthest_points
+
+    assert knn_points.knn_distance is knn_points.knn_points
+    assert sample_farthest_points.farthest_point_sample is sample_farthest_points.sample_farthest_points
+    assert interpolate_feature.three_interpolate is interpolate_feature.interpolate_feature
+    assert group_points.gather_points is group_points.group_points
+    assert torkit3d_amd.knn_distance is knn_points.knn_points
+    assert torkit3d_amd.farthest_point_sample is sample_farthest_points.sample_farthest_points

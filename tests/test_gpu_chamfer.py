@@ -404,3 +404,65 @@ def test_split_sweep_with_slices_that_hold_no_finite_distance(cuda, n1, n2):
     c[1] = float("nan")                 # a cloud without any candidate: (inf, -1) everywhere
     a[0, 7] = float("nan")
     check_forward(a, c, cuda)
+
+
+# ---- channel-first clouds, read in place ---------------------------------------------------
+
+def check_forward_channels_first(a, c, cuda):
+    """nn_distance(transpose=True) on [B,3,N] device tensors against the oracle on [B,N,3]."""
+    from torkit3d_amd.ops.chamfer_distance import nn_distance
+
+    a_bcn = a.to(cuda).transpose(1, 2).contiguous()
+    c_bcn = c.to(cuda).transpose(1, 2).contiguous()
+    out = nn_distance(a_bcn, c_bcn, transpose=True)
+    want = oracle.chamfer_forward(a.contiguous().numpy(), c.contiguous().numpy())
+    for name, got, exp in zip(("dist1", "idx1", "dist2", "idx2"), out, want):
+        np.testing.assert_array_equal(got.cpu().numpy(), exp, err_msg=name)
+
+
+@pytest.mark.parametrize("b,n1,n2", [(2, 1024, 1024), (3, 2043, 1999), (1, 1, 1), (2, 5000, 33),
+                                     (2, 33, 5000), (4, 255, 257), (2, 4096, 4100),
+                                     (8, 8192, 8192),     # the sorted path, [3,N] read in place
+                                     (5, 16384, 6000),    # sorted path, four parts per cloud
+                                     (1, 20000, 3001),    # beyond the sorted path's [3,N] reach
+                                     (40, 1500, 1100)])
+def test_forward_channels_first(cuda, b, n1, n2):
+    # reference: chamfer_distance / nn_distance with transpose=True
+    # (torkit3d/ops/chamfer_distance.py:52-55,68-70; tests/ops/test_chamfer_distance.py:86-99)
+    g = gen(31)
+    check_forward_channels_first(uniform_cloud(g, b, n1), uniform_cloud(g, b, n2), cuda)
+    check_forward_channels_first(sphere_cloud(g, b, n1), sphere_cloud(g, b, n2), cuda)
+
+
+@pytest.mark.parametrize("kind", HARD_KINDS)
+def test_channels_first_on_hard_inputs(cuda, kind):
+    a, c = _clouds(kind, gen(sum(map(ord, kind)) + 9), 2, 2500, 3001)
+    check_forward_channels_first(a, c, cuda)
+    a, c = _clouds(kind, gen(sum(map(ord, kind)) + 10), 3, 5000, 6001)   # sorted path sizes
+    check_forward_channels_first(a, c, cuda)
+
+
+def test_channels_first_fp64_and_gradients(cuda):
+    from torkit3d_amd.ops.chamfer_distance import chamfer_distance, nn_distance
+
+    g = gen(33)
+    a = torch.rand(3, 3, 700, generator=g, dtype=torch.float64)
+    c = torch.rand(3, 3, 900, generator=g, dtype=torch.float64)
+    out = nn_distance(a.to(cuda), c.to(cuda), transpose=True)
+    want = oracle.chamfer_forward(a.transpose(1, 2).contiguous().numpy(),
+                                  c.transpose(1, 2).contiguous().numpy())
+    for got, exp in zip(out, want):
+        np.testing.assert_array_equal(got.cpu().numpy(), exp)
+    # gradients of the channel-first call equal those of the [B,N,3] call, transposed
+    for dtype in (torch.float32, torch.float64):
+        x1 = a.to(dtype).to(cuda).requires_grad_()
+        x2 = c.to(dtype).to(cuda).requires_grad_()
+        d1, d2 = chamfer_distance(x1, x2, transpose=True)
+        (d1.sum() + 2 * d2.sum()).backward()
+        y1 = a.to(dtype).transpose(1, 2).contiguous().to(cuda).requires_grad_()
+        y2 = c.to(dtype).transpose(1, 2).contiguous().to(cuda).requires_grad_()
+        e1, e2 = chamfer_distance(y1, y2)
+        (e1.sum() + 2 * e2.sum()).backward()
+        assert torch.equal(d1, e1) and torch.equal(d2, e2)
+        assert torch.equal(x1.grad, y1.grad.transpose(1, 2))
+        assert torch.equal(x2.grad, y2.grad.transpose(1, 2))

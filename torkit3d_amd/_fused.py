@@ -16,6 +16,7 @@ __all__ = [
     "sample_farthest_points_gather",
     "ball_query_bcn",
     "knn_distance_bcn",
+    "chamfer_forward_bcn",
     "group_points_concat_forward",
     "group_points_concat_backward",
     "three_nn",
@@ -177,3 +178,33 @@ def three_nn(query, key, channels_first, eps=1e-10):
                   ctypes.c_double(float(eps)), ptr(distance), ptr(index), ptr(weight),
                   stream_of(query))
     return distance, index, weight
+
+
+def chamfer_forward_bcn(xyz1, xyz2):
+    """xyz1 [B,3,N1], xyz2 [B,3,N2] -> [dist1, idx1, dist2, idx2], the clouds read in place
+    (the reference copies them to [B,N,3] first, torkit3d/ops/chamfer_distance.py:52-55)."""
+    b, n1 = _cloud_dims("xyz1", xyz1, True)
+    b2, n2 = _cloud_dims("xyz2", xyz2, True)
+    _check_eq(b, b2, "xyz1.size(0) == xyz2.size(0)")
+    _check_same("xyz1", xyz1, "xyz2", xyz2)
+    dev = xyz1.device
+    with _lib.on_device_of(xyz1):
+        dist1 = torch.empty((b, n1), dtype=xyz1.dtype, device=dev)
+        idx1 = torch.empty((b, n1), dtype=torch.int64, device=dev)
+        dist2 = torch.empty((b, n2), dtype=xyz1.dtype, device=dev)
+        idx2 = torch.empty((b, n2), dtype=torch.int64, device=dev)
+        if xyz1.dtype == torch.float32:
+            ws_bytes = _lib.chamfer_workspace_bytes(b, n1, n2) if max(n1, n2) <= 16384 else 0
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
+            fn = _lib.lib().tk3d_chamfer_distance_forward_bcn_f32
+            fn.restype = ctypes.c_int
+            _lib.check(fn(ptr(xyz1), ptr(xyz2), i64(b), i64(n1), i64(n2), ptr(dist1), ptr(idx1),
+                          ptr(dist2), ptr(idx2),
+                          ctypes.c_void_p(ws.data_ptr() if ws is not None else 0),
+                          ctypes.c_size_t(ws_bytes), stream_of(xyz1)),
+                       "tk3d_chamfer_distance_forward_bcn_f32")
+        else:
+            _lib.call("tk3d_chamfer_distance_forward_bcn", xyz1, ptr(xyz1), ptr(xyz2), i64(b),
+                      i64(n1), i64(n2), ptr(dist1), ptr(idx1), ptr(dist2), ptr(idx2),
+                      stream_of(xyz1))
+    return [dist1, idx1, dist2, idx2]

@@ -60,6 +60,34 @@ template <> __device__ __forceinline__ double chamfer_init_min<double>()
     return 1e40;
 }
 
+// A cloud as the kernels read it: coordinate a of point j of the cloud at `base` is
+// base[j * 3 + a] in a [N,3] cloud and base[a * plane + j] in a [3,N] one (SOA; `plane` is
+// the number of points of the whole cloud, also when `base` points at a slice of it).
+template <bool SOA, typename T>
+__device__ __forceinline__ T chamfer_coord(const T *__restrict__ base, int plane, int j, int a)
+{
+    return SOA ? base[(int64_t)a * plane + j] : base[(int64_t)j * 3 + a];
+}
+template <bool SOA, typename T>
+__device__ __forceinline__ TkPoint3<T> chamfer_point(const T *__restrict__ base, int plane, int j)
+{
+    if constexpr (SOA) {
+        TkPoint3<T> p;
+        p.x = base[j];
+        p.y = base[(int64_t)plane + j];
+        p.z = base[(int64_t)2 * plane + j];
+        return p;
+    } else {
+        return tk_load3<T>(base + (int64_t)j * 3);
+    }
+}
+// Start of batch element b's key slice beginning at key k0, in either layout.
+template <bool SOA, typename T>
+__device__ __forceinline__ const T *chamfer_key_base(const T *key, int b, int nk_cloud, int k0)
+{
+    return SOA ? key + (int64_t)b * nk_cloud * 3 + k0 : key + ((int64_t)b * nk_cloud + k0) * 3;
+}
+
 // Decodes blockIdx into (direction, batch, query block). Workgroups are handed to
 // the 8 XCDs round-robin by blockIdx; the remap gives each XCD a contiguous range of
 // logical workgroups, so the workgroups that sweep the same key cloud share one L2
@@ -115,7 +143,7 @@ __device__ __forceinline__ void chamfer_emit(const ChamferDir<T> &d, int b, int 
 
 // Exact sweep of one workgroup: QPL*BLOCK queries against the whole key cloud.
 // `skey` is STAGE*4 elements of LDS.
-template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
+template <typename T, int QPL, int BLOCK, int TILE, int STAGE, bool SOA = false>
 __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int b, int qblock,
                                                     int slice, T *skey)
 {
@@ -125,7 +153,7 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
     const int k0 = slice * d.slice_len;  // this workgroup sweeps keys [k0, k0 + nk)
     const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
     const T *__restrict__ Q = d.query + (int64_t)b * nq * 3;
-    const T *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
+    const T *__restrict__ K = chamfer_key_base<SOA, T>(d.key, b, d.nk, k0);
 
     T qx[QPL], qy[QPL], qz[QPL], best[QPL];
     int btile[QPL];
@@ -133,9 +161,9 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
     for (int i = 0; i < QPL; ++i) {
         const int qi = (qblock * QPL + i) * BLOCK + tid;
         const bool ok = qi < nq;
-        qx[i] = ok ? Q[(int64_t)qi * 3 + 0] : (T)0;
-        qy[i] = ok ? Q[(int64_t)qi * 3 + 1] : (T)0;
-        qz[i] = ok ? Q[(int64_t)qi * 3 + 2] : (T)0;
+        qx[i] = ok ? chamfer_coord<SOA, T>(Q, nq, qi, 0) : (T)0;
+        qy[i] = ok ? chamfer_coord<SOA, T>(Q, nq, qi, 1) : (T)0;
+        qz[i] = ok ? chamfer_coord<SOA, T>(Q, nq, qi, 2) : (T)0;
         best[i] = chamfer_init_min<T>();
         btile[i] = -1;
     }
@@ -146,7 +174,7 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
             const int kj = stage0 + j;
             T x = tk_inf<T>(), y = tk_inf<T>(), z = tk_inf<T>();
             if (kj < nk) {
-                const TkPoint3<T> p = tk_load3<T>(K + (int64_t)kj * 3);
+                const TkPoint3<T> p = chamfer_point<SOA, T>(K, d.nk, kj);
                 x = p.x, y = p.y, z = p.z;
             }
             // Keys past the end sit at +inf: their distance is +inf or NaN and
@@ -204,7 +232,7 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
             const int j0 = btile[i] * TILE;
             const int j1 = (j0 + TILE < nk) ? j0 + TILE : nk;
             for (int j = j1 - 1; j >= j0; --j) {
-                const TkPoint3<T> p = tk_load3<T>(K + (int64_t)j * 3);
+                const TkPoint3<T> p = chamfer_point<SOA, T>(K, d.nk, j);
                 const T dd = tk_dist2<T>(p.x, p.y, p.z, qx[i], qy[i], qz[i]);
                 found = (dd == best[i]) ? j : found;
             }
@@ -213,13 +241,13 @@ __device__ __forceinline__ void chamfer_exact_sweep(const ChamferDir<T> &d, int 
     }
 }
 
-template <typename T, int QPL, int BLOCK, int TILE, int STAGE>
+template <typename T, int QPL, int BLOCK, int TILE, int STAGE, bool SOA = false>
 __global__ __launch_bounds__(BLOCK) void chamfer_forward_kernel(ChamferFwdArgs<T> args)
 {
     __shared__ T skey[STAGE * 4 + 8];  // + 2 keys for the read-ahead
     int b, qblock, slice;
     const ChamferDir<T> &d = chamfer_decode_block<T>(args, b, qblock, slice);
-    chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE>(d, b, qblock, slice, skey);
+    chamfer_exact_sweep<T, QPL, BLOCK, TILE, STAGE, SOA>(d, b, qblock, slice, skey);
 }
 
 // ---- fp32 forward with a bounded-error pre-filter -------------------------------
@@ -297,11 +325,11 @@ __device__ __forceinline__ float wave_reduce_max(float v)
 // keys t, t+BLOCK, ... in ascending order with strict '<'; the workgroup keeps the
 // smallest distance and, among equal distances, the lowest key index. Every lane
 // returns the result. `sval` / `sidx` hold one entry per wave.
-template <int BLOCK>
+template <int BLOCK, bool SOA = false>
 __device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict__ K, int nk,
                                                          float qx, float qy, float qz,
                                                          float *sval, int *sidx, float &out_d,
-                                                         int &out_j)
+                                                         int &out_j, int kplane = 0)
 {
     constexpr int NW = BLOCK / TK_WAVE;
     const int tid = threadIdx.x;
@@ -309,7 +337,7 @@ __device__ __forceinline__ void chamfer_block_exact_scan(const float *__restrict
     int bj = -1;
 #pragma unroll 8
     for (int j = tid; j < nk; j += BLOCK) {
-        const TkPoint3<float> p = tk_load3<float>(K + (int64_t)j * 3);
+        const TkPoint3<float> p = chamfer_point<SOA, float>(K, kplane, j);
         const float d = tk_dist2<float>(p.x, p.y, p.z, qx, qy, qz);
         if (d < best) {
             best = d;
@@ -779,7 +807,7 @@ __device__ __forceinline__ float chamfer_fold16(float m, const tk_f32x16 &acc)
 
 // One workgroup's share: query block `qblock` of batch element `b` against key slice
 // `slice` of direction `d`.
-template <int NQB, int BLOCK, int STAGE>
+template <int NQB, int BLOCK, int STAGE, bool SOA = false>
 __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, const int b,
                                                    const int qblock, const int slice)
 {
@@ -809,7 +837,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     const int k0 = slice * d.slice_len;
     const int nk = (d.nk - k0 < d.slice_len) ? d.nk - k0 : d.slice_len;
     const float *__restrict__ Q = d.query + (int64_t)b * nq * 3;
-    const float *__restrict__ K = d.key + ((int64_t)b * d.nk + k0) * 3;
+    const float *__restrict__ K = chamfer_key_base<SOA, float>(d.key, b, d.nk, k0);
     const float INF = __builtin_huge_valf();
 
     // ---- centre and scale from a strided sample of the key cloud ----
@@ -819,7 +847,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
 #pragma unroll
         for (int r = 0; r < SAMPLES; ++r) {
             const int j = (int)(((int64_t)(r * BLOCK + tid) * nk) / (SAMPLES * BLOCK));
-            sp[r] = tk_load3<float>(K + (int64_t)j * 3);
+            sp[r] = chamfer_point<SOA, float>(K, d.nk, j);
         }
 #pragma unroll
         for (int r = 0; r < SAMPLES; ++r) {
@@ -874,7 +902,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     const bool safe = nk > 0 && (c0 - c0 == 0.0f) && (c1 - c1 == 0.0f) && (c2 - c2 == 0.0f) &&
                       (ext - ext == 0.0f) && (ext == 0.0f || (ebits >= -40 && ebits <= 40));
     if (!safe) {  // uniform over the workgroup
-        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512, SOA>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
     }
@@ -890,9 +918,9 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     for (int g = 0; g < NQB; ++g) {
         const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
         const bool ok = qi < nq;
-        const float px = ((ok ? Q[(int64_t)qi * 3 + 0] : c0) - c0) * scale;
-        const float py = ((ok ? Q[(int64_t)qi * 3 + 1] : c1) - c1) * scale;
-        const float pz = ((ok ? Q[(int64_t)qi * 3 + 2] : c2) - c2) * scale;
+        const float px = ((ok ? chamfer_coord<SOA, float>(Q, nq, qi, 0) : c0) - c0) * scale;
+        const float py = ((ok ? chamfer_coord<SOA, float>(Q, nq, qi, 1) : c1) - c1) * scale;
+        const float pz = ((ok ? chamfer_coord<SOA, float>(Q, nq, qi, 2) : c2) - c2) * scale;
         qnorm[g] =
             1.000001f * __builtin_sqrtf(__builtin_fmaf(pz, pz, __builtin_fmaf(py, py, px * px)));
         const bool in_range = qnorm[g] <= 16000.0f;  // false for NaN
@@ -915,7 +943,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
             pre[r][1] = c1;
             pre[r][2] = c2;
             if (kj < nk) {
-                const TkPoint3<float> p = tk_load3<float>(K + (int64_t)kj * 3);
+                const TkPoint3<float> p = chamfer_point<SOA, float>(K, d.nk, kj);
                 pre[r][0] = p.x;
                 pre[r][1] = p.y;
                 pre[r][2] = p.z;
@@ -1029,7 +1057,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
             if (tid == 0)
                 s_count = 0;
             if (total * 4 > 2 * QB) {  // uniform over the workgroup
-                chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+                chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512, SOA>(
                     d, b, qblock, slice, reinterpret_cast<float *>(sterm));
                 return;
             }
@@ -1049,7 +1077,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     // identical keys, scale 1, beside keys that differ a little: the fp16 terms have no
     // precision for those; with a sample that has an extent max|k'| >= 1)
     if (!(kmax2 <= 32768.0f) || (kmax2 > 0.0f && kmax2 < 0.25f)) {  // uniform
-        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512, SOA>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
     }
@@ -1057,15 +1085,17 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     const float guard = 1e-36f * scale * scale;  // scale^2 <= 2^80
 
     // ---- epilogue: exact evaluation of each half's candidate groups, then the merge ----
-    const bool k_aligned = (reinterpret_cast<uintptr_t>(K) & 15) == 0;  // runs of 4 keys: 48 B
+    // runs of 4 keys: 48 bytes of a [N,3] cloud, 16 bytes of each coordinate of a [3,N] one
+    const bool k_aligned =
+        (reinterpret_cast<uintptr_t>(K) & 15) == 0 && (!SOA || (d.nk & 3) == 0);
     float qx[NQB], qy[NQB], qz[NQB];
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
         const int qi = qblock * QB + (wave * NQB + g) * 32 + col;
         const bool ok = qi < nq;
-        qx[g] = ok ? Q[(int64_t)qi * 3 + 0] : 0.0f;
-        qy[g] = ok ? Q[(int64_t)qi * 3 + 1] : 0.0f;
-        qz[g] = ok ? Q[(int64_t)qi * 3 + 2] : 0.0f;
+        qx[g] = ok ? chamfer_coord<SOA, float>(Q, nq, qi, 0) : 0.0f;
+        qy[g] = ok ? chamfer_coord<SOA, float>(Q, nq, qi, 1) : 0.0f;
+        qz[g] = ok ? chamfer_coord<SOA, float>(Q, nq, qi, 2) : 0.0f;
     }
 #pragma unroll
     for (int g = 0; g < NQB; ++g) {
@@ -1096,25 +1126,36 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
                     continue;
                 // this half's keys of the group: runs of 4 keys, 8 keys apart
                 if (k_aligned && (group + 1) * GROUP <= nk) {
-                    const float4 *p4 =
-                        reinterpret_cast<const float4 *>(K + (int64_t)(group * GROUP + half * 4) * 3);
+                    const float4 *p4 = reinterpret_cast<const float4 *>(
+                        K + (int64_t)(group * GROUP + half * 4) * (SOA ? 1 : 3));
+                    const int plane4 = d.nk >> 2;  // ([3,N]: quads between the coordinates)
 #pragma unroll
                     for (int r0 = 0; r0 < GROUP / 8; r0 += 4) {
                         float4 f[4][3];
 #pragma unroll
-                        for (int rr = 0; rr < 4; ++rr) {  // a run is 48 bytes, runs 96 bytes apart
-                            f[rr][0] = p4[(r0 + rr) * 6 + 0];
-                            f[rr][1] = p4[(r0 + rr) * 6 + 1];
-                            f[rr][2] = p4[(r0 + rr) * 6 + 2];
+                        for (int rr = 0; rr < 4; ++rr) {
+                            if constexpr (SOA) {  // x, y, z of 4 keys; runs 32 bytes apart
+                                f[rr][0] = p4[(r0 + rr) * 2];
+                                f[rr][1] = p4[(r0 + rr) * 2 + plane4];
+                                f[rr][2] = p4[(r0 + rr) * 2 + 2 * plane4];
+                            } else {  // a run is 48 bytes, runs 96 bytes apart
+                                f[rr][0] = p4[(r0 + rr) * 6 + 0];
+                                f[rr][1] = p4[(r0 + rr) * 6 + 1];
+                                f[rr][2] = p4[(r0 + rr) * 6 + 2];
+                            }
                         }
 #pragma unroll
                         for (int rr = 0; rr < 4; ++rr) {
                             const int j = group * GROUP + (r0 + rr) * 8 + half * 4;
                             const float4 f0 = f[rr][0], f1 = f[rr][1], f2 = f[rr][2];
-                            const float dd0 = tk_dist2<float>(f0.x, f0.y, f0.z, qx[g], qy[g], qz[g]);
-                            const float dd1 = tk_dist2<float>(f0.w, f1.x, f1.y, qx[g], qy[g], qz[g]);
-                            const float dd2 = tk_dist2<float>(f1.z, f1.w, f2.x, qx[g], qy[g], qz[g]);
-                            const float dd3 = tk_dist2<float>(f2.y, f2.z, f2.w, qx[g], qy[g], qz[g]);
+                            const float dd0 = SOA ? tk_dist2<float>(f0.x, f1.x, f2.x, qx[g], qy[g], qz[g])
+                                                  : tk_dist2<float>(f0.x, f0.y, f0.z, qx[g], qy[g], qz[g]);
+                            const float dd1 = SOA ? tk_dist2<float>(f0.y, f1.y, f2.y, qx[g], qy[g], qz[g])
+                                                  : tk_dist2<float>(f0.w, f1.x, f1.y, qx[g], qy[g], qz[g]);
+                            const float dd2 = SOA ? tk_dist2<float>(f0.z, f1.z, f2.z, qx[g], qy[g], qz[g])
+                                                  : tk_dist2<float>(f1.z, f1.w, f2.x, qx[g], qy[g], qz[g]);
+                            const float dd3 = SOA ? tk_dist2<float>(f0.w, f1.w, f2.w, qx[g], qy[g], qz[g])
+                                                  : tk_dist2<float>(f2.y, f2.z, f2.w, qx[g], qy[g], qz[g]);
                             if (dd0 < bestd) { bestd = dd0; bestj = j; }
                             if (dd1 < bestd) { bestd = dd1; bestj = j + 1; }
                             if (dd2 < bestd) { bestd = dd2; bestj = j + 2; }
@@ -1125,7 +1166,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
                     for (int run = 0; run < GROUP / 8; ++run) {
                         const int j = group * GROUP + run * 8 + half * 4;
                         for (int e = j; e < j + 4 && e < nk; ++e) {
-                            const TkPoint3<float> p = tk_load3<float>(K + (int64_t)e * 3);
+                            const TkPoint3<float> p = chamfer_point<SOA, float>(K, d.nk, e);
                             const float dd = tk_dist2<float>(p.x, p.y, p.z, qx[g], qy[g], qz[g]);
                             if (dd < bestd) {
                                 bestd = dd;
@@ -1158,7 +1199,7 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
     __syncthreads();
     const int nscan = s_count;
     if (nscan > MAX_SCANS) {  // uniform over the workgroup
-        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512>(
+        chamfer_exact_sweep<float, QB / BLOCK, BLOCK, 64, 512, SOA>(
             d, b, qblock, slice, reinterpret_cast<float *>(sterm));
         return;
     }
@@ -1166,20 +1207,22 @@ __device__ __forceinline__ void chamfer_mfma_block(const ChamferDir<float> &d, c
         const int qi = qblock * QB + s_list[e];
         float bd;
         int bj;
-        chamfer_block_exact_scan<BLOCK>(K, nk, Q[(int64_t)qi * 3 + 0], Q[(int64_t)qi * 3 + 1],
-                                        Q[(int64_t)qi * 3 + 2], &sred[0][0], sidx, bd, bj);
+        chamfer_block_exact_scan<BLOCK, SOA>(K, nk, chamfer_coord<SOA, float>(Q, nq, qi, 0),
+                                             chamfer_coord<SOA, float>(Q, nq, qi, 1),
+                                             chamfer_coord<SOA, float>(Q, nq, qi, 2), &sred[0][0],
+                                             sidx, bd, bj, d.nk);
         if (tid == 0)
             chamfer_emit<float>(d, b, qi, k0, bd, bj);
     }
 }
 
-template <int NQB, int BLOCK, int STAGE>
+template <int NQB, int BLOCK, int STAGE, bool SOA = false>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
 {
     int b, qblock, slice;
     const ChamferDir<float> &d = chamfer_decode_block<float>(args, b, qblock, slice);
-    chamfer_mfma_block<NQB, BLOCK, STAGE>(d, b, qblock, slice);
+    chamfer_mfma_block<NQB, BLOCK, STAGE, SOA>(d, b, qblock, slice);
 }
 
 // The same sweep for the clouds another kernel has flagged (args.only_if: a word per
@@ -1187,7 +1230,7 @@ chamfer_forward_mfma_kernel(ChamferFwdArgs<float> args)
 // number of workgroups go through all (direction, batch element, query block) shares and
 // work on those whose cloud carries a flag; a launch that finds no flag at all leaves at
 // once.
-template <int NQB, int BLOCK, int STAGE>
+template <int NQB, int BLOCK, int STAGE, bool SOA = false>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 chamfer_forward_mfma_flagged_kernel(ChamferFwdArgs<float> args, int total)
 {
@@ -1202,7 +1245,7 @@ chamfer_forward_mfma_flagged_kernel(ChamferFwdArgs<float> args, int total)
         const int qblock = rest / d.slices, slice = rest - qblock * d.slices;
         if (args.only_if[which * args.nbatch + b] == 0)  // uniform over the workgroup
             continue;
-        chamfer_mfma_block<NQB, BLOCK, STAGE>(d, b, qblock, slice);
+        chamfer_mfma_block<NQB, BLOCK, STAGE, SOA>(d, b, qblock, slice);
         __syncthreads();  // the next share reuses the stage buffers
     }
 }
@@ -1626,7 +1669,7 @@ int chamfer_forward_run(Kernel kernel, int block, const ChamferFwdArgs<T> &a, in
     return tk_launch_status();
 }
 
-template <typename T, int QPL, int BLOCK = 256, int TILE = 32, int STAGE = 1024>
+template <typename T, int QPL, int BLOCK = 256, int TILE = 32, int STAGE = 1024, bool SOA = false>
 int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
                            int64_t N2, T *dist1, int64_t *idx1, T *dist2,
                            int64_t *idx2, hipStream_t stream, int slices = 1)
@@ -1637,7 +1680,7 @@ int chamfer_forward_launch(const T *xyz1, const T *xyz2, int64_t B, int64_t N1,
                                                            dist2, idx2, slices, nblocks);
     if (rc != TK3D_OK)
         return rc;
-    return chamfer_forward_run<T>(chamfer_forward_kernel<T, QPL, BLOCK, TILE, STAGE>, BLOCK, a,
+    return chamfer_forward_run<T>(chamfer_forward_kernel<T, QPL, BLOCK, TILE, STAGE, SOA>, BLOCK, a,
                                   nblocks, B, stream);
 }
 
@@ -1657,7 +1700,7 @@ int chamfer_forward_filter_launch(const float *xyz1, const float *xyz2, int64_t 
 }
 
 // The matrix pre-filter on the clouds flagged in `only_if` ([2, B]), unsplit.
-template <int NQB, int BLOCK = 256, int STAGE = 512>
+template <int NQB, bool SOA = false, int BLOCK = 256, int STAGE = 512>
 int chamfer_forward_mfma_flagged_launch(const float *xyz1, const float *xyz2, int64_t B,
                                         int64_t N1, int64_t N2, float *dist1, int64_t *idx1,
                                         float *dist2, int64_t *idx2, hipStream_t stream,
@@ -1673,12 +1716,12 @@ int chamfer_forward_mfma_flagged_launch(const float *xyz1, const float *xyz2, in
     const int64_t grid = nblocks < 4 * tk_cu_count() ? nblocks : 4 * tk_cu_count();
     if (grid == 0)
         return TK3D_OK;
-    hipLaunchKernelGGL((chamfer_forward_mfma_flagged_kernel<NQB, BLOCK, STAGE>),
+    hipLaunchKernelGGL((chamfer_forward_mfma_flagged_kernel<NQB, BLOCK, STAGE, SOA>),
                        dim3((unsigned)grid), dim3(BLOCK), 0, stream, a, (int)nblocks);
     return tk_launch_status();
 }
 
-template <int NQB, int BLOCK = 256, int STAGE = 512>
+template <int NQB, bool SOA = false, int BLOCK = 256, int STAGE = 512>
 int chamfer_forward_mfma_launch(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                                 int64_t N2, float *dist1, int64_t *idx1, float *dist2,
                                 int64_t *idx2, hipStream_t stream, int slices0 = 1, int slices1 = 1)
@@ -1689,7 +1732,7 @@ int chamfer_forward_mfma_launch(const float *xyz1, const float *xyz2, int64_t B,
         a, xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, slices0, nblocks, slices1);
     if (rc != TK3D_OK)
         return rc;
-    return chamfer_forward_run<float>(chamfer_forward_mfma_kernel<NQB, BLOCK, STAGE>, BLOCK, a,
+    return chamfer_forward_run<float>(chamfer_forward_mfma_kernel<NQB, BLOCK, STAGE, SOA>, BLOCK, a,
                                       nblocks, B, stream);
 }
 
@@ -1727,7 +1770,7 @@ inline double chamfer_sweep_cost(int64_t B, int64_t N1, int64_t N2, int qpl, int
     return (want_slices > 1 ? 20.0 : 12.0) + cycles / 2100.0;
 }
 
-template <typename T>
+template <typename T, bool SOA = false>
 int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t N2,
                     T *dist1, int64_t *idx1, T *dist2, int64_t *idx2, void *stream)
 {
@@ -1789,14 +1832,16 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
             // lose to the key terms every workgroup stages for itself (B=32, 16384 x 16384:
             // 0.59 -> 0.64 ms).
             const int64_t nkmax = N1 > N2 ? N1 : N2;
-            if (blocks >= 96 && (blocks <= 384 || (blocks <= 640 && nkmax <= 4096)))
-                return chamfer_forward_mfma_launch<2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
-                                                      idx2, s, want[0], want[1]);
+            // ([3,N] clouds: the vector pre-filter below reads [N,3] only, so the matrix
+            // pre-filter also takes the launches of under 96 workgroups)
+            if ((SOA || blocks >= 96) && (blocks <= 384 || (blocks <= 640 && nkmax <= 4096)))
+                return chamfer_forward_mfma_launch<2, SOA>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                           dist2, idx2, s, want[0], want[1]);
             if (blocks >= 96)
-                return chamfer_forward_mfma_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
-                                                      idx2, s, want[0], want[1]);
+                return chamfer_forward_mfma_launch<4, SOA>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                           dist2, idx2, s, want[0], want[1]);
         }
-        if (nkmin >= 512) {
+        if (!SOA && nkmin >= 512) {
             // Launch shapes: 4 queries per lane in 512-lane workgroups is the fastest
             // sweep once it fills the chip; below that 2 queries per lane in 256-lane
             // workgroups, with the key cloud cut into slices when even those are too few.
@@ -1817,10 +1862,10 @@ int chamfer_forward(const T *xyz1, const T *xyz2, int64_t B, int64_t N1, int64_t
         }
     }
     if (sizeof(T) == 8 || work < (int64_t)256 * 1024)
-        return chamfer_forward_launch<T, 2>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
-                                            idx2, s);
-    return chamfer_forward_launch<T, 4, 512, 64>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
-                                                 idx2, s);
+        return chamfer_forward_launch<T, 2, 256, 32, 1024, SOA>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                                dist2, idx2, s);
+    return chamfer_forward_launch<T, 4, 512, 64, 1024, SOA>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                            dist2, idx2, s);
 }
 
 // ---- fp32 forward on clouds sorted along a space-filling curve ---------------------
@@ -1896,6 +1941,7 @@ struct ChamferSortArgs {
     int B;
     int three_launches[2];  // this cloud is prepared by the cell, sort and tile kernels
                             // (beyond 16384 points); else by chamfer_prepare_kernel
+    int channels_first;     // the clouds are [B,3,N] (chamfer_prepare_kernel only)
 };
 
 __host__ __device__ constexpr int chamfer_morton5(int v)
@@ -1943,13 +1989,16 @@ __host__ __device__ constexpr int chamfer_hilbert15(unsigned x, unsigned y, unsi
 // of three, over nine points spread through the cloud; and `cap`, 16 times the typical
 // deviation of the nine from it (none, i.e. the nine coincide: no cap).
 __device__ __forceinline__ void chamfer_pilot(const float *__restrict__ P, int n, float (&pilot)[3],
-                                              float (&cap)[3])
+                                              float (&cap)[3], bool channels_first = false)
 {
     const float INF = __builtin_huge_valf();
     TkPoint3<float> q[9];
 #pragma unroll
-    for (int i = 0; i < 9; ++i)
-        q[i] = tk_load3<float>(P + (((int64_t)n * (2 * i + 1)) / 19) * 3);
+    for (int i = 0; i < 9; ++i) {
+        const int j = (int)(((int64_t)n * (2 * i + 1)) / 19);
+        q[i] = channels_first ? chamfer_point<true, float>(P, n, j)
+                              : chamfer_point<false, float>(P, n, j);
+    }
     auto ninther = [](float v0, float v1, float v2, float v3, float v4, float v5, float v6,
                       float v7, float v8) {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_fmed3f(v0, v1, v2),
@@ -2443,6 +2492,20 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
         // into one set of 48 registers that lives across the kernel)
         int t = tid;
         asm volatile("" : "+v"(t));
+        if (a.channels_first) {  // (uniform) a [3,N] cloud: one load per coordinate
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = u * NT + t;
+                const int at = (j < n ? j : n - 1) * 4;
+                p[u].x = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(cloud_rsrc, at, 0, 0));
+                p[u].y = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(cloud_rsrc, at, n * 4, 0));
+                p[u].z = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(cloud_rsrc, at, n * 8, 0));
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             typedef float f3 __attribute__((ext_vector_type(3)));
@@ -2457,7 +2520,7 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
 
     // ---- the pilot centre, the bounding box and the deviations ----
     float pilot[3], cap[3];
-    chamfer_pilot(P, n, pilot, cap);
+    chamfer_pilot(P, n, pilot, cap, a.channels_first != 0);
     for (int i = tid; i < WORDS / 4; i += NT)
         reinterpret_cast<uint4 *>(hist)[i] = make_uint4(0u, 0u, 0u, 0u);
     if (tid < 8)
@@ -3320,8 +3383,10 @@ __global__ __launch_bounds__(256) void chamfer_count_flags_kernel(const int *fla
 int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int64_t N1,
                            int64_t N2, float *dist1, int64_t *idx1, float *dist2, int64_t *idx2,
                            void *workspace, hipStream_t s, unsigned long long *counters = nullptr,
-                           int stages = 7)
+                           int stages = 7, bool channels_first = false)
 {
+    // ([3,N] clouds: read in place by chamfer_prepare_kernel and by the hand-over launch;
+    // the callers keep clouds of more than 16384 points away)
     // stages (tests and the benchmark time them apart): 1 the preparing launches, 2 the
     // pruned sweep, 4 the hand-over check
     constexpr int NQB = 2;
@@ -3350,6 +3415,7 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
     sa.hdr = reinterpret_cast<ChamferSortedHdr *>(ws + l.hdr);
     sa.flags = reinterpret_cast<int *>(ws + l.flags);
     sa.B = (int)B;
+    sa.channels_first = channels_first ? 1 : 0;
     pa.hdr = sa.hdr;
     pa.flags = sa.flags;
     pa.dist[0] = dist1;
@@ -3425,6 +3491,9 @@ int chamfer_forward_sorted(const float *xyz1, const float *xyz2, int64_t B, int6
         return TK3D_OK;
     // whatever the waves above handed over (none on ordinary input: its workgroups leave
     // at once)
+    if (channels_first)
+        return chamfer_forward_mfma_flagged_launch<4, true>(xyz1, xyz2, B, N1, N2, dist1, idx1,
+                                                            dist2, idx2, s, sa.flags);
     return chamfer_forward_mfma_flagged_launch<4>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2,
                                                   idx2, s, sa.flags);
 }
@@ -3603,6 +3672,30 @@ int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2, in
 {
     return chamfer_forward<double>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2,
                                    stream);
+}
+
+int tk3d_chamfer_distance_forward_bcn_f32(const float *xyz1, const float *xyz2, int64_t B,
+                                          int64_t N1, int64_t N2, float *dist1, int64_t *idx1,
+                                          float *dist2, int64_t *idx2, void *workspace,
+                                          size_t workspace_bytes, void *stream)
+{
+    // the sorted path where it serves and a workspace was lent, else the sweep of all pairs
+    if (workspace != nullptr && chamfer_sorted_can_serve(B, N1, N2) && N1 <= PREP_MAX_POINTS &&
+        N2 <= PREP_MAX_POINTS && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0 &&
+        workspace_bytes >= chamfer_sorted_layout(B, N1, N2).total) {
+        if (!xyz1 || !xyz2 || !dist1 || !idx1 || !dist2 || !idx2)
+            return TK3D_ERR_NULL_POINTER;
+        return chamfer_forward_sorted(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, workspace,
+                                      (hipStream_t)stream, nullptr, 7, true);
+    }
+    return chamfer_forward<float, true>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
+}
+
+int tk3d_chamfer_distance_forward_bcn_f64(const double *xyz1, const double *xyz2, int64_t B,
+                                          int64_t N1, int64_t N2, double *dist1, int64_t *idx1,
+                                          double *dist2, int64_t *idx2, void *stream)
+{
+    return chamfer_forward<double, true>(xyz1, xyz2, B, N1, N2, dist1, idx1, dist2, idx2, stream);
 }
 
 int tk3d_chamfer_distance_backward_f32(const float *grad_dist1, const float *grad_dist2,

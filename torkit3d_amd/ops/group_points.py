@@ -64,3 +64,5 @@ def group_points_with_xyz(feature, xyz, centre, index):
         index: [B, N2, K] int64.
     """
     return GroupPointsWithXYZFunction.apply(feature, xyz, centre, index)
+
+gather_points = group_points  # the spelling common elsewhere

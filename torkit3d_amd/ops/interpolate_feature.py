@@ -51,3 +51,5 @@ def three_nn_interpolation(query_xyz, key_xyz, transpose=False, eps=1e-10):
     """
     with torch.no_grad():
         return _fused.three_nn(query_xyz.contiguous(), key_xyz.contiguous(), bool(transpose), eps)
+
+three_interpolate = interpolate_feature  # the spelling common elsewhere

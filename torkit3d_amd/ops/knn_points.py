@@ -49,3 +49,5 @@ def knn_points(query, key, k, sorted=False, sqrt_distance=False, transpose=False
         distance, order = distance.sort(dim=2)
         index = index.gather(2, order)
     return (distance.sqrt() if sqrt_distance else distance), index
+
+knn_distance = knn_points  # the spelling of the compiled op (knn_distance_cuda)

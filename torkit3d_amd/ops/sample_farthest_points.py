@@ -42,3 +42,5 @@ def sample_farthest_points_gather(points, num_samples, transpose=False):
     with torch.no_grad():
         return _fused.sample_farthest_points_gather(points.contiguous(), num_samples,
                                                     bool(transpose))
+
+farthest_point_sample = sample_farthest_points  # the spelling common elsewhere
