@@ -140,11 +140,8 @@ int tk3d_knn_distance_f64(const double *query, const double *key, int64_t B,
 /* KNN on [B,3,N] clouds (query [B,3,N1], key [B,3,N2]), the layout the reference's
  * models hold: knn_points(..., transpose=True) copies both clouds to [B,N,3] before the
  * call (torkit3d/ops/knn_points.py:40-45). Same result as tk3d_knn_distance_* on the
- * transposed clouds, without the copies. Returns TK3D_ERR_UNSUPPORTED (nothing launched)
- * where copying and calling tk3d_knn_distance_* is the faster route or the only one, and
- * the caller then copies as the reference does: k > 64; in fp32 also k > 16, and
- * k = 5..16 on launches too small for the pre-filtered sweep (the LDS tree kernels that
- * serve those read [B,N,3] only). */
+ * transposed clouds, without the copies, for k <= 64. Returns TK3D_ERR_UNSUPPORTED (nothing
+ * launched) for k > 64: the caller then copies as the reference does. */
 int tk3d_knn_distance_bcn_f32(const float *query, const float *key, int64_t B,
                               int64_t N1, int64_t N2, int64_t k, int version,
                               float *distance, int64_t *index, void *stream);

@@ -412,9 +412,13 @@ def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("b,n1,n2,k", [(2, 700, 900, 3), (8, 8192 + 1, 2048 + 3, 4),   # pre-filtered
                                         (2, 300, 1000, 7), (16, 8192, 2048, 16),        # pre-filtered
-                                        (2, 300, 1000, 16), (1, 100, 9000, 6),           # copies
-                                        (1, 100, 500, 33), (1, 64, 300, 64), (1, 40, 200, 65)])
+                                        (2, 300, 1000, 16), (1, 100, 9000, 6),           # LDS tree
+                                        (8, 2048, 2048, 20),   # the k = 20 graph of DGCNN
+                                        (2, 500, 3000, 40), (1, 200, 70000, 12),
+                                        (1, 100, 500, 33), (1, 64, 300, 64),
+                                        (1, 40, 200, 65)])                               # copies
 def test_channels_first_clouds_are_read_in_place_or_copied(cuda, b, n1, n2, k, dtype):
+    # reference: knn_points(transpose=True), torkit3d/ops/knn_points.py:40-45
     # knn_points(transpose=True) on [B,3,N] clouds: same rows as on the [B,N,3] clouds
     from torkit3d_amd import _fused
     from torkit3d_amd.ops.knn_points import knn_points
@@ -428,15 +432,9 @@ def test_channels_first_clouds_are_read_in_place_or_copied(cuda, b, n1, n2, k, d
     np.testing.assert_array_equal(d.cpu().numpy(), od)
     np.testing.assert_array_equal(i.cpu().numpy(), oi)
     raw = _fused.knn_distance_bcn(qt, kt, k, 1)
-    # fp32: the library declines where its faster kernels only read [B,N,3] (k > 16, and
-    # k = 5..16 where the pre-filtered sweep does not pay: short key clouds, or few queries
-    # against a very long one); fp64: k > 64 only
-    if dtype == torch.float64:
-        declined = k > 64
-    else:
-        few_long = b * n1 < 32768 and n2 > (8192 if k <= 8 else 32768)
-        long_enough = n2 >= (512 if k <= 8 else 1024) or (n2 >= 512 and b * n1 >= 131072)
-        declined = k > 16 or (k > 4 and (few_long or not long_enough))
+    # the library reads [B,3,N] in place for every k <= 64 (fp32: the pre-filtered sweep, the
+    # register kernel or the LDS tree kernel); beyond it declines and the wrapper copies
+    declined = k > 64
     assert (raw is None) == declined
     if raw is not None:
         assert torch.equal(raw[0], d) and torch.equal(raw[1], i)

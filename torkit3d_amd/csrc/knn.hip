@@ -1065,7 +1065,7 @@ template <int KMAX, bool IDX16, typename T = float> struct KnnTreeLayout {
     static constexpr int BYTES = LEAF_BYTES + KIDX_BYTES + IVAL_BYTES + IARG_BYTES;
 };
 
-template <typename T, int KMAX, bool IDX16>
+template <typename T, int KMAX, bool IDX16, bool SOA = false>
 __global__ __launch_bounds__(64) void knn_tree_kernel(
     const T *__restrict__ query, const T *__restrict__ key,
     T *__restrict__ distance, int64_t *__restrict__ index, int blocks_per_batch, int n1,
@@ -1095,10 +1095,10 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
     const T *__restrict__ K = key + (int64_t)b * n2 * 3;
     T qx = 0, qy = 0, qz = 0;
     if (active) {
-        const T *q = query + ((int64_t)b * n1 + qi) * 3;
-        qx = q[0];
-        qy = q[1];
-        qz = q[2];
+        const T *__restrict__ Q = query + (int64_t)b * n1 * 3;
+        qx = knn_coord<SOA>(Q, n1, qi, 0);
+        qy = knn_coord<SOA>(Q, n1, qi, 1);
+        qz = knn_coord<SOA>(Q, n1, qi, 2);
     }
 
     // Value and first slot of a node whose children are leaves.
@@ -1115,7 +1115,8 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
     for (int s = 0; s < KMAX; ++s) {
         T d = -tk_inf<T>();
         if (s < k) {
-            d = tk_dist2<T>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+            d = tk_dist2<T>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                                knn_coord<SOA>(K, n2, s, 2), qx, qy, qz);
             if (d != d) {
                 frozen |= s == 0;
                 d = -tk_inf<T>();  // marks the slot: no real distance is -inf
@@ -1158,18 +1159,18 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
         };
         unsigned mask = 0u;
         if (first + CHUNK <= n2) {
-            const T *__restrict__ g = K + (int64_t)first * 3;
 #pragma unroll
-            for (int i = 0; i < CHUNK; ++i) {
-                const T d = tk_dist2<T>(g[3 * i + 0], g[3 * i + 1], g[3 * i + 2], qx,
-                                                qy, qz);
+            for (int i = 0; i < CHUNK; ++i) {  // (wave-uniform addresses: scalar loads)
+                const T d = tk_dist2<T>(knn_coord<SOA>(K, n2, first + i, 0),
+                                        knn_coord<SOA>(K, n2, first + i, 1),
+                                        knn_coord<SOA>(K, n2, first + i, 2), qx, qy, qz);
                 mask = below_max(mask, d);
             }
         } else {
             for (int i = 0; i < CHUNK; ++i) {
                 const int j = first + i < n2 ? first + i : n2 - 1;  // clamped, masked below
-                const T d = tk_dist2<T>(K[(int64_t)j * 3 + 0], K[(int64_t)j * 3 + 1],
-                                                K[(int64_t)j * 3 + 2], qx, qy, qz);
+                const T d = tk_dist2<T>(knn_coord<SOA>(K, n2, j, 0), knn_coord<SOA>(K, n2, j, 1),
+                                        knn_coord<SOA>(K, n2, j, 2), qx, qy, qz);
                 mask = below_max(mask, d);
             }
         }
@@ -1183,16 +1184,17 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
         mask &= valid;
 
         // ---- insertion rounds, the next candidate's key in flight during the current ----
-        const T *__restrict__ ck = K + (int64_t)first * 3;
         bool has = mask != 0u;
         int i = has ? __builtin_clz(mask) : 0;
-        T ex = ck[3 * i + 0], ey = ck[3 * i + 1], ez = ck[3 * i + 2];
+        T ex = knn_coord<SOA>(K, n2, first + i, 0), ey = knn_coord<SOA>(K, n2, first + i, 1),
+          ez = knn_coord<SOA>(K, n2, first + i, 2);
         while (__builtin_amdgcn_ballot_w64(has)) {  // wave-uniform
             mask &= ~(0x80000000u >> i);  // no-op for a lane without a candidate
             const bool has_next = mask != 0u;
             const int i_next = has_next ? __builtin_clz(mask) : 0;
-            const T nx = ck[3 * i_next + 0], ny = ck[3 * i_next + 1],
-                        nz = ck[3 * i_next + 2];
+            const T nx = knn_coord<SOA>(K, n2, first + i_next, 0),
+                    ny = knn_coord<SOA>(K, n2, first + i_next, 1),
+                    nz = knn_coord<SOA>(K, n2, first + i_next, 2);
             const T d = tk_dist2<T>(ex, ey, ez, qx, qy, qz);
             if (has && d < max_key) {
                 const int p = max_idx;
@@ -1242,7 +1244,8 @@ __global__ __launch_bounds__(64) void knn_tree_kernel(
         for (int s = 0; s < k; ++s) {
             T d = leaf[s * NT];
             if (d == -tk_inf<T>())  // a NaN of the fill phase, still in its slot
-                d = tk_dist2<T>(K[s * 3 + 0], K[s * 3 + 1], K[s * 3 + 2], qx, qy, qz);
+                d = tk_dist2<T>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                                knn_coord<SOA>(K, n2, s, 2), qx, qy, qz);
             od[s] = d;
             oi[s] = (int64_t)kidx[s * NT];
         }
@@ -1957,32 +1960,32 @@ int knn_tree_split_launch(const float *query, const float *key, float *distance,
     return launch(std::true_type{});
 }
 
-template <int KMAX, bool IDX16, typename T = float>
+template <int KMAX, bool IDX16, typename T = float, bool SOA = false>
 int knn_tree_launch_as(const T *query, const T *key, T *distance, int64_t *index,
                        int64_t B, int n1, int n2, int k, hipStream_t s)
 {
     constexpr int LDS_BYTES = KnnTreeLayout<KMAX, IDX16, T>::BYTES;
     if (LDS_BYTES > 48 * 1024) {
         const int allowed =
-            tk_allow_dynamic_lds<knn_tree_kernel<T, KMAX, IDX16>>(LDS_BYTES);
+            tk_allow_dynamic_lds<knn_tree_kernel<T, KMAX, IDX16, SOA>>(LDS_BYTES);
         if (allowed != TK3D_OK)
             return allowed;
     }
     const int64_t bpb = ((int64_t)n1 + 63) / 64;
     if (B * bpb > TK_MAX_I32)
         return TK3D_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((knn_tree_kernel<T, KMAX, IDX16>), dim3((unsigned)(B * bpb)), dim3(64),
+    hipLaunchKernelGGL((knn_tree_kernel<T, KMAX, IDX16, SOA>), dim3((unsigned)(B * bpb)), dim3(64),
                        LDS_BYTES, s, query, key, distance, index, (int)bpb, n1, n2, k);
     return tk_launch_status();
 }
 
-template <int KMAX, typename T = float>
+template <int KMAX, typename T = float, bool SOA = false>
 int knn_tree_launch(const T *query, const T *key, T *distance, int64_t *index,
                     int64_t B, int n1, int n2, int k, hipStream_t s)
 {
     if (n2 <= 65536)
-        return knn_tree_launch_as<KMAX, true, T>(query, key, distance, index, B, n1, n2, k, s);
-    return knn_tree_launch_as<KMAX, false, T>(query, key, distance, index, B, n1, n2, k, s);
+        return knn_tree_launch_as<KMAX, true, T, SOA>(query, key, distance, index, B, n1, n2, k, s);
+    return knn_tree_launch_as<KMAX, false, T, SOA>(query, key, distance, index, B, n1, n2, k, s);
 }
 
 // The tree kernel with the matrix-core sweep: pays where the launch fills the chip and the
@@ -2250,12 +2253,12 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
     return tk_launch_status();
 }
 
-// KNN on [B,3,N] clouds with the kernels that read either layout. Where knn() above would
-// pick a kernel that only reads [B,N,3] (the LDS tree kernels: fp32 with k > 16, or
-// k = 5..16 on launches the pre-filtered sweep does not pay for) this returns
-// TK3D_ERR_UNSUPPORTED before launching anything: copying the clouds and calling knn()
-// is the faster route there (k = 20, B=8, 2048 x 2048: 0.21 ms + copies against 0.27 ms
-// with the slots in registers). fp64 runs the same kernels on either layout, k <= 64.
+// KNN on [B,3,N] clouds with the kernels that read either layout, k <= 64 (beyond:
+// TK3D_ERR_UNSUPPORTED before anything is launched; the caller copies the clouds and calls
+// knn()). fp32: the pre-filtered sweep where knn() would launch it, the register kernel for
+// k <= 4, else the LDS tree kernel (the variants of it that share keys among several waves,
+// or sweep on the matrix cores, read [B,N,3] only). fp64 runs the same kernels on either
+// layout.
 template <typename T>
 int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t k,
             int version, T *distance, int64_t *index, void *stream)
@@ -2277,10 +2280,19 @@ int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int
         return TK3D_OK;
     if (!query || !key || !distance || !index)
         return TK3D_ERR_NULL_POINTER;
-    if (sizeof(T) == 4 && k > 4 && !knn_filter_takes(B, n1, n2, kk))
-        return TK3D_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if constexpr (sizeof(T) == 4) {
+        if (k > 4 && !knn_filter_takes(B, n1, n2, kk)) {
+            // k = 17..64, or a launch the pre-filtered sweep does not pay for: the LDS tree,
+            // reading the coordinate planes
+            if (k <= 8)
+                return knn_tree_launch<8, float, true>(query, key, distance, index, B, n1, n2, kk, s);
+            if (k <= 16)
+                return knn_tree_launch<16, float, true>(query, key, distance, index, B, n1, n2, kk, s);
+            if (k <= 32)
+                return knn_tree_launch<32, float, true>(query, key, distance, index, B, n1, n2, kk, s);
+            return knn_tree_launch<64, float, true>(query, key, distance, index, B, n1, n2, kk, s);
+        }
         int rc = TK3D_ERR_UNSUPPORTED;
         if (k <= 4) {
             rc = knn_filter_launch<4, true, false>(query, key, distance, index, nullptr, 0.0f, B,

@@ -15,9 +15,8 @@ class KNNDistanceFunction(NoGradient):
 
 
 class KNNDistanceChannelsFirstFunction(NoGradient):
-    """The same on [B,3,N] clouds, read in place where the library has a kernel for it (the
-    reference copies them to [B,N,3] first, torkit3d/ops/knn_points.py:40-45; so does this
-    for the k and launch sizes the library declines on this layout)."""
+    """The same on [B,3,N] clouds, read in place for k <= 64 (the reference copies them to
+    [B,N,3] first, torkit3d/ops/knn_points.py:40-45; so does this for larger k)."""
 
     @staticmethod
     def run(query_xyz, key_xyz, k, version):
