@@ -3240,15 +3240,18 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
         if (lane == 0)
             atomicAdd(a.counters + 2, (unsigned long long)(nover + nstray));
     }
-    // An exact scan costs about 13 instructions per two swept tiles (a normal wave issues
-    // 2100 in all): beyond 8192 (query, tile) pairs - half of what sweeping the whole cloud
-    // exactly would cost the wave - the cloud is handed to the other kernel (heavy ties:
-    // quantised or duplicated points).
-    if ((int64_t)nover * nswept > 8192) {
+    // An exact scan costs about 13 instructions per two swept tiles and query, a normal wave
+    // issues 2100 in all: beyond 2048 (query, tile) pairs - six times a wave's usual work - the
+    // cloud is handed to the other kernel (heavy ties: quantised or duplicated points; clouds
+    // of duplicated collinear points spent 0.9 ms here before the limit came down from 8192),
+    // and a wave whose cloud another wave has handed over meanwhile does not scan either.
+    if ((int64_t)nover * nswept > 2048) {
         if (lane == 0)
             hand_over();
         return;
     }
+    if (nover > 8 && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+        return;
     // ---- queries with three or more candidate tiles: exact scan of the swept tiles;
     //      stray queries: exact scan of all tiles ----
 #pragma unroll
