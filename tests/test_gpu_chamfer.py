@@ -172,15 +172,17 @@ def test_backward_with_an_empty_cloud_or_unmatched_points(cuda):
     assert float(gx1.abs().max()) == 0.0 and float(gx2.abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("where", [64, 300, 511, 5000 - 1])
-def test_backward_outlier_missed_by_the_magnitude_sample(cuda, where):
-    # The fixed-point scale comes from a sample of the senders (the first 64 of every 512);
-    # a term far above 8x the sampled maximum must send the workgroup through its second
-    # attempt with the exact bound.
+@pytest.mark.parametrize("n2,where", [(5000, 300), (20000, 1500), (20000, 19999), (70000, 8000)])
+def test_backward_outlier_missed_by_the_magnitude_sample(cuda, n2, where):
+    # The fixed-point scale comes from the terms of the first round of senders: runs of 1024
+    # consecutive senders, every rounds-th run, rounds = ceil(n2 / 8192). A term far above 8x
+    # that maximum in a later round must send the workgroup through its second attempt with
+    # the exact bound. (With 5000 senders there is one round and the bound is exact at once.)
     g = gen(3)
-    a, c = uniform_cloud(g, 2, 3000), uniform_cloud(g, 2, 5000)
-    gd1, gd2 = torch.randn(2, 3000, generator=g), torch.randn(2, 5000, generator=g)
-    assert where % 512 >= 64
+    a, c = uniform_cloud(g, 2, 3000), uniform_cloud(g, 2, n2)
+    gd1, gd2 = torch.randn(2, 3000, generator=g), torch.randn(2, n2, generator=g)
+    rounds = -(-n2 // 8192)
+    assert rounds == 1 or (where // 1024) % rounds != 0
     gd2[1, where] = 2.0e6
     _, i1, _, i2 = oracle.chamfer_forward(a.numpy(), c.numpy())
     check_backward(a, c, gd1, gd2, i1, i2, cuda)

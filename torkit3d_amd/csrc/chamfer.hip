@@ -1331,9 +1331,14 @@ __global__ __launch_bounds__(256) void chamfer_backward_scatter_kernel(
 // 64-bit fixed-point LDS accumulators (integer LDS atomics run an order of
 // magnitude faster than floating-point ones on this GPU, and make the sum
 // independent of arrival order), adds the own term and stores each gradient once.
-// Scale: a power of two chosen from a bound on |term| taken over a sample of the
-// senders times 64; a term above the bound raises a flag and the workgroup repeats
-// with the bound over all senders. Non-finite input takes the floating-point path.
+// The senders are taken in rounds of NT * U, a round being U runs of NT consecutive
+// senders spread evenly over the cloud. Scale: a power of two chosen from the largest
+// |term| of the first round's senders times 8 (those terms are in registers by then,
+// so the choice costs no pass of its own); a term above that bound raises a flag and
+// the workgroup repeats with the bound over all senders. Non-finite input takes the
+// floating-point path.
+// The own terms are fetched first, while the accumulators are cleared and the first
+// match indices arrive, and meet the sums at the end.
 template <int R, int NT>
 __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     const float *__restrict__ gd1, const float *__restrict__ gd2,
@@ -1341,10 +1346,14 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     const int64_t *__restrict__ idx1, const int64_t *__restrict__ idx2, int n1, int n2,
     int ranges1, int ranges2, float *__restrict__ gx1, float *__restrict__ gx2)
 {
-    extern __shared__ __align__(16) unsigned long long acc[];  // [R * 3]
+    extern __shared__ __align__(16) unsigned long long acc[];  // [R * 3], then the range
+    float *sx = reinterpret_cast<float *>(acc + R * 3);        // of X itself: [R * 3] floats
     __shared__ unsigned s_max;
     __shared__ int s_exceeded;
     const double MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+    constexpr int U = 8;           // senders per lane and round
+    constexpr int F = R / NT;      // points of the range per lane
+    static_assert(R % NT == 0 && R * 3 % (2 * NT) == 0, "whole steps of the workgroup");
 
     // Decode: a batch's ranges1 + ranges2 workgroups are consecutive logical workgroups
     // (first those that produce grad_xyz1), and each XCD takes a contiguous run of logical
@@ -1357,6 +1366,7 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
         if (lb < full)
             lb = (lb & 7) * per + (lb >> 3);
     }
+    const int tid = threadIdx.x;
     const int b = lb / (ranges1 + ranges2);
     const int r = lb - b * (ranges1 + ranges2);
     const bool second = r >= ranges1;
@@ -1374,178 +1384,288 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
     const int64_t *__restrict__ iY = (second ? idx1 : idx2) + (int64_t)b * ny;
     float *__restrict__ out = (second ? gx2 : gx1) + (int64_t)b * nx * 3;
     const int j1 = (j0 + R < nx) ? j0 + R : nx;
+    const int rounds = (ny + NT * U - 1) / (NT * U);
 
-    bool use_float = false;
-    for (int attempt = 0; attempt < 2; ++attempt) {  // uniform over the workgroup
+    // Everything is fetched through buffer descriptors: a 32-bit offset per element against
+    // a base in scalar registers, where 64-bit addresses for the gathers of a round would
+    // not fit the register file beside the data (the host sends clouds whose byte offsets
+    // pass 2^31 to the other kernels).
+    auto rsrc = [](const void *p, int64_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t rX = rsrc(X, (int64_t)nx * 12);
+    const __amdgpu_buffer_rsrc_t rY = rsrc(Y, (int64_t)(ny > 0 ? ny : 1) * 12);
+    const __amdgpu_buffer_rsrc_t rgX = rsrc(gX, (int64_t)nx * 4);
+    const __amdgpu_buffer_rsrc_t rgY = rsrc(gY, (int64_t)ny * 4);
+    const __amdgpu_buffer_rsrc_t riX = rsrc(iX, (int64_t)nx * 8);
+    const __amdgpu_buffer_rsrc_t riY = rsrc(iY, (int64_t)ny * 8);
+    typedef float f3 __attribute__((ext_vector_type(3)));
+    auto load_f = [](__amdgpu_buffer_rsrc_t rs, int at) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, at, 0, 0));
+    };
+    auto load_f3 = [](__amdgpu_buffer_rsrc_t rs, int at) {
+        return __builtin_bit_cast(f3, __builtin_amdgcn_raw_buffer_load_b96(rs, at, 0, 0));
+    };
+    auto load_i64 = [](__amdgpu_buffer_rsrc_t rs, int at) {
+        return __builtin_bit_cast(int64_t, __builtin_amdgcn_raw_buffer_load_b64(rs, at, 0, 0));
+    };
+
+    // Sender u of a lane in round `round`: runs of NT consecutive senders, the rounds
+    // interleaved so that each of them is spread over the whole cloud.
+    auto sender = [&](int round, int u) { return tid + NT * (u * rounds + round); };
+    // A sender's match as a position within the range, -1 when it lies outside.
+    auto load_matches = [&](int round, int (&jj)[U]) {
+        int64_t m64[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = sender(round, u);
+            m64[u] = load_i64(riY, (i < ny ? i : 0) * 8);
+            m64[u] = i < ny ? m64[u] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            jj[u] = (m64[u] >= j0 && m64[u] < j1) ? (int)(m64[u] - j0) : -1;
+    };
+    // The negated terms of a round's senders that match inside the range. Senders that
+    // match outside it read one fixed element instead (a broadcast), so only the index
+    // stream is paid for per range; everything is requested before anything is used. The
+    // matched points come from the copy of the range in LDS: fetched from memory, each of
+    // these 12-byte reads at a random place pulled a cache line of 128 bytes into the
+    // compute unit, and that traffic was what the kernel waited for.
+    auto load_terms = [&](int round, const int (&jj)[U], float (&v)[U][3]) {
+        float g[U];
+        f3 y[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int is = jj[u] >= 0 ? sender(round, u) : 0;
+            g[u] = load_f(rgY, is * 4) * 2;
+            y[u] = load_f3(rY, is * 12);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float *x = sx + (jj[u] >= 0 ? jj[u] : 0) * 3;  // the matched point, from LDS
+            v[u][0] = -(g[u] * (y[u].x - x[0]));
+            v[u][1] = -(g[u] * (y[u].y - x[1]));
+            v[u][2] = -(g[u] * (y[u].z - x[2]));
+        }
+    };
+    // Adds a round's terms to the accumulators; true when one of them is above the bound.
+    auto accumulate = [&](const int (&jj)[U], const float (&v)[U][3], float bound,
+                          double scale) {
+        bool exceeded = false;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (jj[u] < 0)
+                continue;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                exceeded = exceeded || !(__builtin_fabsf(v[u][a]) <= bound);
+                const double d = __builtin_fma((double)v[u][a], scale, MAGIC);
+                atomicAdd(&acc[jj[u] * 3 + a],
+                          __builtin_bit_cast(unsigned long long, d) -
+                              __builtin_bit_cast(unsigned long long, MAGIC));
+            }
+        }
+        return exceeded;
+    };
+    auto clear = [&]() {
         __syncthreads();
-        for (int t = threadIdx.x; t < R * 3; t += NT)
-            acc[t] = 0ull;
-        if (threadIdx.x == 0) {
+        for (int t = tid; t < R * 3 / 2; t += NT)
+            reinterpret_cast<ulonglong2 *>(acc)[t] = make_ulonglong2(0ull, 0ull);
+        if (tid == 0) {
             s_max = 0u;
             s_exceeded = 0;
         }
-        __syncthreads();
-        // bound on |term| over the senders: every 8th run of 64 consecutive senders on
-        // the first attempt (coalesced), all of them on the second. The match indices
-        // of U senders are fetched together so their latencies overlap.
-        constexpr int U = 8;
-        unsigned m = 0u;
-        const int nsample = attempt == 0 ? (ny + 7) / 8 : ny;
-        for (int s0 = threadIdx.x; s0 < nsample; s0 += NT * U) {
-            int64_t jj[U];
-            int ii[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int sidx = s0 + u * NT;
-                const int i = attempt == 0 ? (sidx >> 6) * 512 + (sidx & 63) : sidx;
-                ii[u] = (sidx < nsample && i < ny) ? i : -1;
-                jj[u] = ii[u] >= 0 ? iY[ii[u]] : -1;
-            }
-            float g[U], y[U][3], x[U][3];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const bool ok = jj[u] >= 0 && jj[u] < nx;
-                const int is = ok ? ii[u] : 0;
-                g[u] = ok ? gY[is] * 2 : 0.0f;
-#pragma unroll
-                for (int a = 0; a < 3; ++a) {
-                    y[u][a] = Y[(int64_t)is * 3 + a];
-                    x[u][a] = X[(ok ? jj[u] : 0) * 3 + a];
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (jj[u] < 0 || jj[u] >= nx)
-                    continue;
-#pragma unroll
-                for (int a = 0; a < 3; ++a) {
-                    const float v = g[u] * (y[u][a] - x[u][a]);
-                    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7fffffffu;
-                    m = bits > m ? bits : m;
-                }
-            }
-        }
-        // one LDS atomic per wave: 64 lanes on one address would be served one by one
+    };
+    // one LDS atomic per wave: 64 lanes on one address would be served one by one
+    auto workgroup_max = [&](unsigned m) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const unsigned t = (unsigned)__shfl_xor((int)m, o);
             m = t > m ? t : m;
         }
-        if ((threadIdx.x & 63) == 0 && m != 0u)
+        if ((tid & 63) == 0 && m != 0u)
             atomicMax(&s_max, m);
         __syncthreads();
-        const float bound = __builtin_bit_cast(float, s_max) * (attempt == 0 ? 8.0f : 1.000001f);
-        if (!(bound < 3.0e38f)) {  // NaN or inf
-            use_float = true;
-            break;
-        }
+        return s_max;
+    };
+    // The power of two that places a term at the bound below 2^50 and leaves room for up to
+    // 2^12 of them (more senders than that on one point lower the scale further).
+    auto scale_exponent = [&](float bound) {
         int e = 0;
         (void)__builtin_frexpf(bound, &e);
-        // a term below 2^50, and up to 2^12 of them (more senders than that on one
-        // point lower the scale further below)
         int log2_count = 1;
         while ((1 << log2_count) < ny + 1)
             ++log2_count;
-        const int kexp = (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
-        const double scale = __builtin_ldexp(1.0, kexp);
+        return (62 - log2_count < 50 ? 62 - log2_count : 50) - e;
+    };
 
-        bool exceeded = false;
-        for (int i0 = threadIdx.x; i0 < ny; i0 += NT * U) {
-            // Everything a sender needs is requested before anything is used: U
-            // match indices, then U gradients and 2U points, all in flight together.
-            int64_t jj[U];
-            float g[U], y[U][3], x[U][3];
+    // ---- the own terms: F points per lane --------------------------------------------------
+    float own[F][3];
+    int jj[U];
+    {
+        int mj[F];  // the point's own match, -1 when it has none
+        f3 xs[F];
+        {
+            int64_t m64[F];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = i0 + u * NT;
-                jj[u] = i < ny ? iY[i] : -1;
+            for (int f = 0; f < F; ++f) {
+                const int j = j0 + tid + f * NT;
+                m64[f] = load_i64(riX, (j < j1 ? j : j0) * 8);
+                m64[f] = j < j1 ? m64[f] : -1;
             }
+            // the lane's points of the range: for its own terms and into LDS for everyone
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = i0 + u * NT;
-                // Senders that match outside the range read one fixed element instead
-                // (a broadcast), so only the index stream is paid for per range.
-                const bool in = jj[u] >= j0 && jj[u] < j1;
-                const int64_t js = in ? jj[u] : (int64_t)j0;
-                const int is = in ? i : 0;
-                g[u] = gY[is] * 2;
-#pragma unroll
-                for (int a = 0; a < 3; ++a) {
-                    y[u][a] = Y[(int64_t)is * 3 + a];
-                    x[u][a] = X[js * 3 + a];
-                }
+            for (int f = 0; f < F; ++f) {
+                const int j = j0 + tid + f * NT;
+                xs[f] = load_f3(rX, (j < j1 ? j : j0) * 12);
             }
+            if (rounds > 0)
+                load_matches(0, jj);
+            clear();
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                mj[f] = (m64[f] >= 0 && m64[f] < ny) ? (int)m64[f] : -1;
+                float *at = sx + (tid + f * NT) * 3;
+                at[0] = xs[f].x;
+                at[1] = xs[f].y;
+                at[2] = xs[f].z;
+            }
+        }
+        __syncthreads();
+        float gg[F];
+        f3 ys[F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            const int j = j0 + tid + f * NT;
+            gg[f] = load_f(rgX, (j < j1 ? j : j0) * 4);
+            ys[f] = load_f3(rY, (mj[f] >= 0 ? mj[f] : 0) * 12);
+        }
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            own[f][0] = mj[f] >= 0 ? (gg[f] * 2) * (xs[f].x - ys[f].x) : 0.0f;
+            own[f][1] = mj[f] >= 0 ? (gg[f] * 2) * (xs[f].y - ys[f].y) : 0.0f;
+            own[f][2] = mj[f] >= 0 ? (gg[f] * 2) * (xs[f].z - ys[f].z) : 0.0f;
+        }
+    }
+    // Own term and the exact sum of the sent terms meet in double: the gradient is rounded
+    // once. A lane stores the 12 bytes of a point at once, so a wave's store covers 768
+    // consecutive bytes.
+    auto finish = [&](int kexp) {
+        const __amdgpu_buffer_rsrc_t rout = rsrc(out, (int64_t)nx * 12);
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            const int p = tid + f * NT;
+            if (j0 + p >= j1)
+                continue;
+            // (kept as three floats until here: converted where they were computed, they
+            // would occupy twice the registers through the whole scan)
+            asm volatile("" : "+v"(own[f][0]), "+v"(own[f][1]), "+v"(own[f][2]));
+            f3 o;
+            o.x = (float)((double)own[f][0] +
+                          __builtin_ldexp((double)(long long)acc[p * 3 + 0], -kexp));
+            o.y = (float)((double)own[f][1] +
+                          __builtin_ldexp((double)(long long)acc[p * 3 + 1], -kexp));
+            o.z = (float)((double)own[f][2] +
+                          __builtin_ldexp((double)(long long)acc[p * 3 + 2], -kexp));
+            typedef unsigned u3 __attribute__((ext_vector_type(3)));
+            __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u3, o), rout, (j0 + p) * 12, 0,
+                                                  0);
+        }
+    };
+
+    // ---- first attempt: the bound comes from the first round ------------------------------
+    {
+        float v[U][3];
+        int jn[U];
+        unsigned m = 0u;
+        if (rounds > 0) {
+            load_terms(0, jj, v);
+            if (rounds > 1)
+                load_matches(1, jn);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (jj[u] < j0 || jj[u] >= j1)
+                if (jj[u] < 0)
                     continue;
 #pragma unroll
                 for (int a = 0; a < 3; ++a) {
-                    const float v = -(g[u] * (y[u][a] - x[u][a]));
-                    exceeded = exceeded || !(__builtin_fabsf(v) <= bound);
-                    const double d = __builtin_fma((double)v, scale, MAGIC);
-                    atomicAdd(&acc[(jj[u] - j0) * 3 + a],
-                              __builtin_bit_cast(unsigned long long, d) -
-                                  __builtin_bit_cast(unsigned long long, MAGIC));
+                    const unsigned bits = __builtin_bit_cast(unsigned, v[u][a]) & 0x7fffffffu;
+                    m = bits > m ? bits : m;
                 }
             }
         }
-        if (exceeded)
-            s_exceeded = 1;
-        __syncthreads();
-        if (!s_exceeded) {
-            // own terms: a lane takes whole points, F of them per round, with the
-            // match indices and then the matched points fetched together
-            constexpr int F = 4;
-            for (int p0 = threadIdx.x; p0 < j1 - j0; p0 += NT * F) {
-                int64_t mj[F];
+        const float bound = __builtin_bit_cast(float, workgroup_max(m)) * 8.0f;
+        if (bound < 3.0e38f) {  // (else NaN or inf: floating point below)
+            const int kexp = scale_exponent(bound);
+            const double scale = __builtin_ldexp(1.0, kexp);
+            bool exceeded = false;
+            for (int round = 0; round < rounds; ++round) {
+                exceeded = accumulate(jj, v, bound, scale) || exceeded;
+                if (round + 1 < rounds) {
 #pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const int p = p0 + f * NT;
-                    mj[f] = p < j1 - j0 ? iX[j0 + p] : -1;
-                }
-                float gg[F], xs[F][3], ys[F][3];
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const int p = p0 + f * NT;
-                    const int j = j0 + (p < j1 - j0 ? p : 0);
-                    const bool ok = mj[f] >= 0 && mj[f] < ny;
-                    gg[f] = ok ? gX[j] * 2 : 0.0f;
-#pragma unroll
-                    for (int a = 0; a < 3; ++a) {
-                        xs[f][a] = X[(int64_t)j * 3 + a];
-                        ys[f][a] = Y[(ok ? mj[f] : 0) * 3 + a];
-                    }
-                }
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const int p = p0 + f * NT;
-                    if (p >= j1 - j0)
-                        continue;
-                    const bool ok = mj[f] >= 0 && mj[f] < ny;
-#pragma unroll
-                    for (int a = 0; a < 3; ++a) {
-                        const float own = ok ? gg[f] * (xs[f][a] - ys[f][a]) : 0.0f;
-                        // own term and the exact sum of the sent terms meet in double:
-                        // the gradient is rounded once
-                        const double sent =
-                            __builtin_ldexp((double)(long long)acc[p * 3 + a], -kexp);
-                        out[(int64_t)(j0 + p) * 3 + a] = (float)((double)own + sent);
-                    }
+                    for (int u = 0; u < U; ++u)
+                        jj[u] = jn[u];
+                    load_terms(round + 1, jj, v);
+                    if (round + 2 < rounds)
+                        load_matches(round + 2, jn);
                 }
             }
-            return;
+            if (exceeded)
+                s_exceeded = 1;
+            __syncthreads();
+            if (!s_exceeded) {
+                finish(kexp);
+                return;
+            }
         }
     }
-    (void)use_float;
+    // ---- second attempt: the bound over all senders ---------------------------------------
+    {
+        clear();
+        __syncthreads();
+        unsigned m = 0u;
+        float v[U][3];
+        for (int round = 0; round < rounds; ++round) {
+            load_matches(round, jj);
+            load_terms(round, jj, v);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (jj[u] < 0)
+                    continue;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    const unsigned bits = __builtin_bit_cast(unsigned, v[u][a]) & 0x7fffffffu;
+                    m = bits > m ? bits : m;
+                }
+            }
+        }
+        const float bound = __builtin_bit_cast(float, workgroup_max(m)) * 1.000001f;
+        if (bound < 3.0e38f) {
+            const int kexp = scale_exponent(bound);
+            const double scale = __builtin_ldexp(1.0, kexp);
+            bool exceeded = false;
+            for (int round = 0; round < rounds; ++round) {
+                load_matches(round, jj);
+                load_terms(round, jj, v);
+                exceeded = accumulate(jj, v, bound, scale) || exceeded;
+            }
+            if (exceeded)
+                s_exceeded = 1;
+            __syncthreads();
+            if (!s_exceeded) {
+                finish(kexp);
+                return;
+            }
+        }
+    }
 
     // Non-finite gradients or coordinates: floating-point LDS accumulation.
     float *facc = reinterpret_cast<float *>(acc);
     __syncthreads();
-    for (int t = threadIdx.x; t < R * 3; t += NT)
+    for (int t = tid; t < R * 3; t += NT)
         facc[t] = 0.0f;
     __syncthreads();
-    for (int i = threadIdx.x; i < ny; i += NT) {
+    for (int i = tid; i < ny; i += NT) {
         const int64_t j = iY[i];
         if (j < j0 || j >= j1)
             continue;
@@ -1555,13 +1675,13 @@ __global__ __launch_bounds__(NT) void chamfer_backward_fixed_kernel(
             atomicAdd(&facc[(j - j0) * 3 + a], -(g * (Y[(int64_t)i * 3 + a] - X[j * 3 + a])));
     }
     __syncthreads();
-    for (int t = threadIdx.x; t < (j1 - j0) * 3; t += NT) {
+    for (int t = tid; t < (j1 - j0) * 3; t += NT) {
         const int j = j0 + t / 3, a = t - (t / 3) * 3;
-        const int64_t jj = iX[j];
-        float own = 0.0f;
-        if (jj >= 0 && jj < ny)
-            own = (gX[j] * 2) * (X[(int64_t)j * 3 + a] - Y[jj * 3 + a]);
-        out[(int64_t)j * 3 + a] = own + facc[t];
+        const int64_t jm = iX[j];
+        float o = 0.0f;
+        if (jm >= 0 && jm < ny)
+            o = (gX[j] * 2) * (X[(int64_t)j * 3 + a] - Y[jm * 3 + a]);
+        out[(int64_t)j * 3 + a] = o + facc[t];
     }
 }
 
@@ -3521,12 +3641,13 @@ int chamfer_backward(const T *gd1, const T *gd2, const T *xyz1, const T *xyz2,
     hipStream_t s = (hipStream_t)stream;
     if constexpr (sizeof(T) == 4) {
         // Every range scans all senders of its batch, so ranges are as long as LDS
-        // allows: 4096 points x 3 x 8 bytes = 96 KiB.
+        // allows: 4096 points x 3 x (8 bytes of accumulator + 4 of the point) = 144 KiB.
         constexpr int R = 4096, NT = 1024;
         const int64_t r1 = (N1 + R - 1) / R, r2 = (N2 + R - 1) / R;
-        if (B * (r1 + r2) <= TK_MAX_I32) {
+        // (the kernel addresses a cloud with 32-bit byte offsets: 12 bytes a point)
+        if (B * (r1 + r2) <= TK_MAX_I32 && N1 <= (1 << 27) && N2 <= (1 << 27)) {
             constexpr auto kernel = chamfer_backward_fixed_kernel<R, NT>;
-            constexpr size_t lds = (size_t)R * 3 * sizeof(unsigned long long);
+            constexpr size_t lds = (size_t)R * 3 * (sizeof(unsigned long long) + sizeof(float));
             const int allowed = tk_allow_dynamic_lds<kernel>((int)lds);
             if (allowed != TK3D_OK)
                 return allowed;
