@@ -305,7 +305,7 @@ def secondary_metrics(dev, steps, warmup, cpu):
     """
     import torch
 
-    from torkit3d_amd import _C
+    from torkit3d_amd import _C, _lib
     from torkit3d_amd.ops.interpolate_feature import three_nn_weights
 
     out = {}
@@ -387,8 +387,19 @@ def secondary_metrics(dev, steps, warmup, cpu):
     _, i1, _, i2 = _C.chamfer_distance_forward_cuda(a, c)
     gd1 = torch.randn(32, 16384, generator=g).to(dev)
     gd2 = torch.randn(32, 16384, generator=g).to(dev)
-    out["chamfer_bwd_B32_N16384_ms"] = gpu_time_ms(
-        lambda: _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2), steps, warmup)
+    # (through the C-ABI on outputs allocated once: the Python wrapper's argument checks take
+    # about as long as this kernel runs, and the events would time the host)
+    gx1, gx2 = torch.empty_like(a), torch.empty_like(c)
+    want = _C.chamfer_distance_backward_cuda(gd1, gd2, a, c, i1, i2)
+
+    def chamfer_bwd():
+        _lib.call("tk3d_chamfer_distance_backward", a, _lib.ptr(gd1), _lib.ptr(gd2), _lib.ptr(a),
+                  _lib.ptr(c), _lib.ptr(i1), _lib.ptr(i2), _lib.i64(32), _lib.i64(16384),
+                  _lib.i64(16384), _lib.ptr(gx1), _lib.ptr(gx2), _lib.stream_of(a))
+
+    out["chamfer_bwd_B32_N16384_ms"] = gpu_time_ms(chamfer_bwd, steps, warmup)
+    if not (torch.equal(gx1, want[0]) and torch.equal(gx2, want[1])):
+        sys.exit("bench.py: chamfer backward through the C-ABI differs from the wrapper's result")
     if cpu:
         ca, cc = a[:4].cpu().numpy(), c[:4].cpu().numpy()
         cg1, cg2 = gd1[:4].cpu().numpy(), gd2[:4].cpu().numpy()
@@ -621,6 +632,10 @@ def main():
                     help="time only the chamfer step (for profiler runs)")
     ap.add_argument("--models-only", action="store_true",
                     help="time only the model zoo's passes and print those (for profiler runs)")
+    ap.add_argument("--step-only", action="store_true",
+                    help="run the warm-up and the timed steps of the chamfer call and nothing "
+                         "else, and print a short line (for profiler runs whose per-kernel "
+                         "figures must cover the timed step alone)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy, whose known traffic "
                          "scales the profiler's FETCH_SIZE / WRITE_SIZE counters")
@@ -667,6 +682,13 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     kernel_ms = start.elapsed_time(stop) / args.steps  # the launches of one step, back to back
+
+    if args.step_only:
+        print(json.dumps({"metric": "chamfer pair-dists/s at B=32,N=M=16384",
+                          "value": 2.0 * B * N * M / (wall_ms * 1e-3), "unit": "pair-dists/s",
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms,
+                          "kernel_ms": kernel_ms}))
+        return
 
     # the same clouds through the entry point that evaluates every pair (one launch)
     full_out = [torch.empty_like(t) for t in out]

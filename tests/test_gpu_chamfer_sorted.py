@@ -136,6 +136,27 @@ def test_disjoint_and_nested_clouds(cuda):
     assert sum(handed_over(ws, 2)) == 0
 
 
+def test_keys_crowded_into_few_cells_are_handed_over(cuda):
+    # A few hundred distinct points on a line, each repeated about 50 times: over a hundred
+    # keys per occupied cell of the 32^3 grid, several tiles of equal keys in front of every
+    # query. Both directions go to the sweep of all pairs before any wave sweeps; the same
+    # repetition spread over a volume (about 50 keys per occupied cell) stays.
+    g = gen(21)
+    n = 8192
+    t = torch.rand(2, n // 50, 1, generator=g) * torch.tensor([1.0, 0.5, -0.25])
+    pick1 = torch.randint(0, n // 50, (n,), generator=g)
+    pick2 = torch.randint(0, n // 50, (n,), generator=g)
+    ws = check_sorted(t[:, pick1].contiguous(), t[:, pick2].contiguous(), cuda)
+    assert handed_over(ws, 2) == [1, 1, 1, 1]
+    v = sphere_cloud(g, 2, n // 50)
+    ws = check_sorted(v[:, pick1].contiguous(), v[:, pick2].contiguous(), cuda)
+    assert sum(handed_over(ws, 2)) == 0
+    # points on a line without repetition: crowded as well (a cell holds 8192 / ~50 keys)
+    line = torch.rand(2, n, 1, generator=g) * torch.tensor([1.0, 0.5, -0.25])
+    ws = check_sorted(line, line.flip(1).contiguous() + 1e-3, cuda)
+    assert handed_over(ws, 2) == [1, 1, 1, 1]
+
+
 def test_workspace_contract(cuda):
     from torkit3d_amd import _lib
 

@@ -1236,9 +1236,12 @@ chamfer_forward_mfma_flagged_kernel(ChamferFwdArgs<float> args, int total)
 {
     if (args.only_if[2 * args.nbatch] == 0)  // no cloud carries a flag: nothing to do
         return;
+    // Shares of the two directions alternate (as far as the shorter one reaches): often only
+    // one direction carries flags, and its workgroups should not be neighbours on the chip.
+    const int n0 = args.nblocks0, n1 = total - args.nblocks0, both = n0 < n1 ? n0 : n1;
     for (int lb = blockIdx.x; lb < total; lb += gridDim.x) {
-        const int which = lb >= args.nblocks0;
-        const int rest0 = lb - (which ? args.nblocks0 : 0);
+        const int which = lb < 2 * both ? (lb & 1) : (n0 > n1 ? 0 : 1);
+        const int rest0 = lb < 2 * both ? (lb >> 1) : lb - both;
         const ChamferDir<float> &d = args.dir[which];
         const int b = rest0 / d.blocks_per_batch;
         const int rest = rest0 - b * d.blocks_per_batch;
@@ -2045,7 +2048,8 @@ struct ChamferSortedHdr {  // 64 bytes per cloud and batch element
     float lo[3], hi[3];    // bounding box of all points, caller's units
     float extent;          // largest extent of the frame, caller's units
     int far_keys;          // keys beyond 4 units of the frame, kept on a list of their own
-    int pad[2];
+    int occupied;          // cells of the 32^3 grid that hold a point
+    int pad;
 };
 
 struct ChamferSortArgs {
@@ -2304,6 +2308,7 @@ __global__ __launch_bounds__(1024) void chamfer_cell_kernel(ChamferSortArgs a)
         hdr->unsafe = safe ? 0 : 1;
         hdr->extent = 2.0f * ext;
         hdr->far_keys = 0;
+        hdr->occupied = 0x7fffffff;  // (not counted on this route: never "crowded")
 #pragma unroll
         for (int ax = 0; ax < 3; ++ax) {
             hdr->lo[ax] = lo[ax];
@@ -2783,18 +2788,22 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     // position is looked up.
     {
         constexpr int PER_WAVE = WORDS / NW;
-        int carry = 0;
+        int carry = 0, occupied = 0;
         for (int i = 0; i < PER_WAVE; i += TK_WAVE) {
             const int at = wave * PER_WAVE + i + lane;
             const unsigned both = hist[at];
             const int even = (int)(both & 0xffffu), odd = (int)(both >> 16);
+            occupied += (even != 0) + (odd != 0);
             const int incl = wave_inclusive_sum(even + odd);
             const int start = carry + incl - (even + odd);
             hist[at] = (unsigned)start | ((unsigned)(start + even) << 16);
             carry += __builtin_amdgcn_readlane(incl, TK_WAVE - 1);
         }
-        if (lane == 0)
+        occupied = __builtin_amdgcn_readlane(wave_inclusive_sum(occupied), TK_WAVE - 1);
+        if (lane == 0) {
             swave[wave] = carry;
+            sred[wave][1] = (float)occupied;  // (at most 2048: exact)
+        }
     }
     __syncthreads();
     if (tid <= NW) {
@@ -2806,12 +2815,15 @@ __global__ __launch_bounds__(1024) void chamfer_prepare_kernel(ChamferSortArgs a
     if (part == 0) {  // what belongs to the cloud as a whole leaves with its first workgroup
         const int nfar = sfar;
         if (tid == 0) {
-            float m = 0.0f;
+            float m = 0.0f, cells = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW; ++w)
+            for (int w = 0; w < NW; ++w) {
                 m = __builtin_fmaxf(m, sred[w][0]);
+                cells += sred[w][1];
+            }
             hdr->kmax2_bits = __builtin_bit_cast(int, m);
             hdr->far_keys = nfar;
+            hdr->occupied = (int)cells;
         }
         if (tid < nfar && tid < CHAMFER_FAR_KEYS)
             a.far_keys[which][(int64_t)b * CHAMFER_FAR_KEYS + tid] = sfar_list[tid];
@@ -3044,8 +3056,11 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // this kernel would sweep all pairs at four times the matrix kernel's cost per tile.
     const bool dwarfed = ntiles >= 16 && hk->extent < 0.25f * hq->extent;
     const int nfar = hk->far_keys;  // keys kept out of the sweep (far outside the frame)
+    // (What follows from the headers alone is the same for every wave of the cloud: its
+    // first wave raises the flag, the others just leave - thousands of atomics on one word
+    // took 50 us.)
     if (hq->unsafe != 0 || hk->unsafe != 0) {  // uniform over the wave
-        if (lane == 0)
+        if (lane == 0 && qw == 0)
             hand_over();
         return;
     }
@@ -3069,8 +3084,13 @@ __global__ __launch_bounds__(256) void chamfer_pruned_kernel(ChamferPrunedArgs a
     // have an absolute floor): a frame that outliers stretched far beyond the bulk of the
     // keys does not give one.
     const bool flat_terms = hk->kmax2_bits < 0x3d800000;  // |k'|^2 < 1/16 for every swept key
-    if (!(far2 <= 6.4e7f) || dwarfed || flat_terms || nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
-        if (lane == 0)
+    // Keys crowded into few cells - over a hundred per occupied cell: points on a line, or a
+    // few hundred distinct points repeated - put several tiles of equal or nearly equal keys
+    // in front of every query; the exact scans that follow cost more than all pairs do.
+    const bool crowded = ntiles >= 16 && (int64_t)hk->occupied * 128 < a.n[1 - which];
+    if (!(far2 <= 6.4e7f) || dwarfed || flat_terms || crowded ||
+        nfar > CHAMFER_FAR_KEYS) {  // uniform over the wave
+        if (lane == 0 && qw == 0)
             hand_over();
         return;
     }
