@@ -73,8 +73,9 @@ int tk3d_chamfer_distance_forward_f64(const double *xyz1, const double *xyz2,
  * scratch memory. With `workspace` (256-byte aligned device memory of at least
  * tk3d_chamfer_distance_forward_workspace_bytes(B, N1, N2, 1) bytes, contents irrelevant
  * before and after) both clouds are first sorted along a space-filling curve, and a wave
- * then sweeps only the key tiles that can hold a nearest neighbour of its queries; five
- * kernels are enqueued. Results are bit-identical to tk3d_chamfer_distance_forward_f32 for
+ * then sweeps only the key tiles that can hold a nearest neighbour of its queries; three
+ * kernels are enqueued (five when a cloud has more than 16384 points). Results are
+ * bit-identical to tk3d_chamfer_distance_forward_f32 for
  * every input. The size function returns 0 for shapes the path cannot serve (a cloud of
  * more than 65536 points, B = 0) and, with always = 0, also for shapes where it is not
  * the faster route (small or very unequal clouds): callers that pass on that size, and a
@@ -224,8 +225,13 @@ int tk3d_sample_farthest_points_f64(const double *points, int64_t B, int64_t N,
  * tk3d_sample_farthest_points_workspace_bytes(B, N, 4) exceeds that size (8 MiB: e.g. one
  * cloud of 2 million points, or 64 clouds of 32000); clouds of up to 16384 points need
  * no workspace at any batch size. Calls no hipMalloc / hipFree. The first call on a GPU
- * looks the array's address up (hipGetSymbolAddress), so make that call outside stream
- * capture. All calls on one GPU share the array: calls that overlap in time on the same
+ * looks the array's address up (hipGetSymbolAddress), and the first call on a GPU for each
+ * kernel shape (points per lane: the size class of the cloud) asks the runtime once to
+ * allow that kernel's LDS size (hipFuncSetAttribute): both are host calls that stream
+ * capture does not record, so make one call per device and cloud-size class outside
+ * capture. Return value as everywhere in this header: 0, a negative TK3D_ERR_*, or the
+ * positive hipError_t of a runtime call that failed (then nothing further was launched).
+ * All calls on one GPU share the array: calls that overlap in time on the same
  * GPU (different streams or threads) race and must be serialised by the caller. */
 #define TK3D_FPS_STATIC_WORKSPACE_BYTES (8u << 20)
 int tk3d_sample_farthest_points_static_f32(const float *points, int64_t B, int64_t N,

@@ -26,14 +26,32 @@ HIPCC_FLAGS = [
     "-ffp-contract=off",
     "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # matrix instructions write ordinary vector registers (no copies out of the
-    # accumulation registers before the vector ALU can use a result)
-    "-mllvm", "-amdgpu-mfma-vgpr-form",
     # the Hilbert curve table of the chamfer sort is worked out at compile time
     "-fconstexpr-steps=200000000",
     "-Wall",
     "-Wno-unused-function",
 ]
+
+
+# Matrix instructions that write ordinary vector registers (no copies out of the
+# accumulation registers before the vector ALU can use a result). An LLVM option: other
+# ROCm releases may not know it, so it is used only where a trial compilation accepts it;
+# the kernels are correct either way.
+MFMA_VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+
+
+def optional_flags():
+    """Those of the optional compiler flags that this hipcc accepts."""
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "probe.hip")
+        with open(src, "w") as f:
+            f.write("__global__ void probe() {}\n")
+        res = subprocess.run([hipcc_path(), "--offload-arch=gfx950", "-c", src, "-o",
+                              os.path.join(tmp, "probe.o")] + MFMA_VGPR_FORM,
+                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    return list(MFMA_VGPR_FORM) if res.returncode == 0 else []
 
 
 def hipcc_path():
@@ -54,7 +72,7 @@ def build(verbose=False, jobs=None):
 
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"] + optional_flags()
     include = ["-I", os.path.join(REPO, "include"), "-I", CSRC]
 
     def run(cmd):
