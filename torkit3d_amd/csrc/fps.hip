@@ -291,6 +291,26 @@ __device__ __forceinline__ void wave_top2_i32(int v, int &first, int &second)
     second = __builtin_amdgcn_readlane(m2, 63);
 }
 
+// Largest of the 64 lanes' values (all >= 0), wave-uniform: a scan along rows of 16 lanes
+// with row shifts, the rows' results carried on with row broadcasts, the total read from
+// lane 63. A lane without a source lane in a step takes 0.
+__device__ __forceinline__ int wave_max_i32(int v)
+{
+#define TK3D_MAX_STEP(ctrl, rows)                                                      \
+    {                                                                                  \
+        const int o = __builtin_amdgcn_update_dpp(0, v, ctrl, rows, 0xf, false);       \
+        v = o > v ? o : v;                                                             \
+    }
+    TK3D_MAX_STEP(0x111, 0xf)  // row_shr:1
+    TK3D_MAX_STEP(0x112, 0xf)  // row_shr:2
+    TK3D_MAX_STEP(0x114, 0xf)  // row_shr:4
+    TK3D_MAX_STEP(0x118, 0xf)  // row_shr:8
+    TK3D_MAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+    TK3D_MAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef TK3D_MAX_STEP
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // FpsWalk that also reports the largest value it passed by: the walk from the root to
 // the first leaf equal to `wmax` sees the sibling of every node on its path, and the
 // largest of those siblings is the lane's second-largest minimum (equal to `wmax` when
@@ -526,9 +546,9 @@ __device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
     return r * L.c + (j >> L.log2_bs);
 }
 
-// fp32 kernel for clouds of 4097 to 16384 points: the multi-step kernel above with the
+// fp32 kernel for clouds of 8193 to 16384 points: the multi-step kernel above with the
 // points laid out by region, so that an update only visits the points a new centre can
-// reach.
+// reach, and with sixteen waves, so that an exchange has sixteen candidates to accept from.
 //
 // At 16 or 32 points per lane a step is dominated by the update of the running minima
 // (nine instructions per point and centre), and almost all of that work changes nothing:
@@ -536,37 +556,48 @@ __device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
 // was the largest of them all, and minima only shrink), so a centre can lower a point's
 // minimum only if it lies within sqrt(tau) of it - a ball that shrinks as the sampling
 // proceeds. Hence:
-//   * the prologue sorts the points along a Morton curve (bitonic sort of (code, index)
-//     in LDS) and cuts the sorted sequence into 32 regions; region R goes to wave R % 8
-//     as block R / 8 of the lanes' registers (P / 4 points per lane and block), so
-//     neighbouring regions sit in different waves, i.e. on different SIMDs;
+//   * the prologue sorts the points along a Morton curve (a counting sort by cell in LDS)
+//     and cuts the sorted sequence into 64 regions; region R goes to wave R % 16 as block
+//     R / 16 of the lanes' registers (P / 4 points per lane and block), so neighbouring
+//     regions sit in different waves, on different SIMDs;
 //   * every wave keeps the bounding boxes of its four blocks. Before an update, lane
-//     (m, q) evaluates the canonical distance from centre m to box q - the same rounded
+//     (a, q) evaluates the canonical distance from candidate a to box q - the same rounded
 //     operations as tk_dist2 on the per-axis gaps, each of which is monotone, so the
 //     result is a lower bound of the canonical distance to every point of the box - and a
 //     block is updated only if that bound is below tau. Skipping is therefore exact: a
 //     skipped update would have changed no minimum.
-// On uniform clouds a centre reaches two to five of the 32 regions once a few hundred
-// points are selected, and the waves that own them update one block each, side by side.
+//
+// Sixteen waves of 16 points per lane instead of eight of 32: an exchange accepts 4.4
+// candidates on uniform clouds where eight waves accepted 3.1, the walk to the winner's leaf
+// is a level shorter and the regions are half the size. The price is what every wave repeats
+// per exchange, now sixteen times on four SIMDs, so that part is kept short: a wave ranks
+// only its own candidate against the sixteen (one ballot per condition) and the verdicts
+// meet in LDS behind a second barrier; the wave's runner-up comes from a second plain
+// maximum scan that runs beside the walk instead of a scan that carries pairs.
 //
 // Ties. With this layout the lane order is no longer the reference's priority order
 // (see the top of the file), so equal maxima are resolved explicitly: a wave that holds
 // its maximum more than once picks the point with the lowest reference position (the
-// rare slow path below), the slots carry that position, and candidates with equal values
-// are ranked by it. The acceptance rules are those of fps_multistep_kernel_f32.
+// rare slow path below), the slots carry the point's sorted rank, and candidates with equal
+// values are ranked by their positions. The acceptance rules are those of
+// fps_multistep_kernel_f32.
 template <int P, bool SOA, int MAXM>
-__global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__restrict__ points,
+__global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__restrict__ points,
                                                              int64_t *__restrict__ index,
                                                              FpsLayout L)
 {
-    constexpr int NT = 512, NW = 8, NB = 4, PB = P / NB, S = NT * P, RS = TK_WAVE * PB;
-    static_assert(P % NB == 0 && (P & (P - 1)) == 0 && MAXM * NB <= TK_WAVE, "shape");
+    constexpr int NT = 1024, NW = 16, NB = 4, PB = P / NB, S = NT * P, RS = TK_WAVE * PB;
+    constexpr int CELLS = 4096;  // 16^3 cells for the sort
+    static_assert(P % NB == 0 && (P & (P - 1)) == 0 && MAXM <= NW && NW * NB == TK_WAVE, "shape");
+    static_assert(CELLS % NT == 0 && S < (1 << 19), "sort");
     constexpr int F32_INF = 0x7f800000;
     constexpr int F32_NEG1 = (int)0xbf800000;
     extern __shared__ __align__(16) unsigned char fps_region_lds[];
-    unsigned long long *const keys = reinterpret_cast<unsigned long long *>(fps_region_lds);
-    __shared__ float4 s_cand[2][8];  // a wave's candidate: x, y, z, running minimum (bits)
-    __shared__ int2 s_aux[2][8];     // the wave's second-largest minimum, the candidate's rank
+    unsigned *const keys = reinterpret_cast<unsigned *>(fps_region_lds);  // [S] points, sorted
+    unsigned *const cnt = keys + S;                                       // [CELLS + 1]
+    __shared__ float4 s_cand[2][NW];  // a wave's candidate: x, y, z, running minimum (bits)
+    __shared__ int2 s_aux[2][NW];     // the wave's second-largest minimum, the candidate's rank
+    __shared__ int s_rank[2][NW];     // a candidate's rank among them, + 256: it passed
     __shared__ float s_box[NW][NB][8];  // lo.xyz, hi.xyz of a wave's block
     __shared__ float s_red[NW][8];
 
@@ -614,66 +645,115 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
         }
         origin[a] = l;
         const float extent = h - l;
-        scale[a] = extent > 0.0f ? 1023.0f / extent : 0.0f;  // also 0 for NaN / inf extents
+        scale[a] = extent > 0.0f ? 15.99f / extent : 0.0f;  // also 0 for NaN / inf extents
     }
 
-    // ---- (Morton code, point) pairs, sorted; slots beyond the cloud sort last ----
-    auto spread = [](unsigned v) {  // 10 bits -> every third bit
-        v = (v | (v << 16)) & 0x030000ffu;
-        v = (v | (v << 8)) & 0x0300f00fu;
-        v = (v | (v << 4)) & 0x030c30c3u;
-        v = (v | (v << 2)) & 0x09249249u;
+    // ---- the points in the order of their cells along a Morton curve; slots beyond the cloud
+    // last. A counting sort: any order that keeps neighbours together is a valid layout, so 16
+    // steps per axis are enough and the order within a cell is whatever the atomics give.
+    // (A bitonic sort of (code, point) pairs took 105 passes with a barrier each: two thirds
+    // of a prologue of 0.19 ms.) ----
+    auto spread = [](unsigned v) {  // 4 bits -> every third bit
+        v = (v | (v << 4)) & 0x0c3u;
+        v = (v | (v << 2)) & 0x249u;
         return v;
     };
-    for (int e = tid; e < S; e += NT) {
-        unsigned code = 0x7fffffffu;
+    for (int i = tid; i <= CELLS; i += NT)
+        cnt[i] = 0u;
+    __syncthreads();
+    unsigned where[P];  // cell, and the point's turn within it from bit 13
+    float own[P][3];    // point tid + k * NT, as read (coalesced) for its cell
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+        const int e = tid + k * NT;
+        unsigned cell = CELLS;
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+            own[k][a] = e < L.n ? fps_coord<SOA>(pts, L.n, e, a) : 0.0f;
         if (e < L.n) {
             unsigned c3[3];
 #pragma unroll
             for (int a = 0; a < 3; ++a) {
-                const float f = (fps_coord<SOA>(pts, L.n, e, a) - origin[a]) * scale[a];
-                // (a NaN or an out-of-range value lands in cell 0 or 1023: any order of the
-                // points is a valid layout)
-                const float g = __builtin_fminf(__builtin_fmaxf(f, 0.0f), 1023.0f);
-                c3[a] = (unsigned)(int)g;
+                const float f = (own[k][a] - origin[a]) * scale[a];
+                // (a NaN or an out-of-range value lands in cell 0 or 15)
+                c3[a] = (unsigned)(int)__builtin_fminf(__builtin_fmaxf(f, 0.0f), 15.0f);
             }
-            code = spread(c3[0]) | (spread(c3[1]) << 1) | (spread(c3[2]) << 2);
+            cell = spread(c3[0]) | (spread(c3[1]) << 1) | (spread(c3[2]) << 2);
         }
-        keys[e] = ((unsigned long long)code << 32) | (unsigned)e;
+        where[k] = cell | (atomicAdd(&cnt[cell], 1u) << 13);
     }
     __syncthreads();
-    for (int kk = 2; kk <= S; kk <<= 1) {
-        for (int jj = kk >> 1; jj > 0; jj >>= 1) {
-            for (int i = tid; i < S / 2; i += NT) {
-                const int a = ((i & ~(jj - 1)) << 1) | (i & (jj - 1));
-                const int b = a + jj;
-                const unsigned long long ka = keys[a], kb = keys[b];
-                const bool ascending = (a & kk) == 0;
-                if ((ka > kb) == ascending) {
-                    keys[a] = kb;
-                    keys[b] = ka;
-                }
+    {
+        // counts -> first positions: a lane sums its run of counters, the waves scan the sums
+        constexpr int RUN = CELLS / NT;
+        unsigned c[RUN], mine = 0u;
+#pragma unroll
+        for (int i = 0; i < RUN; ++i) {
+            c[i] = cnt[tid * RUN + i];
+            mine += c[i];
+        }
+        unsigned incl = mine;
+#pragma unroll
+        for (int o = 1; o < TK_WAVE; o <<= 1) {
+            const unsigned up = (unsigned)__shfl_up((int)incl, o);
+            incl += lane >= o ? up : 0u;
+        }
+        if (lane == TK_WAVE - 1)
+            s_red[wave][0] = __builtin_bit_cast(float, incl);
+        __syncthreads();
+        unsigned start = incl - mine;
+        for (int w = 0; w < wave; ++w)
+            start += __builtin_bit_cast(unsigned, s_red[w][0]);
+#pragma unroll
+        for (int i = 0; i < RUN; ++i) {
+            cnt[tid * RUN + i] = start;
+            start += c[i];
+        }
+        if (tid == 0)
+            cnt[CELLS] = (unsigned)L.n;  // the slots beyond the cloud follow its points
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+        where[k] = cnt[where[k] & 0x1fffu] + (where[k] >> 13);  // the point's sorted rank
+        keys[where[k]] = (unsigned)(tid + k * NT);
+    }
+    __syncthreads();
+
+    // ---- this lane's points: block q, turn u <-> sorted rank (q*8 + wave) * RS + u*64 + lane.
+    // The point indices stay in the sorted list in LDS (16 registers less). ----
+    auto rank_of = [&](int in_lane, int p) {
+        return ((p / PB) * NW + wave) * RS + (p % PB) * TK_WAVE + in_lane;
+    };
+    // The coordinates travel from the lanes that read them to the lanes that own them through
+    // LDS, one coordinate at a time behind the counters (fetched from memory by sorted rank
+    // they were 48 gathers of 64 cache lines per wave: 45 us).
+    float x[P], y[P], z[P];
+    int t[2 * P];  // t[P + p]: running minimum of point p (bits); t[1..P-1]: maxima
+    {
+        float *const plane = reinterpret_cast<float *>(cnt);  // [S]
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+#pragma unroll
+            for (int k = 0; k < P; ++k)
+                plane[where[k]] = own[k][a];
+            __syncthreads();
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const float v = plane[rank_of(lane, p)];
+                if (a == 0)
+                    x[p] = v;
+                else if (a == 1)
+                    y[p] = v;
+                else
+                    z[p] = v;
             }
             __syncthreads();
         }
     }
-
-    // ---- this lane's points: block q, turn u <-> sorted rank (q*8 + wave) * RS + u*64 + lane.
-    // The point indices stay in the sorted list in LDS (32 registers less). ----
-    auto rank_of = [&](int in_lane, int p) {
-        return ((p / PB) * NW + wave) * RS + (p % PB) * TK_WAVE + in_lane;
-    };
-    float x[P], y[P], z[P];
-    int t[2 * P];  // t[P + p]: running minimum of point p (bits); t[1..P-1]: maxima
 #pragma unroll
-    for (int p = 0; p < P; ++p) {
-        const int j = (int)(unsigned)keys[rank_of(lane, p)];
-        const bool ok = j < L.n;
-        x[p] = ok ? fps_coord<SOA>(pts, L.n, j, 0) : 0.0f;
-        y[p] = ok ? fps_coord<SOA>(pts, L.n, j, 1) : 0.0f;
-        z[p] = ok ? fps_coord<SOA>(pts, L.n, j, 2) : 0.0f;
-        t[P + p] = ok ? F32_INF : F32_NEG1;
-    }
+    for (int p = 0; p < P; ++p)
+        t[P + p] = (int)keys[rank_of(lane, p)] < L.n ? F32_INF : F32_NEG1;
     t[0] = 0;
     // boxes of the wave's blocks (an empty block gets an empty box: never reached)
 #pragma unroll
@@ -713,10 +793,9 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
     // From here on a point is named by its rank in the sorted list; the list is consulted
     // only where a point index is needed (output, ties).
     __syncthreads();  // the boxes are written
-    // Lane (a, b) = (lane / 8, lane % 8) relates candidate a to candidate b after an
-    // exchange; with b < 4 it also tests candidate a against the wave's block b, whose
-    // box it keeps in registers.
-    const int ca = lane >> 3, cb = lane & 7;
+    // After an exchange lane (a, q) = (lane / 4, lane % 4) stands for candidate a and tests it
+    // against the wave's block q, whose box it keeps in registers.
+    const int ca = lane >> 2, cb = lane & 3;
     float box_lo[3], box_hi[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -724,19 +803,16 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
         box_hi[a] = s_box[wave][cb & (NB - 1)][3 + a];
     }
     // The centres of the coming update are the candidates of the lanes in `centres`
-    // (lane 8 a stands for candidate a); bit 8 a + q of `reach` says whether candidate a
+    // (lane 4 a stands for candidate a); bit 4 a + q of `reach` says whether candidate a
     // can lower a minimum in block q. The first update is point 0 against every block.
     float ax = fps_coord<SOA>(pts, L.n, 0, 0);
     float ay = fps_coord<SOA>(pts, L.n, 0, 1);
     float az = fps_coord<SOA>(pts, L.n, 0, 2);
     unsigned long long centres = 1ull, reach = (1ull << NB) - 1;
-    // the last point emitted is the candidate of lane ctz(last_mask) / 8's sorted rank in
-    // last_rank; no mask: point 0
+    // the last point emitted is the candidate of lane ctz(last_mask), whose sorted rank that
+    // lane keeps in last_rank; no mask: point 0
     unsigned long long last_mask = 0ull;
     int last_rank = 0;
-    constexpr unsigned long long DIAGONAL = 0x8040201008040201ull;        // lanes a == b
-    constexpr unsigned long long FIRST_OF_EIGHT = 0x0101010101010101ull;  // lanes b == 0
-    constexpr unsigned long long BLOCK_LANES = FIRST_OF_EIGHT * ((1u << NB) - 1);  // b < NB
     int nc = 1;
     if (tid == 0)
         out[0] = 0;
@@ -784,9 +860,12 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
         // Only points strictly above zero are candidates (the reference starts its
         // scan from max_dist = 0 with strict '>').
         const int best = t[1] > 0 ? t[1] : 0;
-        int wmax, second;
-        wave_top2_i32(best, wmax, second);  // second: over the other lanes
+        // The wave's maximum and the first lane that holds it; the runner-up is the largest of
+        // the other lanes' maxima (a second scan that does not wait for the walk) and of what
+        // the walk through the winner lane's own tree passes by.
+        const int wmax = wave_max_i32(best);
         int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
+        int second = wave_max_i32(lane == wl ? 0 : best);
         FpsPick pick;
         FpsWalk3<P, 1>::go(t, x, y, z, wl, wmax, pick, second);  // and inside lane wl
         int pick_rank = rank_of(wl, pick.j);
@@ -832,83 +911,93 @@ __global__ __launch_bounds__(512) void fps_region_kernel_f32(const float *__rest
         // Every wave now works out, redundantly and without a serial chain, how many of
         // the candidates are certain winners of the coming steps. All 64 lanes are active,
         // so conditions are combined as lane masks in scalar registers.
-        const float4 A = s_cand[buf][ca], Bc = s_cand[buf][cb];
-        const int2 Bx = s_aux[buf][cb];  // the wave's second-largest minimum, sorted rank
-        ax = A.x;
-        ay = A.y;
-        az = A.z;
-        const int va = __builtin_bit_cast(int, A.w), vb = __builtin_bit_cast(int, Bc.w);
-        const unsigned long long m_above = __builtin_amdgcn_ballot_w64(vb > va);
-        const unsigned long long m_equal = __builtin_amdgcn_ballot_w64(vb == va);
-        const unsigned long long m_live = __builtin_amdgcn_ballot_w64(va > 0);
-        // b comes before a in the reference's order: larger value, then lower position.
-        // Positions are looked up only when two candidates really hold the same value.
-        unsigned long long m_before = m_above;
-        if ((m_equal & m_live & ~DIAGONAL) != 0ull) {  // uniform
-            const int rank_a = __shfl(Bx.y, ca);  // (lane a holds candidate a as its b)
-            const int pos_a = fps_position_of_point((int)(unsigned)keys[rank_a], L);
-            const int pos_b = fps_position_of_point((int)(unsigned)keys[Bx.y], L);
-            m_before |= m_equal & __builtin_amdgcn_ballot_w64(pos_b < pos_a);
-        }
-        const float dab = tk_dist2<float>(A.x, A.y, A.z, Bc.x, Bc.y, Bc.z);
-        // a survives b's selection: b's update leaves a's minimum alone, and b's wave
-        // holds nothing else at or above it
-        const unsigned long long m_far =
-            __builtin_amdgcn_ballot_w64(__builtin_bit_cast(int, dab) >= va);
-        const unsigned long long m_alone = __builtin_amdgcn_ballot_w64(Bx.x < va);
-        const unsigned long long m_fine = ~m_before | (m_far & m_alone);
-        // byte a of a mask: candidate a against every b
-        const unsigned before_a =
-            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_before : (unsigned)(m_before >> 32),
-                                  (unsigned)(lane & 24), 8u);
-        const unsigned fine_a =
-            __builtin_amdgcn_ubfe(lane < 32 ? (unsigned)m_fine : (unsigned)(m_fine >> 32),
-                                  (unsigned)(lane & 24), 8u);
-        const int rank = __builtin_popcount(before_a);
-        const unsigned long long fine = __builtin_amdgcn_ballot_w64(fine_a == 0xffu) & m_live;
-        // Candidates above zero have distinct ranks. Lane (a, b) asks whether candidate a
-        // has rank b and passed; folding the bytes of that mask together gives, in bit b,
-        // whether the candidate of rank b passed.
-        unsigned long long passed = __builtin_amdgcn_ballot_w64(rank == cb) & fine;
-        passed |= passed >> 32;
-        passed |= passed >> 16;
-        passed |= passed >> 8;
-        const int left = L.k - it;  // steps still wanted
-        int good = __builtin_ctz(~(unsigned)passed | (1u << MAXM));  // ranks 0..good-1 passed
-        good = good < left ? good : left;
-        // Every running minimum is at most tau, the value of the first winner (the largest
-        // value has nobody before it); candidate a reaches block q only if the canonical
-        // distance from it to the block's box - rounded like tk_dist2, each operation
-        // monotone, hence a lower bound for every point of the box - is below tau. (A NaN
-        // bound counts as reachable.)
-        const float tau =
-            read_lane(A.w, __builtin_ctzll(__builtin_amdgcn_ballot_w64(rank == 0)));
-        const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
-        const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
-        const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
-        const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
-        reach = __builtin_amdgcn_ballot_w64(!(bound >= tau)) & BLOCK_LANES;
-        const unsigned long long m_taken = __builtin_amdgcn_ballot_w64(rank < good);
-        centres = m_taken & FIRST_OF_EIGHT;
-        if (good > 0) {  // uniform
-            if (wave == 0) {  // uniform
-                if (ca == cb && rank < good)
-                    out[it + rank] = (int64_t)(unsigned)keys[Bx.y];
+        {
+            // Sixteen candidates. All waves working through all 256 relations would put four
+            // copies of a long chain on every SIMD; instead a wave ranks its own candidate
+            // against the sixteen (lane b holds candidate b; a condition is one ballot), leaves
+            // rank and verdict in LDS, and after a second barrier every wave reads the sixteen
+            // verdicts.
+            const float4 W = s_cand[buf][wave];  // (uniform)
+            const int2 Wx = s_aux[buf][wave];
+            const float4 Bc = s_cand[buf][lane & 15];
+            const int2 Bx = s_aux[buf][lane & 15];
+            {
+                const int vw = __builtin_bit_cast(int, W.w), vb = __builtin_bit_cast(int, Bc.w);
+                unsigned m_before = (unsigned)__builtin_amdgcn_ballot_w64(vb > vw) & 0xffffu;
+                const unsigned m_equal = (unsigned)__builtin_amdgcn_ballot_w64(vb == vw) & 0xffffu;
+                // b comes before the wave's candidate in the reference's order: larger value,
+                // then lower position; positions are looked up only when two candidates really
+                // hold the same value
+                if (vw > 0 && (m_equal & ~(1u << wave)) != 0u) {  // uniform
+                    const int pos_w = fps_position_of_point((int)(unsigned)keys[Wx.y], L);
+                    const int pos_b = fps_position_of_point((int)(unsigned)keys[Bx.y], L);
+                    m_before |= m_equal & (unsigned)__builtin_amdgcn_ballot_w64(pos_b < pos_w);
+                }
+                const float dwb = tk_dist2<float>(W.x, W.y, W.z, Bc.x, Bc.y, Bc.z);
+                // the candidate survives b's selection: b's update leaves its minimum alone, and
+                // b's wave holds nothing else at or above it
+                const unsigned m_far =
+                    (unsigned)__builtin_amdgcn_ballot_w64(__builtin_bit_cast(int, dwb) >= vw);
+                const unsigned m_alone = (unsigned)__builtin_amdgcn_ballot_w64(Bx.x < vw);
+                const unsigned m_fine = (~m_before | (m_far & m_alone)) & 0xffffu;
+                const int verdict =
+                    __builtin_popcount(m_before) | ((vw > 0 && m_fine == 0xffffu) ? 256 : 0);
+                if (lane == 0)
+                    s_rank[buf][wave] = verdict;
             }
-            // the last point emitted, should the cloud run out of distinct points
-            last_mask = __builtin_amdgcn_ballot_w64(rank == good - 1);
-            last_rank = Bx.y;
-            nc = good;
-        } else {
-            // No point lies away from the chosen set: the previous choice is emitted again,
-            // as the reference does. Every minimum is zero already: nothing is updated.
-            if (tid == 0) {
-                int64_t j = 0;
-                if (last_mask != 0ull)
-                    j = (int64_t)(unsigned)keys[read_lane(last_rank, __builtin_ctzll(last_mask) >> 3)];
-                out[it] = j;
+            __syncthreads();
+            const float4 A = s_cand[buf][ca];
+            const int2 Ax = s_aux[buf][ca];  // its wave's second-largest minimum, its sorted rank
+            const int verdict = s_rank[buf][ca];
+            ax = A.x;
+            ay = A.y;
+            az = A.z;
+            const int rank = verdict & 255;  // a permutation of the live candidates
+            const unsigned long long fine = __builtin_amdgcn_ballot_w64(verdict >= 256);
+            // Lane (a, q) asks whether candidate a has rank q + 4 i and passed; folding the
+            // nibbles of that mask together gives, in bit q, whether the candidate of that rank
+            // passed.
+            unsigned passed = 0u;
+#pragma unroll
+            for (int i = 0; i < (MAXM + 3) / 4; ++i) {
+                unsigned long long m = __builtin_amdgcn_ballot_w64(rank == 4 * i + cb) & fine;
+                m |= m >> 32;
+                m |= m >> 16;
+                m |= m >> 8;
+                m |= m >> 4;
+                passed |= ((unsigned)m & 0xfu) << (4 * i);
             }
-            nc = 1;
+            const int left = L.k - it;  // steps still wanted
+            int good = __builtin_ctz(~passed | (1u << MAXM));  // ranks 0..good-1 passed
+            good = good < left ? good : left;
+            // tau and the reach of candidate a into block q: as with eight waves
+            const float tau =
+                read_lane(A.w, __builtin_ctzll(__builtin_amdgcn_ballot_w64(rank == 0)));
+            const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
+            const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
+            const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
+            const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
+            reach = __builtin_amdgcn_ballot_w64(!(bound >= tau));
+            centres = __builtin_amdgcn_ballot_w64(rank < good) & 0x1111111111111111ull;
+            if (good > 0) {  // uniform
+                if (wave == 0) {  // uniform
+                    if (cb == 0 && rank < good)
+                        out[it + rank] = (int64_t)(unsigned)keys[Ax.y];
+                }
+                // the last point emitted, should the cloud run out of distinct points
+                last_mask = __builtin_amdgcn_ballot_w64(rank == good - 1);
+                last_rank = Ax.y;
+                nc = good;
+            } else {
+                // No point lies away from the chosen set: the previous choice is emitted again.
+                if (tid == 0) {
+                    int64_t j = 0;
+                    if (last_mask != 0ull)
+                        j = (int64_t)(unsigned)keys[read_lane(last_rank, __builtin_ctzll(last_mask))];
+                    out[it] = j;
+                }
+                nc = 1;
+            }
         }
     }
 }
@@ -1127,24 +1216,25 @@ template <int P>
 int fps_region_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
                           const FpsLayout &L, hipStream_t s)
 {
-    constexpr int MAXM = 6;
-    constexpr int LDS = 512 * P * 8;  // the sort's (code, point) pairs
+    constexpr int MAXM = 8, NT = 1024;
+    // the sorted list, and behind it the sort's counters, then one coordinate of every point
+    constexpr int LDS = NT * P * 4 + (NT * P > 4100 ? NT * P : 4100) * 4;
     if (soa) {
         constexpr auto kernel = fps_region_kernel_f32<P, true, MAXM>;
         const int allowed = tk_allow_dynamic_lds<kernel>(LDS);
         if (allowed != TK3D_OK)
             return allowed;
-        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(512), LDS, s, points, index, L);
-        hipLaunchKernelGGL((fps_register_kernel<float, P, 512, true>), dim3((unsigned)B),
-                           dim3(512), 0, s, points, index, L, 1);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(NT), LDS, s, points, index, L);
+        hipLaunchKernelGGL((fps_register_kernel<float, P, NT, true>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L, 1);
     } else {
         constexpr auto kernel = fps_region_kernel_f32<P, false, MAXM>;
         const int allowed = tk_allow_dynamic_lds<kernel>(LDS);
         if (allowed != TK3D_OK)
             return allowed;
-        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(512), LDS, s, points, index, L);
-        hipLaunchKernelGGL((fps_register_kernel<float, P, 512, false>), dim3((unsigned)B),
-                           dim3(512), 0, s, points, index, L, 1);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(NT), LDS, s, points, index, L);
+        hipLaunchKernelGGL((fps_register_kernel<float, P, NT, false>), dim3((unsigned)B),
+                           dim3(NT), 0, s, points, index, L, 1);
     }
     return TK3D_OK;
 }
@@ -1171,7 +1261,7 @@ int fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
         // The region kernel's sort costs about 0.15 ms per call, which the skipped updates
         // repay once a few thousand points are sampled from more than 8192 (16384 -> 4096:
         // 3.35 -> 2.9 ms; 16384 -> 512 would go from 0.52 to 0.61 ms).
-        return fps_region_launch_f32<32>(points, soa, B, index, L, s);
+        return fps_region_launch_f32<16>(points, soa, B, index, L, s);
     else
         fps_launch_f32<32, 512>(points, soa, B, index, L, s);
     return TK3D_OK;
