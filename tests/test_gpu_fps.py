@@ -220,9 +220,11 @@ def test_points_at_infinity(cuda):
     np.testing.assert_array_equal(run(pts, 30, cuda), want)
 
 
-# ---- 8193 to 16384 points, 2048 samples or more: the kernel that lays the points out by
-# region (Morton order) and skips the blocks a new centre cannot reach. The lane order is no
-# longer the reference's priority order there, so ties are resolved explicitly. ----
+# ---- 4097 to 16384 points, 256 samples or more: the kernel that lays the points out by
+# region (Morton order), skips the blocks a new centre cannot reach and accepts from sixteen
+# candidates per exchange. The lane order is no longer the reference's priority order there,
+# so ties are resolved explicitly. 4097..8192 points run it with 8 points per lane, more with
+# 16. ----
 
 def _region_cloud(kind, g, b, n):
     if kind == "uniform":
@@ -262,10 +264,17 @@ def test_region_kernel_on_adversarial_clouds(cuda, kind):
     pts = _region_cloud(kind, g, 2, 12000 if kind in ("uniform", "lattice") else 16384)
     k = 2100
     np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
+    # and with 8 points per lane
+    pts = _region_cloud(kind, g, 2, 6000 if kind in ("uniform", "lattice") else 8192)
+    k = 700
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
 
 
 @pytest.mark.parametrize("n,k,transpose", [(8193, 2048, False), (16384, 16384, False),
-                                           (10000, 2049, True), (16383, 4096, True)])
+                                           (10000, 2049, True), (16383, 4096, True),
+                                           (4097, 256, False), (8192, 8192, False),
+                                           (5000, 300, True), (16384, 256, True),
+                                           (8193, 257, False)])
 def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
     pts = torch.rand(2, n, 3, generator=gen(n + k))
     want = oracle.sample_farthest_points(pts.numpy(), k)
@@ -273,13 +282,14 @@ def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
     np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
 
 
-def test_region_kernel_with_non_finite_points(cuda):
-    pts = torch.rand(3, 9000, 3, generator=gen(71))
+@pytest.mark.parametrize("n", [9000, 5000])
+def test_region_kernel_with_non_finite_points(cuda, n):
+    pts = torch.rand(3, n, 3, generator=gen(71))
     pts[0, 7, 1] = float("nan")
     pts[0, 4500] = float("nan")
     pts[1, 100, 0] = float("inf")
     pts[2, 0, 2] = float("nan")        # point 0 itself: every distance is NaN
-    k = 2048
+    k = 2048 if n == 9000 else 400
     want = oracle.sample_farthest_points(pts.numpy(), k)
     np.testing.assert_array_equal(run(pts, k, cuda), want)
 

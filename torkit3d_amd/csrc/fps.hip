@@ -246,8 +246,9 @@ __global__ __launch_bounds__(NT) void fps_register_kernel(const T *__restrict__ 
 //     order like signed integers; integer min/max need no NaN canonicalisation
 //     and the -1.0f marker of unused slots (a negative integer) stays put;
 //   * a lane reduces its P minima through a binary tree of maxima kept in
-//     registers; the wave reduction is a DPP scan written out by hand (the compiler
-//     does not fold the lane moves into the max) that carries the two largest values;
+//     registers; the wave's maximum is a scan with DPP row shifts and broadcasts, and
+//     the runner-up (the largest value of the other lanes) a second such scan that runs
+//     beside the walk below;
 //   * the winning lane comes from one ballot + scalar find-first; its winning
 //     point is found by walking the winner lane's tree with v_readlane and
 //     scalar branches (left child first = lowest position), and the leaf reached
@@ -261,35 +262,6 @@ struct FpsPick {
     float x, y, z;
     int j;
 };
-
-// Largest and second-largest of the 64 lanes' values (with multiplicity: two lanes
-// holding the maximum give second == first), both wave-uniform. The scan of
-// wave_max_i32 carrying a pair: every step merges two disjoint lane sets, for which
-// second = max(second_a, second_b, min(first_a, first_b)). The two chains fill each
-// other's DPP wait states. Lanes whose source lane does not exist skip a step's DPP
-// writes and re-apply a stale `t` that their `second` already contains.
-__device__ __forceinline__ void wave_top2_i32(int v, int &first, int &second)
-{
-    int m1 = v, m2 = 0, t = 0;  // values are >= 0
-#define TK3D_TOP2_STEP(CTRL, MASK)                                                         \
-    "s_nop 0\n\t"                                                                           \
-    "v_min_i32_dpp %2, %0, %0 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
-    "v_max_i32_dpp %1, %1, %1 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
-    "v_max_i32_dpp %0, %0, %0 " CTRL " row_mask:" MASK " bank_mask:0xf\n\t"                 \
-    "v_max_i32_dpp %1, %2, %1 quad_perm:[0,1,2,3] row_mask:" MASK " bank_mask:0xf\n\t"
-    asm volatile("s_nop 1\n\t"
-                 TK3D_TOP2_STEP("row_shr:1", "0xf")
-                 TK3D_TOP2_STEP("row_shr:2", "0xf")
-                 TK3D_TOP2_STEP("row_shr:4", "0xf")
-                 TK3D_TOP2_STEP("row_shr:8", "0xf")
-                 TK3D_TOP2_STEP("row_bcast:15", "0xa")
-                 TK3D_TOP2_STEP("row_bcast:31", "0xc")
-                 "s_nop 1"
-                 : "+v"(m1), "+v"(m2), "+v"(t));
-#undef TK3D_TOP2_STEP
-    first = __builtin_amdgcn_readlane(m1, 63);
-    second = __builtin_amdgcn_readlane(m2, 63);
-}
 
 // Largest of the 64 lanes' values (all >= 0), wave-uniform: a scan along rows of 16 lanes
 // with row shifts, the rows' results carried on with row broadcasts, the total read from
@@ -465,9 +437,9 @@ __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__re
         // Only points strictly above zero are candidates (the reference starts its
         // scan from max_dist = 0 with strict '>').
         const int best = t[1] > 0 ? t[1] : 0;
-        int wmax, second;
-        wave_top2_i32(best, wmax, second);  // second: over the other lanes
+        const int wmax = wave_max_i32(best);
         const int wl = __builtin_ctzll(__builtin_amdgcn_ballot_w64(best == wmax));
+        int second = wave_max_i32(lane == wl ? 0 : best);  // over the other lanes
         FpsPick pick;
         FpsWalk2<P, 1>::go(t, x, y, z, jv, wl, wmax, pick, second);  // and inside lane wl
         const int buf = round & 1;
@@ -546,7 +518,7 @@ __device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
     return r * L.c + (j >> L.log2_bs);
 }
 
-// fp32 kernel for clouds of 8193 to 16384 points: the multi-step kernel above with the
+// fp32 kernel for clouds of 4097 to 16384 points: the multi-step kernel above with the
 // points laid out by region, so that an update only visits the points a new centre can
 // reach, and with sixteen waves, so that an exchange has sixteen candidates to accept from.
 //
@@ -1255,12 +1227,15 @@ int fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
         fps_launch_f32<4, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 8)
         fps_launch_f32<8, 512>(points, soa, B, index, L, s);
+    // Beyond 4096 points the region kernel (sixteen waves; its prologue costs about 30 us) wins
+    // from a few hundred samples on: B=16, 8192 -> 2048 1.20 -> 0.94 ms, B=4, 10000 -> 512
+    // 0.53 -> 0.34 ms, B=8, 16384 -> 512 0.51 -> 0.38 ms; at 4096 points it is level with the
+    // kernel above at 1024 samples and behind it below.
+    else if (npos <= 512 * 16 && L.k >= 256)
+        return fps_region_launch_f32<8>(points, soa, B, index, L, s);
     else if (npos <= 512 * 16)
         fps_launch_f32<16, 512>(points, soa, B, index, L, s);
-    else if (L.k >= 2048)
-        // The region kernel's sort costs about 0.15 ms per call, which the skipped updates
-        // repay once a few thousand points are sampled from more than 8192 (16384 -> 4096:
-        // 3.35 -> 2.9 ms; 16384 -> 512 would go from 0.52 to 0.61 ms).
+    else if (L.k >= 256)
         return fps_region_launch_f32<16>(points, soa, B, index, L, s);
     else
         fps_launch_f32<32, 512>(points, soa, B, index, L, s);
