@@ -51,9 +51,9 @@ PAIRS_PER_MATRIX_INSTRUCTION = 1024  # v_mfma_f32_32x32x16_f16: 32 keys x 32 que
 # HBM bytes per launch at B=32, N=M=16384 cannot be measured from inside the run: they come
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by a copy kernel of
 # known size, and are kept in the profile summaries named here.
-CHAMFER_SORTED_TRAFFIC_BYTES = 128.8e6
+CHAMFER_SORTED_TRAFFIC_BYTES = 129.0e6
 CHAMFER_SORTED_TRAFFIC_SOURCE = "profiles/chamfer_forward_sorted_B32_N16384.md"
-CHAMFER_TRAFFIC_BYTES = 55.8e6
+CHAMFER_TRAFFIC_BYTES = 55.7e6
 CHAMFER_TRAFFIC_SOURCE = "profiles/chamfer_forward_mfma_B32_N16384.md"
 
 
