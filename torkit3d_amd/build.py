@@ -96,6 +96,7 @@ def build(verbose=False, jobs=None):
     run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH + ".tmp"]
         + objects)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    shutil.rmtree(objdir, ignore_errors=True)  # (objects are rebuilt by every call anyway)
     return LIB_PATH
 
 

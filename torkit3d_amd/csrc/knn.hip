@@ -441,7 +441,11 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 //     canonical d2, |k'|^2 as staged, thr itself             10 u R + 3 u (M + R)
 // below 59 u R + 40 u M; the kernel uses slack = 64 u R + 48 u M. Queries further than 200
 // from the centre (rescaled; thr would leave fp16's range) take every key as a candidate.
-template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK>
+// KI_LDS: the key indices of the slots live in LDS (16-bit, so clouds of up to 65536 keys),
+// one column per lane: they are only written during the sweep, and a write into a column of
+// one's own is one instruction where the slot in registers takes a select per slot.
+template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK,
+          bool KI_LDS = false>
 __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
@@ -469,6 +473,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
         skey[STAGING_FLOATS > TRANSPOSE_FLOATS ? STAGING_FLOATS : TRANSPOSE_FLOATS];
     float4 *const sraw = reinterpret_cast<float4 *>(skey + SCORE_FLOATS);
     uint4 *const sterm = reinterpret_cast<uint4 *>(skey);
+    extern __shared__ __align__(16) unsigned short knn_filter_ski[];  // KI_LDS: [QPL][KMAX][LANES]
     const int half = (threadIdx.x >> 5) & 1;
     __shared__ float sred[NW][8];
     const int tid = threadIdx.x;
@@ -565,7 +570,10 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     // pattern of -inf (below everything) and is recomputed when the results are written, and
     // a NaN in slot 0 freezes the query (maximum -inf: no key compares below it).
     int kd[QPL][KMAX];
-    int ki[QPL][KMAX];
+    int ki[QPL][KI_LDS ? 1 : KMAX];
+    auto ski = [&](int i, int slot) -> unsigned short & {
+        return knn_filter_ski[(i * KMAX + slot) * LANES + threadIdx.x];
+    };
     float max_key[QPL];
     int max_idx[QPL];
     unsigned nan_slots[QPL];
@@ -611,14 +619,18 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
 #pragma unroll
         for (int s = 0; s < KMAX; ++s) {
             kd[i][s] = NEG_INF_BITS;
-            ki[i][s] = 0;
+            if constexpr (KI_LDS)
+                ski(i, s) = (unsigned short)(s < k ? s : 0);
+            else
+                ki[i][s] = 0;
             if (s < k) {  // uniform
                 const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0),
                                                 knn_coord<SOA>(K, n2, s, 1),
                                                 knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
                 const bool isnan = d != d;
                 kd[i][s] = isnan ? NEG_INF_BITS : __builtin_bit_cast(int, d);
-                ki[i][s] = s;
+                if constexpr (!KI_LDS)
+                    ki[i][s] = s;
                 nan_slots[i] |= isnan ? (1u << s) : 0u;
                 frozen |= isnan && s == 0;
                 if (s == 0 || d > max_key[i]) {
@@ -694,7 +706,12 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
             for (int s = 0; s < KMAX; ++s) {
                 const bool here = ins && s == max_idx[i];
                 kd[i][s] = here ? dbits : kd[i][s];
-                ki[i][s] = here ? kj[i] : ki[i][s];
+                if constexpr (!KI_LDS)
+                    ki[i][s] = here ? kj[i] : ki[i][s];
+            }
+            if constexpr (KI_LDS) {
+                if (ins)
+                    ski(i, max_idx[i]) = (unsigned short)kj[i];
             }
             // ... and the new maximum is the largest pattern: it stays in the written slot
             // when nothing is strictly above the new key, otherwise it is the first slot
@@ -742,8 +759,11 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
             asm volatile("" : "+v"(pq[i].b0), "+v"(pq[i].b1), "+v"(pq[i].b2), "+v"(pq[i].b3));
             asm volatile("" : "+v"(qlen[i]), "+v"(pending[i]), "+v"(max_key[i]), "+v"(max_idx[i]));
 #pragma unroll
-            for (int s = 0; s < KMAX; ++s)
-                asm volatile("" : "+v"(kd[i][s]), "+v"(ki[i][s]));
+            for (int s = 0; s < KMAX; ++s) {
+                asm volatile("" : "+v"(kd[i][s]));
+                if constexpr (!KI_LDS)
+                    asm volatile("" : "+v"(ki[i][s]));
+            }
         }
     };
     auto must_serve = [&]() {
@@ -987,7 +1007,10 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
                                     knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
             kd[i][s] = __builtin_bit_cast(int, d);
             tbuf[lane * ROW + s] = d;
-            ibuf[lane * ROW + s] = ki[i][s];
+            if constexpr (KI_LDS)
+                ibuf[lane * ROW + s] = (int)ski(i, s);
+            else
+                ibuf[lane * ROW + s] = ki[i][s];
         }
         const int nvalid = n1 - q0 < TK_WAVE ? n1 - q0 : TK_WAVE;  // may be <= 0
         const int total = nvalid * k;
@@ -2136,6 +2159,18 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
     const int64_t bpb = ((int64_t)n1 + 511) / 512;
     if (B * bpb > TK_MAX_I32 || !(whatever_the_size || knn_filter_takes(B, n1, n2, k)))
         return TK3D_ERR_UNSUPPORTED;
+    if constexpr (KMAX == 16) {
+        if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
+            constexpr auto kernel = knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512, true>;
+            constexpr int lds = KMAX * 512 * (int)sizeof(unsigned short);
+            const int allowed = tk_allow_dynamic_lds<kernel>(lds);
+            if (allowed != TK3D_OK)
+                return allowed;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(512), lds, s, query, key,
+                               distance, index, weight, eps, (int)bpb, n1, n2, k);
+            return tk_launch_status();
+        }
+    }
     hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512>),
                        dim3((unsigned)(B * bpb)), dim3(512), 0, s, query, key, distance, index,
                        weight, eps, (int)bpb, n1, n2, k);
