@@ -448,3 +448,21 @@ def test_shapes_the_reference_author_profiled(cuda, b, n1, n2, k):
     q = torch.randn(b, n1, 3, generator=g)
     key = torch.randn(b, n2, 3, generator=g)
     check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("n2,k", [(65536, 16), (65537, 16), (70001, 11)])
+def test_prefilter_kernel_around_the_16_bit_index_limit(cuda, n2, k):
+    # With up to 65536 keys the 16-slot pre-filter kernel keeps its slots' key indices in LDS
+    # as 16-bit values, beyond that in registers; both forced through the test-only entry
+    # point, with the winners placed at the far end of the cloud
+    from debug_abi import knn_filter
+
+    g = gen(n2 + k)
+    q, key = uniform_cloud(g, 1, 700), uniform_cloud(g, 1, n2)
+    key[0, -40:] = q[0, :40] + 1e-4      # the last keys are the nearest of the first queries
+    got = knn_filter(q.to(cuda), key.to(cuda), k)
+    assert got is not None
+    od, oi = oracle.knn(q.numpy(), key.numpy(), k)
+    np.testing.assert_array_equal(got[0].cpu().numpy(), od)
+    np.testing.assert_array_equal(got[1].cpu().numpy(), oi)
+    assert int(oi.max()) >= n2 - 40
