@@ -136,6 +136,28 @@ def test_disjoint_and_nested_clouds(cuda):
     assert sum(handed_over(ws, 2)) == 0
 
 
+def test_queries_clustered_inside_a_shell_of_keys_are_handed_over(cuda):
+    # All queries in a small cluster at the centre of a shell of keys: every key tile is about
+    # as far from them as the nearest one, and every wave would sweep nearly all of them.
+    # From 256 key tiles (8192 keys) on that direction is handed over as well (the other way
+    # round the keys are dwarfed); inside a filled cube of keys the same cluster has a few
+    # tiles next to it and stays on the sorted path, and so does a shell of fewer tiles.
+    g = gen(22)
+    shell, cluster = sphere_cloud(g, 2, 9000), sphere_cloud(g, 2, 8200) * 0.01
+    ws = check_sorted(cluster, shell, cuda)
+    assert handed_over(ws, 2) == [1, 1, 1, 1]
+    ws = check_sorted(shell, cluster, cuda)
+    assert handed_over(ws, 2) == [1, 1, 1, 1]
+    ws = check_sorted(cluster, uniform_cloud(g, 2, 9000), cuda)
+    assert handed_over(ws, 2) == [0, 0, 1, 1]
+    ws = check_sorted(cluster + 0.5, uniform_cloud(g, 2, 9000), cuda)   # off centre
+    assert handed_over(ws, 2) == [0, 0, 1, 1]
+    ws = check_sorted(cluster + 3.0, uniform_cloud(g, 2, 9000), cuda)   # outside the keys
+    assert handed_over(ws, 2) == [0, 0, 1, 1]
+    ws = check_sorted(cluster, sphere_cloud(g, 2, 8000), cuda)          # 250 tiles
+    assert handed_over(ws, 2) == [0, 0, 1, 1]
+
+
 def test_keys_crowded_into_few_cells_are_handed_over(cuda):
     # A few hundred distinct points on a line, each repeated about 50 times: over a hundred
     # keys per occupied cell of the 32^3 grid, several tiles of equal keys in front of every
