@@ -444,8 +444,27 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
 // KI_LDS: the key indices of the slots live in LDS (16-bit, so clouds of up to 65536 keys),
 // one column per lane: they are only written during the sweep, and a write into a column of
 // one's own is one instruction where the slot in registers takes a select per slot.
+//
+// SORTED (16 slots, key indices in LDS): the registers hold the distances in descending
+// order instead of slot order, and a 64-bit word holds the slot number of every position,
+// a nibble each. MinK's maximum is then position 0, and an insertion is one v_med3_i32 per
+// position (remove the head, let the new key x sink to its place: position p becomes the
+// median of its old value, its lower neighbour's and x) plus a rotation of the nibbles of
+// positions 0..m, m being x's new position, found by a binary search through the registers
+// (4 compares, 11 selects): 86 instructions per step where the slot-ordered registers take
+// 116 (a select per slot to write, a max3 tree and a sign-bit scan for the first slot that
+// holds the new maximum). MinK's order among equal distances (mink.cuh:74-87: the rescan
+// starts from the inserted key and moves on only to a strictly larger one, so the maximum
+// is the inserted slot if nothing is strictly above it, else the lowest slot holding the
+// largest distance) becomes: equal distances are kept in ascending slot order, except
+// that a key with nothing strictly above it goes to the head. With R the list without its
+// head, x goes to position 0 if no element of R is above it, else behind the elements of R
+// that are above it or equal to it with a lower slot number. Equal distances are rare
+// outside quantised clouds: the binary search counts the elements >= x and hands back the
+// last of them; only when that equals x in some lane does the wave count both kinds
+// position by position.
 template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK,
-          bool KI_LDS = false>
+          bool KI_LDS = false, bool SORTED = false>
 __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     const float *__restrict__ query, const float *__restrict__ key,
     float *__restrict__ distance, int64_t *__restrict__ index, float *__restrict__ weight,
@@ -459,6 +478,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     constexpr int T = 6;
     constexpr int PER = STAGE / BLOCK;
     static_assert(STAGE % BLOCK == 0 && STAGE % CHUNK == 0, "stage shape");
+    static_assert(!SORTED || (KI_LDS && QPL == 1 && KMAX == 16 && !WEIGHTS),
+                  "the sorted list is written out for one query of 16 slots per lane");
     static_assert(2 * STAGE * 4 * (int)sizeof(float) >= KNN_STAGE * 4 * (int)sizeof(float),
                   "the staging buffers double as the exact sweep's stage");
     // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
@@ -577,7 +598,15 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     float max_key[QPL];
     int max_idx[QPL];
     unsigned nan_slots[QPL];
+    unsigned long long ids[QPL];  // SORTED: nibble p = the slot of position p of kd
     constexpr int NEG_INF_BITS = (int)0xff800000u;
+    constexpr int INT_LOWEST = (int)0x80000000u, INT_HIGHEST = 0x7fffffff;
+    // the median of three (v_med3_i32)
+    auto med3 = [](int a, int b, int c) {
+        const int lo = a < b ? a : b, hi = a < b ? b : a;
+        const int t = hi < c ? hi : c;
+        return lo > t ? lo : t;
+    };
     // Pending chunk masks per query, oldest first (bit 31 = first key of the chunk), and
     // the key index of bit 31 of each. Named members and no loops over the queue, so it
     // stays in registers (an array indexed through a loop ends up in scratch memory).
@@ -616,13 +645,47 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
         max_idx[i] = 0;
         nan_slots[i] = 0u;
         bool frozen = false;
+        ids[i] = 0xfedcba9876543210ull;
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s)
+            kd[i][s] = NEG_INF_BITS;
 #pragma unroll
         for (int s = 0; s < KMAX; ++s) {
-            kd[i][s] = NEG_INF_BITS;
             if constexpr (KI_LDS)
                 ski(i, s) = (unsigned short)(s < k ? s : 0);
             else
                 ki[i][s] = 0;
+            if constexpr (SORTED) {
+                if (s < k) {  // uniform
+                    const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0),
+                                                    knn_coord<SOA>(K, n2, s, 1),
+                                                    knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
+                    const bool isnan = d != d;
+                    const int x = isnan ? NEG_INF_BITS : __builtin_bit_cast(int, d);
+                    nan_slots[i] |= isnan ? (1u << s) : 0u;
+                    frozen |= isnan && s == 0;
+                    // Positions 0..s-1 hold the keys so far, all of lower slot numbers: key s
+                    // goes behind those that are >= it, the rest move down one position
+                    // (position s held the placeholder of slot s).
+                    int m = 0;
+#pragma unroll
+                    for (int p = 0; p < s; ++p)
+                        m += kd[i][p] >= x ? 1 : 0;
+#pragma unroll
+                    for (int p = s; p >= 1; --p)
+                        kd[i][p] = med3(kd[i][p - 1], kd[i][p], x);
+                    kd[i][0] = kd[i][0] > x ? kd[i][0] : x;
+                    if (s > 0) {
+                        // nibbles m..s move up one position, slot s enters at position m
+                        const unsigned long long field =
+                            (~0ull >> (60 - 4 * s)) & (~0ull << (4 * m));
+                        const unsigned long long moved =
+                            ((ids[i] & field) << 4) & field;
+                        ids[i] = (ids[i] & ~field) | moved | ((unsigned long long)s << (4 * m));
+                    }
+                }
+                continue;
+            }
             if (s < k) {  // uniform
                 const float d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0),
                                                 knn_coord<SOA>(K, n2, s, 1),
@@ -639,6 +702,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
                 }
             }
         }
+        if constexpr (SORTED)
+            max_key[i] = __builtin_bit_cast(float, kd[i][0]);  // (-inf if every key is a NaN)
         max_key[i] = frozen ? -INF : max_key[i];
         pq[i] = Pending{0u, 0u, 0u, 0u, 0, 0, 0, 0};
         qlen[i] = 0;
@@ -701,6 +766,47 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
             const float d = tk_dist2<float>(raw[i].x, raw[i].y, raw[i].z, qx[i], qy[i], qz[i]);
             const bool ins = has[i] && d < max_key[i];  // MinK's strict test (mink.cuh:74)
             const int dbits = __builtin_bit_cast(int, d);
+            if constexpr (SORTED) {
+                int(&v)[KMAX] = kd[i];
+                // a key that is not inserted sinks nowhere: above every pattern
+                const int x = ins ? dbits : INT_HIGHEST;
+                // m: how many of positions 1..15 are >= x; last: the last of them
+                const bool b3 = v[8] >= x;
+                const int p2 = b3 ? v[12] : v[4];
+                const bool b2 = p2 >= x;
+                const int t0 = b2 ? v[6] : v[2], t1 = b2 ? v[14] : v[10];
+                const int p1 = b3 ? t1 : t0;
+                const bool b1 = p1 >= x;
+                const int u0 = b1 ? v[3] : v[1], u1 = b1 ? v[7] : v[5];
+                const int u2 = b1 ? v[11] : v[9], u3 = b1 ? v[15] : v[13];
+                const int w0 = b2 ? u1 : u0, w1 = b2 ? u3 : u2;
+                const int p0 = b3 ? w1 : w0;
+                const bool b0 = p0 >= x;
+                int m = (b3 ? 8 : 0) + (b2 ? 4 : 0) + (b1 ? 2 : 0) + (b0 ? 1 : 0);
+                const int last = b0 ? p0 : b1 ? p1 : b2 ? p2 : b3 ? v[8] : INT_LOWEST;
+                const unsigned slot = (unsigned)ids[i] & 15u;  // of the maximum: x takes it
+                if (__builtin_amdgcn_ballot_w64(last == x) != 0) {  // uniform: equal distances
+                    int above = 0, before = 0;
+#pragma unroll
+                    for (int p = 1; p < KMAX; ++p) {
+                        const unsigned other = (unsigned)(ids[i] >> (4 * p)) & 15u;
+                        above += v[p] > x ? 1 : 0;
+                        before += (v[p] == x && other < slot) ? 1 : 0;
+                    }
+                    m = above == 0 ? 0 : above + before;
+                }
+#pragma unroll
+                for (int p = 0; p < KMAX; ++p)
+                    v[p] = med3(v[p], p + 1 < KMAX ? v[p + 1] : INT_LOWEST, x);
+                // the nibbles of positions 0..m turn by one: the head's slot goes to m
+                const unsigned long long turning = ~0ull >> (60 - 4 * m);
+                ids[i] = (ids[i] & ~turning) | ((ids[i] & turning) >> 4) |
+                         ((unsigned long long)slot << (4 * m));
+                if (ins)
+                    ski(i, slot) = (unsigned short)kj[i];
+                max_key[i] = ins ? __builtin_bit_cast(float, v[0]) : max_key[i];
+                continue;
+            }
             // the key takes the slot of the maximum ...
 #pragma unroll
             for (int s = 0; s < KMAX; ++s) {
@@ -758,6 +864,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
             asm volatile("" : "+v"(pq[i].m0), "+v"(pq[i].m1), "+v"(pq[i].m2), "+v"(pq[i].m3));
             asm volatile("" : "+v"(pq[i].b0), "+v"(pq[i].b1), "+v"(pq[i].b2), "+v"(pq[i].b3));
             asm volatile("" : "+v"(qlen[i]), "+v"(pending[i]), "+v"(max_key[i]), "+v"(max_idx[i]));
+            if constexpr (SORTED)
+                asm volatile("" : "+v"(ids[i]));
 #pragma unroll
             for (int s = 0; s < KMAX; ++s) {
                 asm volatile("" : "+v"(kd[i][s]));
@@ -999,8 +1107,25 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
 #pragma unroll
     for (int i = 0; i < QPL; ++i) {
         const int q0 = (qblock * QPL + i) * BLOCK + wave * TK_WAVE;  // first query of the wave
+        if constexpr (SORTED) {
 #pragma unroll
-        for (int s = 0; s < KMAX; ++s) {
+            for (int p = 0; p < KMAX; ++p) {
+                const int slot = (int)((unsigned)(ids[i] >> (4 * p)) & 15u);
+                tbuf[lane * ROW + slot] = __builtin_bit_cast(float, kd[i][p]);
+                ibuf[lane * ROW + p] = (int)ski(i, p);
+            }
+            if (nan_slots[i] != 0u) {  // NaNs of the fill, still in their slots
+#pragma unroll
+                for (int s = 0; s < KMAX; ++s) {
+                    if (s < k && ((nan_slots[i] >> s) & 1u))
+                        tbuf[lane * ROW + s] = tk_dist2<float>(
+                            knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
+                            knn_coord<SOA>(K, n2, s, 2), qx[i], qy[i], qz[i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < (SORTED ? 0 : KMAX); ++s) {
             float d = __builtin_bit_cast(float, kd[i][s]);
             if (s < k && ((nan_slots[i] >> s) & 1u))  // a NaN of the fill, still in its slot
                 d = tk_dist2<float>(knn_coord<SOA>(K, n2, s, 0), knn_coord<SOA>(K, n2, s, 1),
@@ -2161,7 +2286,8 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
         return TK3D_ERR_UNSUPPORTED;
     if constexpr (KMAX == 16) {
         if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
-            constexpr auto kernel = knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512, true>;
+            constexpr auto kernel =
+                knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512, true, !WEIGHTS>;
             constexpr int lds = KMAX * 512 * (int)sizeof(unsigned short);
             const int allowed = tk_allow_dynamic_lds<kernel>(lds);
             if (allowed != TK3D_OK)
