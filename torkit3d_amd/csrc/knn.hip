@@ -786,12 +786,27 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
                 const int last = b0 ? p0 : b1 ? p1 : b2 ? p2 : b3 ? v[8] : INT_LOWEST;
                 const unsigned slot = (unsigned)ids[i] & 15u;  // of the maximum: x takes it
                 if (__builtin_amdgcn_ballot_w64(last == x) != 0) {  // uniform: equal distances
-                    int above = 0, before = 0;
-#pragma unroll
-                    for (int p = 1; p < KMAX; ++p) {
-                        const unsigned other = (unsigned)(ids[i] >> (4 * p)) & 15u;
-                        above += v[p] > x ? 1 : 0;
-                        before += (v[p] == x && other < slot) ? 1 : 0;
+                    // the same search for the positions strictly above x ...
+                    const bool c3 = v[8] > x;
+                    const int r2 = c3 ? v[12] : v[4];
+                    const bool c2 = r2 > x;
+                    const int e0 = c2 ? v[6] : v[2], e1 = c2 ? v[14] : v[10];
+                    const int r1 = c3 ? e1 : e0;
+                    const bool c1 = r1 > x;
+                    const int f0 = c1 ? v[3] : v[1], f1 = c1 ? v[7] : v[5];
+                    const int f2 = c1 ? v[11] : v[9], f3 = c1 ? v[15] : v[13];
+                    const int h0 = c2 ? f1 : f0, h1 = c2 ? f3 : f2;
+                    const int r0 = c3 ? h1 : h0;
+                    const bool c0 = r0 > x;
+                    const int above = (c3 ? 8 : 0) + (c2 ? 4 : 0) + (c1 ? 2 : 0) + (c0 ? 1 : 0);
+                    // ... and positions above + 1 .. m hold x, in ascending slot order: x goes
+                    // behind those of lower slots
+                    const int equal = m - above;
+                    int before = 0;
+                    for (int q = 0; __builtin_amdgcn_ballot_w64(q < equal) != 0; ++q) {
+                        const unsigned other =
+                            (unsigned)(ids[i] >> ((4 * (above + 1 + q)) & 63)) & 15u;
+                        before += (q < equal && other < slot) ? 1 : 0;
                     }
                     m = above == 0 ? 0 : above + before;
                 }
