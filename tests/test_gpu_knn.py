@@ -332,7 +332,7 @@ def _filter_case(kind, g, k, b=8, n1=8192 + 5, n2=2048 + 37):  # ragged: partial
     return q.contiguous(), key.contiguous()
 
 
-@pytest.mark.parametrize("k", [1, 3, 4, 7, 16])
+@pytest.mark.parametrize("k", [1, 3, 4, 7, 9, 13, 16])
 @pytest.mark.parametrize("kind", ["uniform", "lattice", "far_to_near", "near_to_far",
                                   "far_from_origin", "separated", "tiny", "huge", "huge_queries",
                                   "scaled_small", "scaled_large", "far_queries",
@@ -340,6 +340,24 @@ def _filter_case(kind, g, k, b=8, n1=8192 + 5, n2=2048 + 37):  # ragged: partial
 def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
     q, key = _filter_case(kind, gen(sum(map(ord, kind)) + k), k)
     check_raw(q, key, k, cuda)
+
+
+@pytest.mark.parametrize("k", [9, 12, 16])
+@pytest.mark.parametrize("steps", [1, 2, 16])
+def test_prefiltered_kernel_with_sorted_slots_on_equal_distances(cuda, steps, k):
+    # For 9 to 16 neighbours the kernel keeps a query's distances in descending order and the
+    # slot numbers beside them; among equal distances MinK's rescan (mink.cuh:74-87) decides
+    # which slot is overwritten next: the slot just written if nothing is strictly above it,
+    # else the lowest slot holding the largest distance. Lattices of 3, 5 and 33 positions
+    # per axis: a handful of distinct distances, so nearly every insertion meets equals, and
+    # runs of equals that are longer than the list.
+    g = gen(100 * steps + k)
+    check_raw(lattice_cloud(g, 4, 8192 + 5, steps), lattice_cloud(g, 4, 2048 + 37, steps), k, cuda)
+    # the same keys sorted from far to near the first query, so that every key is inserted
+    key = lattice_cloud(g, 4, 2048 + 37, steps)
+    order = key.norm(dim=2).argsort(dim=1, descending=True)
+    key = torch.gather(key, 1, order[:, :, None].expand(-1, -1, 3)).contiguous()
+    check_raw(0.01 * uniform_cloud(g, 4, 8192 + 5), key, k, cuda)
 
 
 # ---- k = 17..32 with 32768 to 131071 queries against 4096 keys or more: the same matrix
