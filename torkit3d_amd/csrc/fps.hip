@@ -570,6 +570,8 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
     __shared__ float4 s_cand[2][NW];  // a wave's candidate: x, y, z, running minimum (bits)
     __shared__ int2 s_aux[2][NW];     // the wave's second-largest minimum, the candidate's rank
     __shared__ int s_rank[2][NW];     // a candidate's rank among them, + 256: it passed
+    __shared__ int s_byrank[2][NW];   // by rank: the exchange's number << 9, + 256: that one passed
+    __shared__ float s_tau[2];        // the running minimum of the candidate of rank 0
     __shared__ float s_box[NW][NB][8];  // lo.xyz, hi.xyz of a wave's block
     __shared__ float s_red[NW][8];
 
@@ -914,8 +916,16 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
                 const unsigned m_fine = (~m_before | (m_far & m_alone)) & 0xffffu;
                 const int verdict =
                     __builtin_popcount(m_before) | ((vw > 0 && m_fine == 0xffffu) ? 256 : 0);
-                if (lane == 0)
+                if (lane == 0) {
+                    // (The table by rank saves every wave the folding of sixteen verdicts into
+                    // one mask, scalar work that sixteen waves repeated. Candidates without a
+                    // point left share a rank: an entry counts only with this exchange's
+                    // number on it.)
                     s_rank[buf][wave] = verdict;
+                    s_byrank[buf][verdict & 15] = (round << 9) | (verdict & 256);
+                    if ((verdict & 255) == 0)
+                        s_tau[buf] = W.w;
+                }
             }
             __syncthreads();
             const float4 A = s_cand[buf][ca];
@@ -925,26 +935,15 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
             ay = A.y;
             az = A.z;
             const int rank = verdict & 255;  // a permutation of the live candidates
-            const unsigned long long fine = __builtin_amdgcn_ballot_w64(verdict >= 256);
-            // Lane (a, q) asks whether candidate a has rank q + 4 i and passed; folding the
-            // nibbles of that mask together gives, in bit q, whether the candidate of that rank
-            // passed.
-            unsigned passed = 0u;
-#pragma unroll
-            for (int i = 0; i < (MAXM + 3) / 4; ++i) {
-                unsigned long long m = __builtin_amdgcn_ballot_w64(rank == 4 * i + cb) & fine;
-                m |= m >> 32;
-                m |= m >> 16;
-                m |= m >> 8;
-                m |= m >> 4;
-                passed |= ((unsigned)m & 0xfu) << (4 * i);
-            }
+            // lane r (of the first sixteen): did the candidate of rank r pass
+            const int by_rank = s_byrank[buf][lane & 15];
+            const unsigned passed =
+                (unsigned)__builtin_amdgcn_ballot_w64(by_rank == ((round << 9) | 256)) & 0xffffu;
             const int left = L.k - it;  // steps still wanted
             int good = __builtin_ctz(~passed | (1u << MAXM));  // ranks 0..good-1 passed
             good = good < left ? good : left;
             // tau and the reach of candidate a into block q: as with eight waves
-            const float tau =
-                read_lane(A.w, __builtin_ctzll(__builtin_amdgcn_ballot_w64(rank == 0)));
+            const float tau = s_tau[buf];  // (stale without a live candidate: unused then)
             const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
             const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
             const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
