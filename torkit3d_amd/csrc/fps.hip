@@ -882,46 +882,48 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
             s_aux[buf][wave] = make_int2(second, pick_rank);
         }
         __syncthreads();
-        // Every wave now works out, redundantly and without a serial chain, how many of
-        // the candidates are certain winners of the coming steps. All 64 lanes are active,
-        // so conditions are combined as lane masks in scalar registers.
+        // How many of the candidates are certain winners of the coming steps. All 64 lanes are
+        // active, so conditions are combined as lane masks in scalar registers.
         {
-            // Sixteen candidates. All waves working through all 256 relations would put four
-            // copies of a long chain on every SIMD; instead a wave ranks its own candidate
-            // against the sixteen (lane b holds candidate b; a condition is one ballot), leaves
-            // rank and verdict in LDS, and after a second barrier every wave reads the sixteen
-            // verdicts.
-            const float4 W = s_cand[buf][wave];  // (uniform)
-            const int2 Wx = s_aux[buf][wave];
-            const float4 Bc = s_cand[buf][lane & 15];
-            const int2 Bx = s_aux[buf][lane & 15];
-            {
+            // Sixteen candidates, 256 relations between them. Four waves (one per SIMD) rank
+            // four candidates each: lane (c, b) = (lane / 16, lane % 16) compares candidate
+            // 4 wave + c with candidate b, a condition is one ballot whose sixteen-bit groups
+            // belong to the four candidates, and rank and verdict go to LDS, where every wave
+            // reads them after a second barrier. (Every wave ranking its own candidate in
+            // sixteen of its lanes put four copies of the chain on every SIMD; all waves
+            // working through all 256 relations, sixteen.)
+            if (wave < NW / 4) {  // uniform
+                const int mine = 4 * wave + (lane >> 4), other = lane & 15;
+                const float4 W = s_cand[buf][mine];
+                const int2 Wx = s_aux[buf][mine];
+                const float4 Bc = s_cand[buf][other];
+                const int2 Bx = s_aux[buf][other];
                 const int vw = __builtin_bit_cast(int, W.w), vb = __builtin_bit_cast(int, Bc.w);
-                unsigned m_before = (unsigned)__builtin_amdgcn_ballot_w64(vb > vw) & 0xffffu;
-                const unsigned m_equal = (unsigned)__builtin_amdgcn_ballot_w64(vb == vw) & 0xffffu;
-                // b comes before the wave's candidate in the reference's order: larger value,
-                // then lower position; positions are looked up only when two candidates really
-                // hold the same value
-                if (vw > 0 && (m_equal & ~(1u << wave)) != 0u) {  // uniform
+                // b comes before the candidate in the reference's order: larger value, then
+                // lower position; positions are looked up only when two candidates really hold
+                // the same value
+                bool before = vb > vw;
+                const bool equal = vb == vw && other != mine && vw > 0;
+                if (__builtin_amdgcn_ballot_w64(equal) != 0ull) {  // uniform
                     const int pos_w = fps_position_of_point((int)(unsigned)keys[Wx.y], L);
                     const int pos_b = fps_position_of_point((int)(unsigned)keys[Bx.y], L);
-                    m_before |= m_equal & (unsigned)__builtin_amdgcn_ballot_w64(pos_b < pos_w);
+                    before |= equal && pos_b < pos_w;
                 }
                 const float dwb = tk_dist2<float>(W.x, W.y, W.z, Bc.x, Bc.y, Bc.z);
                 // the candidate survives b's selection: b's update leaves its minimum alone, and
                 // b's wave holds nothing else at or above it
-                const unsigned m_far =
-                    (unsigned)__builtin_amdgcn_ballot_w64(__builtin_bit_cast(int, dwb) >= vw);
-                const unsigned m_alone = (unsigned)__builtin_amdgcn_ballot_w64(Bx.x < vw);
-                const unsigned m_fine = (~m_before | (m_far & m_alone)) & 0xffffu;
-                const int verdict =
-                    __builtin_popcount(m_before) | ((vw > 0 && m_fine == 0xffffu) ? 256 : 0);
-                if (lane == 0) {
+                const bool fine = !before || (__builtin_bit_cast(int, dwb) >= vw && Bx.x < vw);
+                const unsigned long long m_before = __builtin_amdgcn_ballot_w64(before);
+                const unsigned long long m_fine = __builtin_amdgcn_ballot_w64(fine);
+                const unsigned mb = (unsigned)(m_before >> (lane & 48)) & 0xffffu;
+                const unsigned mf = (unsigned)(m_fine >> (lane & 48)) & 0xffffu;
+                const int verdict = __builtin_popcount(mb) | ((vw > 0 && mf == 0xffffu) ? 256 : 0);
+                if (other == 0) {
                     // (The table by rank saves every wave the folding of sixteen verdicts into
                     // one mask, scalar work that sixteen waves repeated. Candidates without a
                     // point left share a rank: an entry counts only with this exchange's
                     // number on it.)
-                    s_rank[buf][wave] = verdict;
+                    s_rank[buf][mine] = verdict;
                     s_byrank[buf][verdict & 15] = (round << 9) | (verdict & 256);
                     if ((verdict & 255) == 0)
                         s_tau[buf] = W.w;
