@@ -929,9 +929,25 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
                         s_tau[buf] = W.w;
                 }
             }
+            // Candidate a for lane (a, q) and how near it comes to the box of block q: known
+            // since the first barrier. The twelve waves that have nothing to rank work that
+            // out while they would wait, the four others behind the second barrier.
+            float4 A;
+            int2 Ax;  // its wave's second-largest minimum, its sorted rank
+            float bound;
+            auto approach = [&]() {
+                A = s_cand[buf][ca];
+                Ax = s_aux[buf][ca];
+                const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
+                const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
+                const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
+                bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
+            };
+            if (wave >= NW / 4)  // uniform
+                approach();
             __syncthreads();
-            const float4 A = s_cand[buf][ca];
-            const int2 Ax = s_aux[buf][ca];  // its wave's second-largest minimum, its sorted rank
+            if (wave < NW / 4)  // uniform
+                approach();
             const int verdict = s_rank[buf][ca];
             ax = A.x;
             ay = A.y;
@@ -946,10 +962,6 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
             good = good < left ? good : left;
             // tau and the reach of candidate a into block q: as with eight waves
             const float tau = s_tau[buf];  // (stale without a live candidate: unused then)
-            const float gx = __builtin_fmaxf(__builtin_fmaxf(box_lo[0] - A.x, A.x - box_hi[0]), 0.0f);
-            const float gy = __builtin_fmaxf(__builtin_fmaxf(box_lo[1] - A.y, A.y - box_hi[1]), 0.0f);
-            const float gz = __builtin_fmaxf(__builtin_fmaxf(box_lo[2] - A.z, A.z - box_hi[2]), 0.0f);
-            const float bound = __builtin_fmaf(gz, gz, __builtin_fmaf(gy, gy, gx * gx));
             reach = __builtin_amdgcn_ballot_w64(!(bound >= tau));
             centres = __builtin_amdgcn_ballot_w64(rank < good) & 0x1111111111111111ull;
             if (good > 0) {  // uniform
