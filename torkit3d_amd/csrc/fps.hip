@@ -542,10 +542,12 @@ __device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
 // Sixteen waves of 16 points per lane instead of eight of 32: an exchange accepts 4.4
 // candidates on uniform clouds where eight waves accepted 3.1, the walk to the winner's leaf
 // is a level shorter and the regions are half the size. The price is what every wave repeats
-// per exchange, now sixteen times on four SIMDs, so that part is kept short: a wave ranks
-// only its own candidate against the sixteen (one ballot per condition) and the verdicts
-// meet in LDS behind a second barrier; the wave's runner-up comes from a second plain
-// maximum scan that runs beside the walk instead of a scan that carries pairs.
+// per exchange, now sixteen times on four SIMDs, so that part is kept short: four waves, one
+// per SIMD, rank four candidates each (one ballot per condition) while the others work out
+// how near the candidates come to their boxes, and ranks and verdicts meet in LDS behind a
+// second barrier, as tables that one read and one ballot turn into the mask of certain
+// winners; the wave's runner-up comes from a second plain maximum scan that runs beside the
+// walk instead of a scan that carries pairs.
 //
 // Ties. With this layout the lane order is no longer the reference's priority order
 // (see the top of the file), so equal maxima are resolved explicitly: a wave that holds
