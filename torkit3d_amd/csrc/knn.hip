@@ -373,6 +373,122 @@ __global__ __launch_bounds__(KNN_BLOCK) void knn_batched_kernel_f32(
                                          k, skey);
 }
 
+// The slot number of every position of a sorted list of KMAX distances (see SORTED below).
+// Up to 16 positions: a nibble each in one 64-bit word. 32 positions: the low nibbles in two
+// 64-bit words and the fifth bits in a 32-bit word.
+template <int KMAX> struct KnnSlotNumbers;
+
+template <> struct KnnSlotNumbers<16> {
+    unsigned long long w;
+    __device__ __forceinline__ void identity() { w = 0xfedcba9876543210ull; }
+    __device__ __forceinline__ unsigned head() const { return (unsigned)w & 15u; }
+    __device__ __forceinline__ unsigned at(int p) const { return (unsigned)(w >> ((4 * p) & 63)) & 15u; }
+    // positions 0..m turn by one towards the head; `slot` (the old head's) goes to position m
+    __device__ __forceinline__ void turn(int m, unsigned slot)
+    {
+        const unsigned long long turning = ~0ull >> (60 - 4 * m);
+        w = (w & ~turning) | ((w & turning) >> 4) | ((unsigned long long)slot << (4 * m));
+    }
+    // positions m..s move one position down (s is a compile-time constant, s > 0), `slot`
+    // enters at position m
+    __device__ __forceinline__ void make_room(int m, int s, unsigned slot)
+    {
+        const unsigned long long field = (~0ull >> (60 - 4 * s)) & (~0ull << (4 * m));
+        w = (w & ~field) | (((w & field) << 4) & field) | ((unsigned long long)slot << (4 * m));
+    }
+    __device__ __forceinline__ void keep() { asm volatile("" : "+v"(w)); }
+};
+
+template <> struct KnnSlotNumbers<32> {
+    unsigned long long w0, w1;  // low nibbles of positions 0..15 and 16..31
+    unsigned fifth;             // bit p: the fifth bit of position p's slot
+    __device__ __forceinline__ void identity()
+    {
+        w0 = w1 = 0xfedcba9876543210ull;
+        fifth = 0xffff0000u;
+    }
+    __device__ __forceinline__ unsigned head() const
+    {
+        return ((unsigned)w0 & 15u) | ((fifth & 1u) << 4);
+    }
+    __device__ __forceinline__ unsigned at(int p) const
+    {
+        const unsigned long long w = p < 16 ? w0 : w1;
+        return ((unsigned)(w >> ((4 * p) & 63)) & 15u) | (((fifth >> (p & 31)) & 1u) << 4);
+    }
+    __device__ __forceinline__ void turn(int m, unsigned slot)
+    {
+        const unsigned turning5 = ~0u >> (31 - m);
+        fifth = (fifth & ~turning5) | ((fifth & turning5) >> 1) | ((slot >> 4) << m);
+        const bool far = m >= 16;
+        const unsigned long long low = slot & 15u;
+        // the first word turns as far as m reaches in it and takes the second word's first
+        // nibble, or the slot, at the end of that range
+        const int m0 = far ? 15 : m;
+        const unsigned long long t0 = ~0ull >> (60 - 4 * m0);
+        const unsigned long long in0 = far ? (w1 & 15ull) : low;
+        w0 = (w0 & ~t0) | ((w0 & t0) >> 4) | (in0 << (4 * m0));
+        const int m1 = far ? m - 16 : 0;
+        const unsigned long long t1 = far ? ~0ull >> (60 - 4 * m1) : 0ull;
+        w1 = (w1 & ~t1) | ((w1 & t1) >> 4) | (far ? low << (4 * m1) : 0ull);
+    }
+    __device__ __forceinline__ void make_room(int m, int s, unsigned slot)
+    {
+        const unsigned field5 = (~0u >> (31 - s)) & (~0u << m);
+        fifth = (fifth & ~field5) | (((fifth & field5) << 1) & field5) | ((slot >> 4) << m);
+        const unsigned long long low = slot & 15u;
+        if (s < 16) {  // (compile-time) only the first word
+            const unsigned long long field = (~0ull >> (60 - 4 * s)) & (~0ull << (4 * m));
+            w0 = (w0 & ~field) | (((w0 & field) << 4) & field) | (low << (4 * m));
+        } else {
+            const bool far = m >= 16;  // the first word stays as it is
+            // second word: positions max(m, 16)..s move down; what enters at its start is
+            // the first word's last nibble, or the slot itself
+            const int m1 = far ? m - 16 : 0;
+            const unsigned long long f1 = (~0ull >> (60 - 4 * (s - 16))) & (~0ull << (4 * m1));
+            const unsigned long long in1 = far ? low : (w0 >> 60);
+            w1 = (w1 & ~f1) | (((w1 & f1) << 4) & f1) | (in1 << (4 * m1));
+            const unsigned long long f0 = far ? 0ull : ~0ull << (4 * m);
+            w0 = (w0 & ~f0) | ((w0 & f0) << 4) | (far ? 0ull : low << (4 * m));
+        }
+    }
+    __device__ __forceinline__ void keep() { asm volatile("" : "+v"(w0), "+v"(w1), "+v"(fifth)); }
+};
+
+// How many of positions 1..KMAX-1 of a descending list satisfy `above` (true for a prefix of
+// them), by bisection through the registers: the pivot of a level is chosen among its 2^level
+// possible places by selects on the outcomes so far (KMAX - 1 - log2 KMAX selects in all).
+// `last` returns the last position's value that satisfied it (`none` without one).
+template <int KMAX, typename Above>
+__device__ __forceinline__ int knn_sorted_position(const int (&v)[KMAX], Above above, int none,
+                                                   int &last)
+{
+    constexpr int LEVELS = KMAX == 32 ? 5 : KMAX == 16 ? 4 : KMAX == 8 ? 3 : 2;
+    static_assert((1 << LEVELS) == KMAX, "KMAX is a power of two from 4 to 32");
+    bool taken[LEVELS];
+    int m = 0;
+    last = none;
+#pragma unroll
+    for (int level = 0; level < LEVELS; ++level) {
+        const int step = KMAX >> (level + 1);
+        int c[1 << (LEVELS - 1)];
+#pragma unroll
+        for (int j = 0; j < (1 << level); ++j)
+            c[j] = v[(2 * j + 1) * step];
+        // the outcome of the previous level is the lowest bit of the place, and so on
+#pragma unroll
+        for (int d = level - 1; d >= 0; --d) {
+#pragma unroll
+            for (int j = 0; j < (1 << d); ++j)
+                c[j] = taken[d] ? c[2 * j + 1] : c[2 * j];
+        }
+        taken[level] = above(c[0]);
+        last = taken[level] ? c[0] : last;
+        m = 2 * m + (taken[level] ? 1 : 0);
+    }
+    return m;
+}
+
 // fp32, k <= 16, launches with many queries: pre-filtered sweep with deferred insertions.
 //
 // Two costs dominate the batched kernel above: its sweep spends 8 vector instructions per
@@ -478,8 +594,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     constexpr int T = 6;
     constexpr int PER = STAGE / BLOCK;
     static_assert(STAGE % BLOCK == 0 && STAGE % CHUNK == 0, "stage shape");
-    static_assert(!SORTED || (KI_LDS && QPL == 1 && KMAX == 16 && !WEIGHTS),
-                  "the sorted list is written out for one query of 16 slots per lane");
+    static_assert(!SORTED || (KI_LDS && QPL == 1 && (KMAX == 16 || KMAX == 32) && !WEIGHTS),
+                  "the sorted list is for one query of 16 or 32 slots per lane");
     static_assert(2 * STAGE * 4 * (int)sizeof(float) >= KNN_STAGE * 4 * (int)sizeof(float),
                   "the staging buffers double as the exact sweep's stage");
     // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
@@ -488,7 +604,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     static_assert(!MATRIX || QPL == 1 || QPL == 2, "two or four blocks of 32 queries per wave");
     constexpr int SCORE_FLOATS = MATRIX ? 2 * STAGE * 8 : 2 * STAGE * 4 + 32;
     constexpr int STAGING_FLOATS = SCORE_FLOATS + 2 * STAGE * 4;
-    constexpr int TWAVES = NW < 4 ? NW : 4;  // waves that transpose their results together
+    // waves that transpose their results together (32 slots: two, 34 KB of LDS)
+    constexpr int TWAVES = NW < 4 ? NW : KMAX > 16 ? 2 : 4;
     constexpr int TRANSPOSE_FLOATS = TWAVES * 2 * TK_WAVE * (KMAX + 1);  // see the end of the kernel
     __shared__ __align__(16) float
         skey[STAGING_FLOATS > TRANSPOSE_FLOATS ? STAGING_FLOATS : TRANSPOSE_FLOATS];
@@ -598,7 +715,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     float max_key[QPL];
     int max_idx[QPL];
     unsigned nan_slots[QPL];
-    unsigned long long ids[QPL];  // SORTED: nibble p = the slot of position p of kd
+    KnnSlotNumbers<(SORTED ? KMAX : 16)> ids[QPL];  // SORTED: the slot of every position of kd
     constexpr int NEG_INF_BITS = (int)0xff800000u;
     constexpr int INT_LOWEST = (int)0x80000000u, INT_HIGHEST = 0x7fffffff;
     // the median of three (v_med3_i32)
@@ -645,7 +762,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
         max_idx[i] = 0;
         nan_slots[i] = 0u;
         bool frozen = false;
-        ids[i] = 0xfedcba9876543210ull;
+        ids[i].identity();
 #pragma unroll
         for (int s = 0; s < KMAX; ++s)
             kd[i][s] = NEG_INF_BITS;
@@ -675,14 +792,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
                     for (int p = s; p >= 1; --p)
                         kd[i][p] = med3(kd[i][p - 1], kd[i][p], x);
                     kd[i][0] = kd[i][0] > x ? kd[i][0] : x;
-                    if (s > 0) {
-                        // nibbles m..s move up one position, slot s enters at position m
-                        const unsigned long long field =
-                            (~0ull >> (60 - 4 * s)) & (~0ull << (4 * m));
-                        const unsigned long long moved =
-                            ((ids[i] & field) << 4) & field;
-                        ids[i] = (ids[i] & ~field) | moved | ((unsigned long long)s << (4 * m));
-                    }
+                    if (s > 0)
+                        ids[i].make_room(m, s, (unsigned)s);
                 }
                 continue;
             }
@@ -770,42 +881,22 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
                 int(&v)[KMAX] = kd[i];
                 // a key that is not inserted sinks nowhere: above every pattern
                 const int x = ins ? dbits : INT_HIGHEST;
-                // m: how many of positions 1..15 are >= x; last: the last of them
-                const bool b3 = v[8] >= x;
-                const int p2 = b3 ? v[12] : v[4];
-                const bool b2 = p2 >= x;
-                const int t0 = b2 ? v[6] : v[2], t1 = b2 ? v[14] : v[10];
-                const int p1 = b3 ? t1 : t0;
-                const bool b1 = p1 >= x;
-                const int u0 = b1 ? v[3] : v[1], u1 = b1 ? v[7] : v[5];
-                const int u2 = b1 ? v[11] : v[9], u3 = b1 ? v[15] : v[13];
-                const int w0 = b2 ? u1 : u0, w1 = b2 ? u3 : u2;
-                const int p0 = b3 ? w1 : w0;
-                const bool b0 = p0 >= x;
-                int m = (b3 ? 8 : 0) + (b2 ? 4 : 0) + (b1 ? 2 : 0) + (b0 ? 1 : 0);
-                const int last = b0 ? p0 : b1 ? p1 : b2 ? p2 : b3 ? v[8] : INT_LOWEST;
-                const unsigned slot = (unsigned)ids[i] & 15u;  // of the maximum: x takes it
+                // m: how many of positions 1..KMAX-1 are >= x; last: the last of them
+                int last;
+                int m = knn_sorted_position<KMAX>(v, [&](int pivot) { return pivot >= x; },
+                                                  INT_LOWEST, last);
+                const unsigned slot = ids[i].head();  // of the maximum: x takes it
                 if (__builtin_amdgcn_ballot_w64(last == x) != 0) {  // uniform: equal distances
                     // the same search for the positions strictly above x ...
-                    const bool c3 = v[8] > x;
-                    const int r2 = c3 ? v[12] : v[4];
-                    const bool c2 = r2 > x;
-                    const int e0 = c2 ? v[6] : v[2], e1 = c2 ? v[14] : v[10];
-                    const int r1 = c3 ? e1 : e0;
-                    const bool c1 = r1 > x;
-                    const int f0 = c1 ? v[3] : v[1], f1 = c1 ? v[7] : v[5];
-                    const int f2 = c1 ? v[11] : v[9], f3 = c1 ? v[15] : v[13];
-                    const int h0 = c2 ? f1 : f0, h1 = c2 ? f3 : f2;
-                    const int r0 = c3 ? h1 : h0;
-                    const bool c0 = r0 > x;
-                    const int above = (c3 ? 8 : 0) + (c2 ? 4 : 0) + (c1 ? 2 : 0) + (c0 ? 1 : 0);
+                    int unused;
+                    const int above = knn_sorted_position<KMAX>(
+                        v, [&](int pivot) { return pivot > x; }, INT_LOWEST, unused);
                     // ... and positions above + 1 .. m hold x, in ascending slot order: x goes
                     // behind those of lower slots
                     const int equal = m - above;
                     int before = 0;
                     for (int q = 0; __builtin_amdgcn_ballot_w64(q < equal) != 0; ++q) {
-                        const unsigned other =
-                            (unsigned)(ids[i] >> ((4 * (above + 1 + q)) & 63)) & 15u;
+                        const unsigned other = ids[i].at((above + 1 + q) & (KMAX - 1));
                         before += (q < equal && other < slot) ? 1 : 0;
                     }
                     m = above == 0 ? 0 : above + before;
@@ -813,10 +904,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
 #pragma unroll
                 for (int p = 0; p < KMAX; ++p)
                     v[p] = med3(v[p], p + 1 < KMAX ? v[p + 1] : INT_LOWEST, x);
-                // the nibbles of positions 0..m turn by one: the head's slot goes to m
-                const unsigned long long turning = ~0ull >> (60 - 4 * m);
-                ids[i] = (ids[i] & ~turning) | ((ids[i] & turning) >> 4) |
-                         ((unsigned long long)slot << (4 * m));
+                ids[i].turn(m, slot);  // the head's slot goes with x to position m
                 if (ins)
                     ski(i, slot) = (unsigned short)kj[i];
                 max_key[i] = ins ? __builtin_bit_cast(float, v[0]) : max_key[i];
@@ -880,7 +968,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
             asm volatile("" : "+v"(pq[i].b0), "+v"(pq[i].b1), "+v"(pq[i].b2), "+v"(pq[i].b3));
             asm volatile("" : "+v"(qlen[i]), "+v"(pending[i]), "+v"(max_key[i]), "+v"(max_idx[i]));
             if constexpr (SORTED)
-                asm volatile("" : "+v"(ids[i]));
+                ids[i].keep();
 #pragma unroll
             for (int s = 0; s < KMAX; ++s) {
                 asm volatile("" : "+v"(kd[i][s]));
@@ -1125,7 +1213,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
         if constexpr (SORTED) {
 #pragma unroll
             for (int p = 0; p < KMAX; ++p) {
-                const int slot = (int)((unsigned)(ids[i] >> (4 * p)) & 15u);
+                const int slot = (int)ids[i].at(p);
                 tbuf[lane * ROW + slot] = __builtin_bit_cast(float, kd[i][p]);
                 ibuf[lane * ROW + p] = (int)ski(i, p);
             }
@@ -2275,6 +2363,8 @@ inline bool knn_filter_pays(int64_t queries, int n2, int k)
 {
     if (k <= 4)
         return n2 >= 512 || (n2 >= 256 && queries >= 4096);
+    if (k > 16)  // 32 slots as a sorted list, key indices in LDS
+        return n2 >= 1024 && n2 <= 65536 && queries >= 32768;
     if (queries < 32768 && n2 > (k <= 8 ? 8192 : 32768))
         return false;
     return n2 >= (k <= 8 ? 512 : 1024) || (n2 >= 512 && queries >= 131072);
@@ -2285,7 +2375,7 @@ inline bool knn_filter_pays(int64_t queries, int n2, int k)
 inline bool knn_filter_takes(int64_t B, int n1, int n2, int k)
 {
     const int64_t bpb = ((int64_t)n1 + 511) / 512;
-    return k <= 16 && knn_filter_pays(B * n1, n2, k) && B * bpb <= TK_MAX_I32;
+    return k <= 32 && knn_filter_pays(B * n1, n2, k) && B * bpb <= TK_MAX_I32;
 }
 
 template <int KMAX, bool SOA, bool WEIGHTS>
@@ -2299,7 +2389,7 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
     const int64_t bpb = ((int64_t)n1 + 511) / 512;
     if (B * bpb > TK_MAX_I32 || !(whatever_the_size || knn_filter_takes(B, n1, n2, k)))
         return TK3D_ERR_UNSUPPORTED;
-    if constexpr (KMAX == 16) {
+    if constexpr (KMAX >= 16) {
         if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
             constexpr auto kernel =
                 knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512, true, !WEIGHTS>;
@@ -2311,7 +2401,10 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
                                distance, index, weight, eps, (int)bpb, n1, n2, k);
             return tk_launch_status();
         }
+        if constexpr (KMAX > 16)
+            return TK3D_ERR_UNSUPPORTED;  // 32 slots exist as a sorted list only
     }
+    if constexpr (KMAX <= 16)
     hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512>),
                        dim3((unsigned)(B * bpb)), dim3(512), 0, s, query, key, distance, index,
                        weight, eps, (int)bpb, n1, n2, k);
@@ -2353,13 +2446,16 @@ int knn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int64_t
         // fp32, k >= 5: slots in LDS as a tournament tree (k = 16 at B=32, 8192 x 2048:
         // 0.30 ms against 0.41 ms with the slots in registers). Small launches with k <= 8
         // are a little faster in registers.
-        if (k <= 16) {
+        if (k <= 32) {
             // pre-filtered sweep on the matrix cores, slots in registers: wherever it pays
             const int rc =
                 k <= 8 ? knn_filter_launch<8, false, false>(query, key, distance, index, nullptr,
                                                             0.0f, B, n1, n2, kk, s)
-                       : knn_filter_launch<16, false, false>(query, key, distance, index, nullptr,
-                                                             0.0f, B, n1, n2, kk, s);
+                : k <= 16
+                    ? knn_filter_launch<16, false, false>(query, key, distance, index, nullptr,
+                                                          0.0f, B, n1, n2, kk, s)
+                    : knn_filter_launch<32, false, false>(query, key, distance, index, nullptr,
+                                                          0.0f, B, n1, n2, kk, s);
             if (rc != TK3D_ERR_UNSUPPORTED)
                 return rc;
         }
@@ -2480,8 +2576,11 @@ int knn_bcn(const T *query, const T *key, int64_t B, int64_t N1, int64_t N2, int
         } else if (k <= 8) {
             rc = knn_filter_launch<8, true, false>(query, key, distance, index, nullptr, 0.0f, B,
                                                    n1, n2, kk, s);
-        } else {
+        } else if (k <= 16) {
             rc = knn_filter_launch<16, true, false>(query, key, distance, index, nullptr, 0.0f, B,
+                                                    n1, n2, kk, s);
+        } else {
+            rc = knn_filter_launch<32, true, false>(query, key, distance, index, nullptr, 0.0f, B,
                                                     n1, n2, kk, s);
         }
         return rc;
