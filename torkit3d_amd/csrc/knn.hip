@@ -2363,8 +2363,9 @@ inline bool knn_filter_pays(int64_t queries, int n2, int k)
 {
     if (k <= 4)
         return n2 >= 512 || (n2 >= 256 && queries >= 4096);
-    if (k > 16)  // 32 slots as a sorted list, key indices in LDS
-        return n2 >= 1024 && n2 <= 65536 && queries >= 32768;
+    if (k > 16)  // 32 slots as a sorted list, key indices in LDS; the tree kernel keeps
+                 // short clouds with many queries (B=24, 4096 x 700: 117 against 137 us)
+        return n2 <= 65536 && queries >= 4096 && (n2 >= 1024 || (n2 >= 512 && queries <= 32768));
     if (queries < 32768 && n2 > (k <= 8 ? 8192 : 32768))
         return false;
     return n2 >= (k <= 8 ? 512 : 1024) || (n2 >= 512 && queries >= 131072);
@@ -2378,6 +2379,33 @@ inline bool knn_filter_takes(int64_t B, int n1, int n2, int k)
     return k <= 32 && knn_filter_pays(B * n1, n2, k) && B * bpb <= TK_MAX_I32;
 }
 
+template <int KMAX, bool SOA, bool WEIGHTS, int LANES>
+int knn_filter_launch_as(const float *query, const float *key, float *distance, int64_t *index,
+                         float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
+{
+    const int64_t bpb = ((int64_t)n1 + LANES - 1) / LANES;
+    if constexpr (KMAX >= 16) {
+        if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
+            constexpr auto kernel =
+                knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, LANES, true, !WEIGHTS>;
+            constexpr int lds = KMAX * LANES * (int)sizeof(unsigned short);
+            const int allowed = tk_allow_dynamic_lds<kernel>(lds);
+            if (allowed != TK3D_OK)
+                return allowed;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(LANES), lds, s, query, key,
+                               distance, index, weight, eps, (int)bpb, n1, n2, k);
+            return tk_launch_status();
+        }
+        if constexpr (KMAX > 16)
+            return TK3D_ERR_UNSUPPORTED;  // 32 slots exist as a sorted list only
+    }
+    if constexpr (KMAX <= 16)
+        hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, LANES>),
+                           dim3((unsigned)(B * bpb)), dim3(LANES), 0, s, query, key, distance,
+                           index, weight, eps, (int)bpb, n1, n2, k);
+    return tk_launch_status();
+}
+
 template <int KMAX, bool SOA, bool WEIGHTS>
 int knn_filter_launch(const float *query, const float *key, float *distance, int64_t *index,
                       float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s,
@@ -2386,29 +2414,18 @@ int knn_filter_launch(const float *query, const float *key, float *distance, int
     // One query per lane, 512 lanes: two workgroups (16 waves) per CU. Two queries per lane
     // in 256 lanes need twice the registers, which leaves two waves per SIMD, and were 1.1
     // to 1.4 times slower on every shape (k = 16 at B=32, 8192 x 2048: 222 -> 191 us).
+    // A launch of few such workgroups leaves CUs without one: 256 lanes then (128 workgroups,
+    // B=8, 8192 x 2048: k = 3 52 -> 48 us, k = 16 96 -> 85 us, k = 32 189 -> 142 us; at 160
+    // workgroups with up to 8 slots, at 192 with more, the larger workgroup wins: its staged
+    // keys serve more queries).
     const int64_t bpb = ((int64_t)n1 + 511) / 512;
     if (B * bpb > TK_MAX_I32 || !(whatever_the_size || knn_filter_takes(B, n1, n2, k)))
         return TK3D_ERR_UNSUPPORTED;
-    if constexpr (KMAX >= 16) {
-        if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
-            constexpr auto kernel =
-                knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512, true, !WEIGHTS>;
-            constexpr int lds = KMAX * 512 * (int)sizeof(unsigned short);
-            const int allowed = tk_allow_dynamic_lds<kernel>(lds);
-            if (allowed != TK3D_OK)
-                return allowed;
-            hipLaunchKernelGGL(kernel, dim3((unsigned)(B * bpb)), dim3(512), lds, s, query, key,
-                               distance, index, weight, eps, (int)bpb, n1, n2, k);
-            return tk_launch_status();
-        }
-        if constexpr (KMAX > 16)
-            return TK3D_ERR_UNSUPPORTED;  // 32 slots exist as a sorted list only
-    }
-    if constexpr (KMAX <= 16)
-    hipLaunchKernelGGL((knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, 512>),
-                       dim3((unsigned)(B * bpb)), dim3(512), 0, s, query, key, distance, index,
-                       weight, eps, (int)bpb, n1, n2, k);
-    return tk_launch_status();
+    if (B * bpb <= (KMAX <= 8 ? 128 : 160))
+        return knn_filter_launch_as<KMAX, SOA, WEIGHTS, 256>(query, key, distance, index, weight,
+                                                             eps, B, n1, n2, k, s);
+    return knn_filter_launch_as<KMAX, SOA, WEIGHTS, 512>(query, key, distance, index, weight, eps,
+                                                         B, n1, n2, k, s);
 }
 
 template <typename T>
