@@ -332,7 +332,7 @@ def _filter_case(kind, g, k, b=8, n1=8192 + 5, n2=2048 + 37):  # ragged: partial
     return q.contiguous(), key.contiguous()
 
 
-@pytest.mark.parametrize("k", [1, 3, 4, 7, 9, 13, 16])
+@pytest.mark.parametrize("k", [1, 3, 4, 7, 9, 13, 16, 17, 25, 32])
 @pytest.mark.parametrize("kind", ["uniform", "lattice", "far_to_near", "near_to_far",
                                   "far_from_origin", "separated", "tiny", "huge", "huge_queries",
                                   "scaled_small", "scaled_large", "far_queries",
@@ -342,10 +342,10 @@ def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
     check_raw(q, key, k, cuda)
 
 
-@pytest.mark.parametrize("k", [9, 12, 16])
+@pytest.mark.parametrize("k", [9, 12, 16, 17, 24, 32])
 @pytest.mark.parametrize("steps", [1, 2, 16])
 def test_prefiltered_kernel_with_sorted_slots_on_equal_distances(cuda, steps, k):
-    # For 9 to 16 neighbours the kernel keeps a query's distances in descending order and the
+    # For 9 to 32 neighbours the kernel keeps a query's distances in descending order and the
     # slot numbers beside them; among equal distances MinK's rescan (mink.cuh:74-87) decides
     # which slot is overwritten next: the slot just written if nothing is strictly above it,
     # else the lowest slot holding the largest distance. Lattices of 3, 5 and 33 positions
@@ -407,7 +407,7 @@ def test_prefiltered_three_nn_on_both_layouts(cuda):
         np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=3e-7, atol=0)
 
 
-@pytest.mark.parametrize("k", [3, 4, 5, 8, 16])
+@pytest.mark.parametrize("k", [3, 4, 5, 8, 16, 20, 32])
 def test_prefiltered_kernel_on_the_hand_worked_mink_run(cuda, k):
     # the literal rows of tests/util.py again, now with enough queries (140000 copies) and
     # keys (5000 far ones behind the run) for the dispatcher to take the pre-filtered kernel
