@@ -561,8 +561,8 @@ __device__ __forceinline__ int knn_sorted_position(const int (&v)[KMAX], Above a
 // one column per lane: they are only written during the sweep, and a write into a column of
 // one's own is one instruction where the slot in registers takes a select per slot.
 //
-// SORTED (16 slots, key indices in LDS): the registers hold the distances in descending
-// order instead of slot order, and a 64-bit word holds the slot number of every position,
+// SORTED (8 to 32 slots, key indices in LDS; described for 16): the registers hold the
+// distances in descending order instead of slot order, and a 64-bit word holds the slot number of every position,
 // a nibble each. MinK's maximum is then position 0, and an insertion is one v_med3_i32 per
 // position (remove the head, let the new key x sink to its place: position p becomes the
 // median of its old value, its lower neighbour's and x) plus a rotation of the nibbles of
@@ -594,8 +594,8 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     constexpr int T = 6;
     constexpr int PER = STAGE / BLOCK;
     static_assert(STAGE % BLOCK == 0 && STAGE % CHUNK == 0, "stage shape");
-    static_assert(!SORTED || (KI_LDS && QPL == 1 && (KMAX == 16 || KMAX == 32) && !WEIGHTS),
-                  "the sorted list is for one query of 16 or 32 slots per lane");
+    static_assert(!SORTED || (KI_LDS && QPL == 1 && KMAX >= 4 && KMAX <= 32 && !WEIGHTS),
+                  "the sorted list is for one query of 4 to 32 slots per lane, no weights");
     static_assert(2 * STAGE * 4 * (int)sizeof(float) >= KNN_STAGE * 4 * (int)sizeof(float),
                   "the staging buffers double as the exact sweep's stage");
     // Two stage buffers of centred keys (x', y', z', |k'|^2) (+ 8 keys the read-ahead of
@@ -715,7 +715,7 @@ __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
     float max_key[QPL];
     int max_idx[QPL];
     unsigned nan_slots[QPL];
-    KnnSlotNumbers<(SORTED ? KMAX : 16)> ids[QPL];  // SORTED: the slot of every position of kd
+    KnnSlotNumbers<(KMAX > 16 ? 32 : 16)> ids[QPL];  // SORTED: the slot of every position of kd
     constexpr int NEG_INF_BITS = (int)0xff800000u;
     constexpr int INT_LOWEST = (int)0x80000000u, INT_HIGHEST = 0x7fffffff;
     // the median of three (v_med3_i32)
@@ -2384,7 +2384,7 @@ int knn_filter_launch_as(const float *query, const float *key, float *distance, 
                          float *weight, float eps, int64_t B, int n1, int n2, int k, hipStream_t s)
 {
     const int64_t bpb = ((int64_t)n1 + LANES - 1) / LANES;
-    if constexpr (KMAX >= 16) {
+    if constexpr (KMAX >= 8) {  // (4 slots: the slot-ordered registers are 2-7 % faster)
         if (n2 <= 65536) {  // the slots' key indices in LDS, 16 bits each
             constexpr auto kernel =
                 knn_filter_kernel_f32<KMAX, 1, SOA, WEIGHTS, true, LANES, true, !WEIGHTS>;
