@@ -268,13 +268,19 @@ def test_region_kernel_on_adversarial_clouds(cuda, kind):
     pts = _region_cloud(kind, g, 2, 6000 if kind in ("uniform", "lattice") else 8192)
     k = 700
     np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
+    # and with 4 (2049 to 4096 points)
+    pts = _region_cloud(kind, g, 2, 2700 if kind in ("uniform", "lattice") else 4096)
+    k = 600
+    np.testing.assert_array_equal(run(pts, k, cuda), oracle.sample_farthest_points(pts.numpy(), k))
 
 
 @pytest.mark.parametrize("n,k,transpose", [(8193, 2048, False), (16384, 16384, False),
                                            (10000, 2049, True), (16383, 4096, True),
                                            (4097, 256, False), (8192, 8192, False),
                                            (5000, 300, True), (16384, 256, True),
-                                           (8193, 257, False)])
+                                           (8193, 257, False), (2049, 256, False),
+                                           (4096, 4096, False), (3072, 256, True),
+                                           (3073, 512, True), (2500, 2500, False)])
 def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
     pts = torch.rand(2, n, 3, generator=gen(n + k))
     want = oracle.sample_farthest_points(pts.numpy(), k)
@@ -282,11 +288,11 @@ def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
     np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
 
 
-@pytest.mark.parametrize("n", [9000, 5000])
+@pytest.mark.parametrize("n", [9000, 5000, 3000])
 def test_region_kernel_with_non_finite_points(cuda, n):
     pts = torch.rand(3, n, 3, generator=gen(71))
     pts[0, 7, 1] = float("nan")
-    pts[0, 4500] = float("nan")
+    pts[0, n // 2] = float("nan")
     pts[1, 100, 0] = float("inf")
     pts[2, 0, 2] = float("nan")        # point 0 itself: every distance is NaN
     k = 2048 if n == 9000 else 400

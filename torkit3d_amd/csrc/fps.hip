@@ -1240,6 +1240,11 @@ int fps_dispatch_f32(const float *points, bool soa, int64_t B, int64_t *index,
         fps_launch_f32<2, 512>(points, soa, B, index, L, s);
     else if (npos <= 512 * 4)
         fps_launch_f32<4, 512>(points, soa, B, index, L, s);
+    // From 2049 points on the region kernel with 4 points per lane, once its prologue is paid
+    // for: B=16, 4096 -> 1024 0.44 -> 0.40 ms, 3000 -> 1024 0.47 -> 0.39 ms, 2100 -> 512
+    // 0.26 -> 0.21 ms, 4096 -> 4096 1.65 -> 1.38 ms; 4096 -> 384 is level, -> 256 10 % behind.
+    else if (npos > 512 * 4 && npos <= 512 * 8 && L.k >= (npos <= 512 * 6 ? 256 : 512))
+        return fps_region_launch_f32<4>(points, soa, B, index, L, s);
     else if (npos <= 512 * 8)
         fps_launch_f32<8, 512>(points, soa, B, index, L, s);
     // Beyond 4096 points the region kernel (sixteen waves; its prologue costs about 30 us) wins
