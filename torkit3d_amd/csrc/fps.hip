@@ -518,7 +518,7 @@ __device__ __forceinline__ int fps_position_of_point(int j, const FpsLayout &L)
     return r * L.c + (j >> L.log2_bs);
 }
 
-// fp32 kernel for clouds of 4097 to 16384 points: the multi-step kernel above with the
+// fp32 kernel for clouds of 2049 to 16384 points: the multi-step kernel above with the
 // points laid out by region, so that an update only visits the points a new centre can
 // reach, and with sixteen waves, so that an exchange has sixteen candidates to accept from.
 //
@@ -1197,7 +1197,7 @@ void fps_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
     }
 }
 
-// Clouds of 4097 to 16384 points: the region kernel, then the same check for non-finite
+// Clouds of 2049 to 16384 points: the region kernel, then the same check for non-finite
 // coordinates as above.
 template <int P>
 int fps_region_launch_f32(const float *points, bool soa, int64_t B, int64_t *index,
