@@ -342,10 +342,10 @@ def test_prefiltered_kernel_is_exact_on_hard_inputs(cuda, kind, k):
     check_raw(q, key, k, cuda)
 
 
-@pytest.mark.parametrize("k", [9, 12, 16, 17, 24, 32])
+@pytest.mark.parametrize("k", [5, 8, 9, 12, 16, 17, 24, 32])
 @pytest.mark.parametrize("steps", [1, 2, 16])
 def test_prefiltered_kernel_with_sorted_slots_on_equal_distances(cuda, steps, k):
-    # For 9 to 32 neighbours the kernel keeps a query's distances in descending order and the
+    # For 5 to 32 neighbours the kernel keeps a query's distances in descending order and the
     # slot numbers beside them; among equal distances MinK's rescan (mink.cuh:74-87) decides
     # which slot is overwritten next: the slot just written if nothing is strictly above it,
     # else the lowest slot holding the largest distance. Lattices of 3, 5 and 33 positions
