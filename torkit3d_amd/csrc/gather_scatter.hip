@@ -144,15 +144,35 @@ __global__ __launch_bounds__(NT) void gather_lds_kernel(
     auto fetch = [&](int64_t p0) {
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-#pragma unroll
-            for (int i = 0; i < KK; ++i) {
-                const int64_t p = p0 + v * 64;
-                jn[v][i] = -1;
-                wn[v][i] = (T)0;
+            const int64_t p = p0 + v * 64;
+            if constexpr (KK == 3) {
+                // a point's three indices and three weights as one run each: element by
+                // element a wave's request touches every cache line of the run three times
+                struct __attribute__((aligned(8))) Idx3 { int64_t a, b, c; };
+                struct __attribute__((aligned(sizeof(T)))) W3 { T a, b, c; };
+                Idx3 ji = {-1, -1, -1};
+                W3 wi = {(T)0, (T)0, (T)0};
                 if (p < pe) {
-                    jn[v][i] = idx[((int64_t)b * np + p) * KK + i];
+                    ji = *reinterpret_cast<const Idx3 *>(idx + ((int64_t)b * np + p) * 3);
                     if (HAS_W)
-                        wn[v][i] = w[((int64_t)b * np + p) * KK + i];
+                        wi = *reinterpret_cast<const W3 *>(w + ((int64_t)b * np + p) * 3);
+                }
+                jn[v][0] = ji.a;
+                jn[v][1] = ji.b;
+                jn[v][2] = ji.c;
+                wn[v][0] = wi.a;
+                wn[v][1] = wi.b;
+                wn[v][2] = wi.c;
+            } else {
+#pragma unroll
+                for (int i = 0; i < KK; ++i) {
+                    jn[v][i] = -1;
+                    wn[v][i] = (T)0;
+                    if (p < pe) {
+                        jn[v][i] = idx[((int64_t)b * np + p) * KK + i];
+                        if (HAS_W)
+                            wn[v][i] = w[((int64_t)b * np + p) * KK + i];
+                    }
                 }
             }
         }
@@ -777,10 +797,30 @@ scatter_fixed_rows_kernel(const float *__restrict__ gout, const int64_t *__restr
         for (int v = 0; v < V; ++v) {
             unsigned po = chunk * (64 * V) + v * 64 + lane;
             po = po < jb.len ? po : jb.len - 1;
+            if constexpr (KK == 3) {
+                // a point's three indices and three weights as one run each (a 16-byte and an
+                // 8-byte load, a 12-byte load): loaded one element at a time, a wave's
+                // request touches every cache line of the run three times
+                struct __attribute__((aligned(8))) Idx3 { int64_t a, b, c; };
+                struct __attribute__((aligned(4))) W3 { float a, b, c; };
+                const Idx3 ji = *reinterpret_cast<const Idx3 *>(jb.ibase + (int64_t)po * 3);
+                st.j[v][0] = ji.a;
+                st.j[v][1] = ji.b;
+                st.j[v][2] = ji.c;
+                if constexpr (HAS_W) {
+                    const W3 wi = *reinterpret_cast<const W3 *>(jb.wbase + (int64_t)po * 3);
+                    st.w[v][0] = wi.a;
+                    st.w[v][1] = wi.b;
+                    st.w[v][2] = wi.c;
+                } else {
+                    st.w[v][0] = st.w[v][1] = st.w[v][2] = 1.0f;
+                }
+            } else {
 #pragma unroll
-            for (int i = 0; i < KK; ++i) {
-                st.j[v][i] = jb.ibase[po * KK + i];
-                st.w[v][i] = HAS_W ? jb.wbase[po * KK + i] : 1.0f;
+                for (int i = 0; i < KK; ++i) {
+                    st.j[v][i] = jb.ibase[po * KK + i];
+                    st.w[v][i] = HAS_W ? jb.wbase[po * KK + i] : 1.0f;
+                }
             }
 #pragma unroll
             for (int c = 0; c < CG; ++c)
