@@ -288,6 +288,33 @@ def test_region_kernel_shapes_and_layouts(cuda, n, k, transpose):
     np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
 
 
+@pytest.mark.parametrize("n,k,transpose", [(4096, 1024, False), (3000, 512, True), (2049, 2049, False)])
+def test_clouds_in_sampling_order_between_2049_and_4096_points(cuda, n, k, transpose):
+    # A cloud that is itself a farthest point sample in sampling order (the next level of a
+    # PointNet++ encoder): its point 1 is the point farthest from point 0, by which the region
+    # kernel recognises it and leaves it to the multi-step kernel launched behind it. The
+    # answer is the first k indices in order. Then a cloud in random order whose point 1
+    # happens to be the farthest from point 0: it takes the same route and must come out right
+    # as well, and one with a NaN in that place.
+    big = torch.rand(2, 3 * n, 3, generator=gen(n + k))
+    first = oracle.sample_farthest_points(big.numpy(), n)
+    pts = torch.gather(big, 1, torch.from_numpy(first)[:, :, None].expand(-1, -1, 3)).contiguous()
+    want = oracle.sample_farthest_points(pts.numpy(), k)
+    np.testing.assert_array_equal(want, np.tile(np.arange(k), (2, 1)))
+    dev = pts.transpose(1, 2).contiguous() if transpose else pts
+    np.testing.assert_array_equal(run(dev, k, cuda, transpose), want)
+    rnd = torch.rand(2, n, 3, generator=gen(n))
+    rnd[:, 0] = 0.0
+    rnd[:, 1] = 5.0                      # farther from point 0 than anything in the unit cube
+    dev = rnd.transpose(1, 2).contiguous() if transpose else rnd
+    np.testing.assert_array_equal(run(dev, k, cuda, transpose),
+                                  oracle.sample_farthest_points(rnd.numpy(), k))
+    rnd[0, 1, 2] = float("nan")
+    dev = rnd.transpose(1, 2).contiguous() if transpose else rnd
+    np.testing.assert_array_equal(run(dev, k, cuda, transpose),
+                                  oracle.sample_farthest_points(rnd.numpy(), k))
+
+
 @pytest.mark.parametrize("n", [9000, 5000, 3000])
 def test_region_kernel_with_non_finite_points(cuda, n):
     pts = torch.rand(3, n, 3, generator=gen(71))

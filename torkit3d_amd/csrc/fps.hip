@@ -361,12 +361,16 @@ template <int P, int NODE> struct FpsWalk3 {
 // instructions is its cost: conditions are single compares whose lane masks are combined
 // in scalar registers, and the accepted candidates never go back to LDS - the coming
 // update reads their coordinates with v_readlane from the lanes that already hold them.
-template <int P, int NT, bool SOA, int MAXM>
+template <int P, int NT, bool SOA, int MAXM, bool GATED = false>
 __global__ __launch_bounds__(NT) void fps_multistep_kernel_f32(const float *__restrict__ points,
                                                                int64_t *__restrict__ index,
                                                                FpsLayout L)
 {
     static_assert((P & (P - 1)) == 0, "P must be a power of two");
+    if constexpr (GATED) {  // only the clouds the region kernel left (see its ORDER_PROBE)
+        if (index[(int64_t)blockIdx.x * L.k + L.k - 1] != -1)  // uniform over the workgroup
+            return;
+    }
     constexpr int NW = NT / TK_WAVE;
     static_assert(NW <= 8, "the cross-wave step relates 8 x 8 candidates");
     constexpr int F32_INF = 0x7f800000;
@@ -585,13 +589,28 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
     const float INF = __builtin_huge_valf();
 
     // ---- bounding box of the cloud ----
+    // (4 points per lane: also the point farthest from point 0, lowest index first - see
+    // ORDER_PROBE below)
+    constexpr bool ORDER_PROBE = P == 4;
     float lo[3] = {INF, INF, INF}, hi[3] = {-INF, -INF, -INF};
+    float far_d = -1.0f;
+    int far_j = 0;
+    const float p0x = fps_coord<SOA>(pts, L.n, 0, 0), p0y = fps_coord<SOA>(pts, L.n, 0, 1),
+                p0z = fps_coord<SOA>(pts, L.n, 0, 2);
     for (int j = tid; j < L.n; j += NT) {
+        float v[3];
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-            const float v = fps_coord<SOA>(pts, L.n, j, a);
-            lo[a] = __builtin_fminf(lo[a], v);
-            hi[a] = __builtin_fmaxf(hi[a], v);
+            v[a] = fps_coord<SOA>(pts, L.n, j, a);
+            lo[a] = __builtin_fminf(lo[a], v[a]);
+            hi[a] = __builtin_fmaxf(hi[a], v[a]);
+        }
+        if constexpr (ORDER_PROBE) {
+            const float d = tk_dist2<float>(v[0], v[1], v[2], p0x, p0y, p0z);
+            if (d > far_d) {  // (j ascends within a lane)
+                far_d = d;
+                far_j = j;
+            }
         }
     }
 #pragma unroll
@@ -602,14 +621,52 @@ __global__ __launch_bounds__(1024) void fps_region_kernel_f32(const float *__res
             hi[a] = __builtin_fmaxf(hi[a], __shfl_xor(hi[a], o));
         }
     }
+    if constexpr (ORDER_PROBE) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float od = __shfl_xor(far_d, o);
+            const int oj = __shfl_xor(far_j, o);
+            const bool take = od > far_d || (od == far_d && oj < far_j);
+            far_d = take ? od : far_d;
+            far_j = take ? oj : far_j;
+        }
+    }
     if (lane == 0) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
             s_red[wave][a] = lo[a];
             s_red[wave][3 + a] = hi[a];
         }
+        s_red[wave][6] = far_d;
+        s_red[wave][7] = __builtin_bit_cast(float, far_j);
     }
     __syncthreads();
+    if constexpr (ORDER_PROBE) {
+        // ORDER_PROBE. A cloud whose point 1 is the point farthest from point 0 is, in
+        // practice, itself the output of a farthest point sampling, in sampling order (the
+        // next level of a PointNet++ encoder): every stretch of such a cloud is spread over
+        // all of it, which is what the multi-step kernel's waves want (their candidates get
+        // in each other's way less: B=16, 4096 -> 1024 0.33 ms there against 0.44 on points
+        // in random order) and this kernel, which sorts the points by cell anyway, cannot
+        // use (0.39 either way). Such a cloud is left to the multi-step kernel, which is
+        // launched behind this one and runs only where it finds the mark: -1 as the last
+        // index. (A cloud in random order passes this test once in n.)
+        float d = s_red[0][6];
+        int j = __builtin_bit_cast(int, s_red[0][7]);
+#pragma unroll
+        for (int w = 1; w < NW; ++w) {
+            const float od = s_red[w][6];
+            const int oj = __builtin_bit_cast(int, s_red[w][7]);
+            const bool take = od > d || (od == d && oj < j);
+            d = take ? od : d;
+            j = take ? oj : j;
+        }
+        if (j == 1) {  // uniform over the workgroup
+            if (tid == 0)
+                out[L.k - 1] = -1;
+            return;
+        }
+    }
     float origin[3], scale[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -1212,6 +1269,9 @@ int fps_region_launch_f32(const float *points, bool soa, int64_t B, int64_t *ind
         if (allowed != TK3D_OK)
             return allowed;
         hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(NT), LDS, s, points, index, L);
+        if constexpr (P == 4)  // clouds in sampling order, which the kernel above leaves
+            hipLaunchKernelGGL((fps_multistep_kernel_f32<8, 512, true, 6, true>),
+                               dim3((unsigned)B), dim3(512), 0, s, points, index, L);
         hipLaunchKernelGGL((fps_register_kernel<float, P, NT, true>), dim3((unsigned)B),
                            dim3(NT), 0, s, points, index, L, 1);
     } else {
@@ -1220,6 +1280,9 @@ int fps_region_launch_f32(const float *points, bool soa, int64_t B, int64_t *ind
         if (allowed != TK3D_OK)
             return allowed;
         hipLaunchKernelGGL(kernel, dim3((unsigned)B), dim3(NT), LDS, s, points, index, L);
+        if constexpr (P == 4)
+            hipLaunchKernelGGL((fps_multistep_kernel_f32<8, 512, false, 6, true>),
+                               dim3((unsigned)B), dim3(512), 0, s, points, index, L);
         hipLaunchKernelGGL((fps_register_kernel<float, P, NT, false>), dim3((unsigned)B),
                            dim3(NT), 0, s, points, index, L, 1);
     }
