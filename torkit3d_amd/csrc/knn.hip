@@ -382,7 +382,10 @@ template <> struct KnnSlotNumbers<16> {
     unsigned long long w;
     __device__ __forceinline__ void identity() { w = 0xfedcba9876543210ull; }
     __device__ __forceinline__ unsigned head() const { return (unsigned)w & 15u; }
-    __device__ __forceinline__ unsigned at(int p) const { return (unsigned)(w >> ((4 * p) & 63)) & 15u; }
+    __device__ __forceinline__ unsigned at(int p) const
+    {
+        return (unsigned)(w >> ((4 * p) & 63)) & 15u;
+    }
     // positions 0..m turn by one towards the head; `slot` (the old head's) goes to position m
     __device__ __forceinline__ void turn(int m, unsigned slot)
     {
@@ -452,7 +455,10 @@ template <> struct KnnSlotNumbers<32> {
             w0 = (w0 & ~f0) | ((w0 & f0) << 4) | (far ? 0ull : low << (4 * m));
         }
     }
-    __device__ __forceinline__ void keep() { asm volatile("" : "+v"(w0), "+v"(w1), "+v"(fifth)); }
+    __device__ __forceinline__ void keep()
+    {
+        asm volatile("" : "+v"(w0), "+v"(w1), "+v"(fifth));
+    }
 };
 
 // How many of positions 1..KMAX-1 of a descending list satisfy `above` (true for a prefix of
@@ -562,9 +568,9 @@ __device__ __forceinline__ int knn_sorted_position(const int (&v)[KMAX], Above a
 // one's own is one instruction where the slot in registers takes a select per slot.
 //
 // SORTED (8 to 32 slots, key indices in LDS; described for 16): the registers hold the
-// distances in descending order instead of slot order, and a 64-bit word holds the slot number of every position,
-// a nibble each. MinK's maximum is then position 0, and an insertion is one v_med3_i32 per
-// position (remove the head, let the new key x sink to its place: position p becomes the
+// distances in descending order instead of slot order, and a 64-bit word holds the slot
+// number of every position, a nibble each. MinK's maximum is then position 0, and an
+// insertion is one v_med3_i32 per position (remove the head, let the new key x sink to its place: position p becomes the
 // median of its old value, its lower neighbour's and x) plus a rotation of the nibbles of
 // positions 0..m, m being x's new position, found by a binary search through the registers
 // (4 compares, 11 selects): 86 instructions per step where the slot-ordered registers take
@@ -577,8 +583,9 @@ __device__ __forceinline__ int knn_sorted_position(const int (&v)[KMAX], Above a
 // head, x goes to position 0 if no element of R is above it, else behind the elements of R
 // that are above it or equal to it with a lower slot number. Equal distances are rare
 // outside quantised clouds: the binary search counts the elements >= x and hands back the
-// last of them; only when that equals x in some lane does the wave count both kinds
-// position by position.
+// last of them; only when that equals x in some lane does the wave search again, for the
+// elements strictly above x, and walk the run of equals between the two results comparing
+// slot numbers.
 template <int KMAX, int QPL, bool SOA, bool WEIGHTS, bool MATRIX, int LANES = KNN_BLOCK,
           bool KI_LDS = false, bool SORTED = false>
 __global__ __launch_bounds__(LANES) void knn_filter_kernel_f32(
